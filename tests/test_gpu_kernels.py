@@ -1,0 +1,408 @@
+"""Each HIP kernel alone against a plain float64 reference, at sizes the engine's models do
+not use (odd widths, head sizes from 16 to 256, several page sizes)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from plain import lfm2_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+
+def _r(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+# ------------------------------------------------------------------------------- GEMM
+@pytest.mark.parametrize("M,N,K", [(1, 7, 5), (3, 100, 33), (65, 130, 17), (130, 65, 250), (64, 64, 64)])
+def test_gemm_f32(gpu, M, N, K):
+    from tuff_amd.csrc import ops
+    x, w = _r(M, K, seed=1), _r(N, K, seed=2)
+    y0 = _r(M, N, seed=3)
+    want = x.double() @ w.double().T
+    out = torch.empty(M, N, device=gpu)
+    ops.gemm(x.to(gpu), w.to(gpu), out)
+    bound = 4e-7 * K * x.abs().max() * w.abs().max()
+    assert (out.cpu().double() - want).abs().max() <= bound
+    acc = y0.to(gpu)
+    ops.gemm(x.to(gpu), w.to(gpu), acc, accumulate=True)
+    assert (acc.cpu().double() - (want + y0.double())).abs().max() <= bound + 1e-6
+    # a row does not depend on the other rows of the call
+    if M > 1:
+        one = torch.empty(1, N, device=gpu)
+        ops.gemm(x[M - 1:].to(gpu), w.to(gpu), one)
+        assert torch.equal(one[0], out[M - 1])
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 16, 8), (5, 1000, 96), (17, 33, 40), (64, 777, 240), (65, 130, 136),
+                                   (200, 300, 328), (300, 64, 2048), (128, 128, 64), (2, 2048, 8192)])
+def test_gemm_bf16(gpu, M, N, K):
+    from tuff_amd.csrc import ops
+    x, w = _r(M, K, seed=4, dtype=torch.bfloat16), _r(N, K, seed=5, dtype=torch.bfloat16)
+    want = x.double() @ w.double().T
+    scale = float(want.abs().max())
+    f32 = torch.empty(M, N, device=gpu)
+    ops.gemm(x.to(gpu), w.to(gpu), f32)
+    assert (f32.cpu().double() - want).abs().max() <= 1e-5 * scale + 1e-6 * K
+    b16 = torch.empty(M, N, device=gpu, dtype=torch.bfloat16)
+    ops.gemm(x.to(gpu), w.to(gpu), b16)
+    assert (b16.cpu().double() - want).abs().max() <= 2 ** -8 * scale
+    y0 = _r(M, N, seed=6)
+    acc = y0.to(gpu)
+    ops.gemm(x.to(gpu), w.to(gpu), acc, accumulate=True)
+    assert (acc.cpu().double() - (want + y0.double())).abs().max() <= 1e-5 * scale + 1e-6 * K
+
+
+def test_gemm_refuses_what_it_cannot_do(gpu):
+    from tuff_amd.csrc import ops
+    x = torch.zeros(2, 12, dtype=torch.bfloat16, device=gpu)
+    w = torch.zeros(4, 12, dtype=torch.bfloat16, device=gpu)
+    with pytest.raises(ops.KernelError, match="multiple of 8"):
+        ops.gemm(x, w, torch.empty(2, 4, device=gpu))
+    with pytest.raises(ops.KernelError, match="no CPU fallback"):
+        ops.gemm(torch.zeros(2, 8), torch.zeros(4, 8), torch.zeros(2, 4))
+    with pytest.raises(ops.KernelError, match="expected shape"):
+        ops.gemm(x, w, torch.empty(3, 4, device=gpu))
+
+
+# ------------------------------------------------------------------------- row kernels
+@pytest.mark.parametrize("n,d", [(5, 64), (3, 777), (1, 2048), (9, 240)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm(gpu, n, d, out_dtype):
+    from tuff_amd.csrc import ops
+    x, w = _r(n, d, seed=7, scale=3.0), 1 + _r(d, seed=8, scale=0.1)
+    for eps in (1e-5, 0.5):
+        want = plain.rms_norm(x.double(), w.double(), eps)
+        out = torch.empty(n, d, device=gpu, dtype=out_dtype)
+        ops.rmsnorm(x.to(gpu), w.to(gpu), out, eps)
+        tol = 1e-5 if out_dtype == torch.float32 else 2 ** -8 * float(want.abs().max())
+        assert (out.cpu().double() - want).abs().max() <= tol
+    rows = torch.tensor([n - 1, 0], dtype=torch.int32)
+    out = torch.empty(2, d, device=gpu, dtype=out_dtype)
+    ops.rmsnorm(x.to(gpu), w.to(torch.bfloat16).to(gpu), out, 1e-5, rows.to(gpu))
+    want = plain.rms_norm(x.double(), w.to(torch.bfloat16).double(), 1e-5)[rows.long()]
+    assert (out.cpu().double() - want).abs().max() <= (1e-5 if out_dtype == torch.float32 else 2 ** -8 * float(want.abs().max()))
+
+
+def test_embed_and_swiglu(gpu):
+    from tuff_amd.csrc import ops
+    table = _r(50, 24, seed=9, dtype=torch.bfloat16)
+    toks = torch.tensor([3, 49, 0, 3], dtype=torch.int32)
+    out = torch.empty(4, 24, device=gpu)
+    ops.embed_rows(table.to(gpu), toks.to(gpu), out)
+    assert torch.equal(out.cpu(), table[toks.long()].float())
+    for dt in (torch.float32, torch.bfloat16):
+        gu = _r(7, 2 * 13, seed=10, scale=2.0, dtype=dt)
+        act = torch.empty(7, 13, device=gpu, dtype=dt)
+        ops.swiglu(gu.to(gpu), act)
+        g, u = gu[:, :13].double(), gu[:, 13:].double()
+        want = g / (1 + torch.exp(-g)) * u
+        assert (act.cpu().double() - want).abs().max() <= (1e-6 if dt == torch.float32 else 2 ** -8 * float(want.abs().max()))
+    z = torch.zeros(2, 8, device=gpu)
+    ops.swiglu(torch.zeros(2, 16, device=gpu), z)
+    assert (z == 0).all()                                # g = 0 gives 0
+
+
+# --------------------------------------------------------------- q/k/v post-processing
+def _interleaved_rope(x, pos, base):
+    hd = x.shape[-1]
+    j = torch.arange(hd // 2, dtype=torch.float64)
+    a = pos.double()[:, None] * base ** (-2 * j / hd)
+    c, s = torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
+    x0, x1 = x[..., 0::2], x[..., 1::2]
+    out = torch.empty_like(x)
+    out[..., 0::2] = x0 * c - x1 * s
+    out[..., 1::2] = x0 * s + x1 * c
+    return out
+
+
+@pytest.mark.parametrize("H,Hkv,hd,ps", [(4, 2, 16, 16), (4, 1, 24, 8), (3, 3, 80, 16), (2, 1, 256, 4), (5, 5, 128, 64)])
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_qkv_post(gpu, H, Hkv, hd, ps, dt):
+    from tuff_amd.csrc import ops
+    T, eps, base = 11, 1e-5, 10000.0
+    qkv = _r(T, (H + 2 * Hkv) * hd, seed=11, dtype=dt)
+    qw, kw = 1 + _r(hd, seed=12, scale=0.1), 1 + _r(hd, seed=13, scale=0.1)
+    pos = torch.tensor([0, 1, 2, 3, 100, 101, 7, 8, 9, 1000, 31], dtype=torch.int32)
+    n_pages = 8
+    slots = torch.randperm(n_pages * ps, generator=torch.Generator().manual_seed(1))[:T].to(torch.int32)
+    j = torch.arange(hd // 2, dtype=torch.float64)
+    inv_freq = (base ** (-2 * j / hd)).float()
+    kc = torch.zeros(n_pages, Hkv, ps, hd, dtype=dt, device=gpu)
+    vc = torch.zeros_like(kc)
+    q = torch.empty(T, H * hd, dtype=dt, device=gpu)
+    ops.qkv_post(qkv.to(gpu), q, H=H, Hkv=Hkv, hd=hd, positions=pos.to(gpu), eps=eps, q_norm_w=qw.to(gpu),
+                 k_norm_w=kw.to(gpu), inv_freq=inv_freq.to(gpu), rotary_dim=hd, k_cache=kc, v_cache=vc,
+                 slot_mapping=slots.to(gpu), page_size=ps)
+    x = qkv.double()
+    qs, ks, vs = x[:, :H * hd].reshape(T, H, hd), x[:, H * hd:(H + Hkv) * hd].reshape(T, Hkv, hd), x[:, (H + Hkv) * hd:].reshape(T, Hkv, hd)
+    want_q = plain.rope_neox(plain.rms_norm(qs, qw.double(), eps), pos, base)
+    want_k = plain.rope_neox(plain.rms_norm(ks, kw.double(), eps), pos, base)
+    # float32 angles: pos * theta carries a relative error of 2^-24, so 1000 rad is known to 6e-5
+    tol = 2e-4 if dt == torch.float32 else 2 ** -7
+    assert (q.cpu().double().reshape(T, H, hd) - want_q).abs().max() <= tol * float(want_q.abs().max())
+    got_k = kc.cpu().double().permute(0, 2, 1, 3).reshape(n_pages * ps, Hkv, hd)[slots.long()]
+    got_v = vc.cpu().double().permute(0, 2, 1, 3).reshape(n_pages * ps, Hkv, hd)[slots.long()]
+    assert (got_k - want_k).abs().max() <= tol * float(want_k.abs().max())
+    assert torch.equal(got_v, vs)
+    # nothing else in the cache was touched
+    untouched = torch.ones(n_pages * ps, dtype=torch.bool)
+    untouched[slots.long()] = False
+    assert (kc.cpu().permute(0, 2, 1, 3).reshape(n_pages * ps, -1)[untouched] == 0).all()
+    # interleaved pairs, no norm, partial rotary dim
+    rd = hd // 2 if (hd // 2) % 2 == 0 else hd
+    q2 = torch.empty(T, H * hd, dtype=dt, device=gpu)
+    k2 = torch.empty(T, Hkv * hd, dtype=dt, device=gpu)
+    jf = torch.arange(rd // 2, dtype=torch.float64)
+    ops.qkv_post(qkv.to(gpu), q2, H=H, Hkv=Hkv, hd=hd, positions=pos.to(gpu), k_out=k2,
+                 inv_freq=(base ** (-2 * jf / rd)).float().to(gpu), rotary_dim=rd, interleaved=True)
+    want = qs.clone()
+    want[..., :rd] = _interleaved_rope(qs[..., :rd], pos, base)
+    assert (q2.cpu().double().reshape(T, H, hd) - want).abs().max() <= tol * float(want.abs().max())
+    wantk = ks.clone()
+    wantk[..., :rd] = _interleaved_rope(ks[..., :rd], pos, base)
+    assert (k2.cpu().double().reshape(T, Hkv, hd) - wantk).abs().max() <= tol * float(wantk.abs().max())
+
+
+# -------------------------------------------------------------------------- attention
+def _attention_reference(q, K, V, pos, window, scale):
+    """q [H, hd]; K, V [n, Hkv, hd] of one request; keys lo..pos."""
+    H, hd = q.shape
+    g = H // K.shape[1]
+    lo = max(0, pos - window + 1) if window else 0
+    k = K[lo:pos + 1].repeat_interleave(g, dim=1)
+    v = V[lo:pos + 1].repeat_interleave(g, dim=1)
+    s = torch.einsum("hd,thd->ht", q, k) * scale
+    p = torch.softmax(s, dim=-1)
+    return torch.einsum("ht,thd->hd", p, v)
+
+
+def _paged_case(gpu, dt, H, Hkv, hd, ps, lens, window, seed=0):
+    """Requests of the given lengths with shuffled pages; queries for the last few tokens of each."""
+    g = torch.Generator().manual_seed(seed)
+    n_blocks = [-(-n // ps) for n in lens]
+    n_pages = sum(n_blocks) + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    kc = _r(n_pages, Hkv, ps, hd, seed=seed + 1, dtype=dt)
+    vc = _r(n_pages, Hkv, ps, hd, seed=seed + 2, dtype=dt)
+    maxb = max(n_blocks) + 1
+    table = torch.full((len(lens), maxb), -1, dtype=torch.int32)
+    Ks, Vs = [], []
+    for r, nb in enumerate(n_blocks):
+        pages = [perm.pop() for _ in range(nb)]
+        table[r, :nb] = torch.tensor(pages, dtype=torch.int32)
+        Ks.append(kc[pages].permute(0, 2, 1, 3).reshape(nb * ps, Hkv, hd).double())
+        Vs.append(vc[pages].permute(0, 2, 1, 3).reshape(nb * ps, Hkv, hd).double())
+    req, pos = [], []
+    for r, n in enumerate(lens):
+        for p in sorted({0, n // 2, max(0, n - 2), n - 1}):
+            req.append(r)
+            pos.append(p)
+    T = len(req)
+    q = _r(T, H * hd, seed=seed + 3, dtype=dt)
+    return kc, vc, table, torch.tensor(req, dtype=torch.int32), torch.tensor(pos, dtype=torch.int32), q, Ks, Vs
+
+
+@pytest.mark.parametrize("H,Hkv,hd,ps", [(4, 2, 16, 16), (4, 1, 24, 8), (3, 3, 80, 16), (2, 1, 256, 32),
+                                          (8, 2, 64, 64), (6, 2, 128, 16), (1, 1, 48, 1)])
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_general(gpu, H, Hkv, hd, ps, dt, window):
+    from tuff_amd.csrc import ops
+    lens = [1, 63, 64, 65, 200, 130]
+    kc, vc, table, req, pos, q, Ks, Vs = _paged_case(gpu, dt, H, Hkv, hd, ps, lens, window)
+    out = torch.empty(q.shape, dtype=dt, device=gpu)
+    ops.attention_general(q.to(gpu), kc.to(gpu), vc.to(gpu), out, block_table=table.to(gpu),
+                          req_of_token=req.to(gpu), positions=pos.to(gpu), H=H, Hkv=Hkv, hd=hd,
+                          page_size=ps, window=window)
+    scale = 1 / math.sqrt(hd)
+    for t in range(len(req)):
+        want = _attention_reference(q[t].double().reshape(H, hd), Ks[req[t]], Vs[req[t]], int(pos[t]), window, scale)
+        got = out[t].cpu().double().reshape(H, hd)
+        tol = 2e-6 if dt == torch.float32 else 2 ** -7
+        assert (got - want).abs().max() <= tol * max(1.0, float(want.abs().max())), (t, int(req[t]), int(pos[t]))
+
+
+def test_attention_finds_a_far_key(gpu):
+    """One key among hundreds matches the query: the output must be that key's value row,
+    wherever the key sits (first position, a page's edge, a tile's edge, the last position)."""
+    from tuff_amd.csrc import ops
+    H = Hkv = 1
+    hd, ps, n = 32, 16, 700
+    for dt in (torch.float32, torch.bfloat16):
+        for hot in (0, 15, 16, 63, 64, 447, 448, 699):
+            kc = _r(n // ps + 1, 1, ps, hd, seed=3, scale=0.05, dtype=dt)
+            vc = _r(n // ps + 1, 1, ps, hd, seed=4, dtype=dt)
+            q = torch.zeros(1, hd, dtype=dt)
+            q[0, 5] = 30.0
+            kc[hot // ps, 0, hot % ps, 5] = 30.0                     # score 900/sqrt(32) = 159 above the rest
+            table = torch.arange(n // ps + 1, dtype=torch.int32)[None]
+            out = torch.empty(1, hd, dtype=dt, device=gpu)
+            ops.attention_general(q.to(gpu), kc.to(gpu), vc.to(gpu), out, block_table=table.to(gpu),
+                                  req_of_token=torch.zeros(1, dtype=torch.int32, device=gpu),
+                                  positions=torch.tensor([n - 1], dtype=torch.int32, device=gpu),
+                                  H=1, Hkv=1, hd=hd, page_size=ps)
+            assert torch.equal(out.cpu()[0], vc[hot // ps, 0, hot % ps]), (dt, hot)
+
+
+def test_attention_window_edge(gpu):
+    """With window W the key at pos - W + 1 is seen and the key at pos - W is not."""
+    from tuff_amd.csrc import ops
+    hd, ps, W, pos = 16, 16, 40, 100
+    for edge, seen in ((pos - W + 1, True), (pos - W, False)):
+        kc = torch.zeros(8, 1, ps, hd)
+        vc = torch.zeros(8, 1, ps, hd)
+        q = torch.zeros(1, hd)
+        q[0, 0] = 20.0
+        kc[edge // ps, 0, edge % ps, 0] = 20.0
+        vc[edge // ps, 0, edge % ps, :] = 1.0
+        out = torch.empty(1, hd, device=gpu)
+        ops.attention_general(q.to(gpu), kc.to(gpu), vc.to(gpu), out,
+                              block_table=torch.arange(8, dtype=torch.int32, device=gpu)[None],
+                              req_of_token=torch.zeros(1, dtype=torch.int32, device=gpu),
+                              positions=torch.tensor([pos], dtype=torch.int32, device=gpu),
+                              H=1, Hkv=1, hd=hd, page_size=ps, window=W)
+        if seen:
+            assert out.min() > 0.999
+        else:
+            assert out.abs().max() == 0
+
+
+# ------------------------------------------------------------------------- short conv
+@pytest.mark.parametrize("d,K", [(64, 3), (96, 4), (240, 2), (300, 7)])
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_shortconv(gpu, d, K, dt):
+    """Two requests cut into different portions; outputs and final states equal the plain
+    whole-sequence convolution."""
+    from tuff_amd.csrc import ops
+    lens = [23, 9]
+    w = _r(d, K, seed=20, dtype=dt)
+    bcx_all = [_r(n, 3 * d, seed=21 + i, dtype=dt) for i, n in enumerate(lens)]
+
+    def whole(bcx):
+        x = bcx.double()
+        u = x[:, :d] * x[:, 2 * d:]
+        hist = torch.cat([torch.zeros(K - 1, d, dtype=torch.float64), u])
+        y = sum(hist[k:k + len(u)] * w.double()[:, k] for k in range(K))
+        return x[:, d:2 * d] * y, hist[-(K - 1):]
+    state = torch.zeros(4, K - 1, d, device=gpu)
+    slots = torch.tensor([2, 0], dtype=torch.int32, device=gpu)
+    cuts = [[5, 1, 1, 10, 6], [1, 2, 6]]
+    outs = [[], []]
+    done = [0, 0]
+    for step in range(5):
+        rows, q_start, q_len, req_of, who = [], [], [], [], []
+        for r in range(2):
+            if step < len(cuts[r]):
+                n = cuts[r][step]
+                q_start.append(sum(q_len))
+                q_len.append(n)
+                req_of += [len(who)] * n
+                who.append(r)
+                rows.append(bcx_all[r][done[r]:done[r] + n])
+                done[r] += n
+        bcx = torch.cat(rows).to(gpu)
+        out = torch.empty(bcx.shape[0], d, dtype=dt, device=gpu)
+        meta = dict(q_start=torch.tensor(q_start, dtype=torch.int32, device=gpu),
+                    state_slot=torch.tensor([[2, 0][r] for r in who], dtype=torch.int32, device=gpu))
+        ops.shortconv_fwd(bcx, w.to(gpu), state, out, req_of_token=torch.tensor(req_of, dtype=torch.int32, device=gpu),
+                          K=K, **meta)
+        ops.shortconv_state(bcx, state, q_len=torch.tensor(q_len, dtype=torch.int32, device=gpu), K=K, **meta)
+        for i, r in enumerate(who):
+            outs[r].append(out[q_start[i]:q_start[i] + q_len[i]].cpu())
+    for r in range(2):
+        want, want_state = whole(bcx_all[r])
+        got = torch.cat(outs[r]).double()
+        tol = 1e-6 if dt == torch.float32 else 2 ** -8
+        assert (got - want).abs().max() <= tol * float(want.abs().max())
+        assert (state[int(slots[r])].cpu().double() - want_state).abs().max() <= 1e-6
+    assert (state[1] == 0).all() and (state[3] == 0).all()       # other requests' slots untouched
+
+
+def test_shortconv_last_tap_is_the_current_token(gpu):
+    from tuff_amd.csrc import ops
+    d, K = 32, 3
+    w = torch.zeros(d, K)
+    w[:, K - 1] = 1.0
+    bcx = _r(6, 3 * d, seed=30)
+    out = torch.empty(6, d, device=gpu)
+    z = torch.zeros(1, dtype=torch.int32, device=gpu)
+    ops.shortconv_fwd(bcx.to(gpu), w.to(gpu), torch.zeros(1, K - 1, d, device=gpu), out,
+                      req_of_token=torch.zeros(6, dtype=torch.int32, device=gpu), q_start=z, state_slot=z, K=K)
+    want = bcx[:, d:2 * d] * bcx[:, :d] * bcx[:, 2 * d:]
+    assert torch.allclose(out.cpu(), want, atol=1e-6)
+
+
+# --------------------------------------------------------------------------- sampling
+def test_argmax_ties_go_to_the_lowest_index(gpu):
+    from tuff_amd.csrc import ops
+    l = _r(5, 1000, seed=40)
+    l[0, 17] = l[0, 700] = 9.0
+    l[1, 999] = 9.0
+    l[2, :] = 0.0
+    l[3, 0] = 9.0
+    out = torch.empty(5, dtype=torch.int32, device=gpu)
+    ops.argmax(l.to(gpu), out)
+    assert out.cpu().tolist() == [17, 999, 0, 0, int(l[4].argmax())]
+    out2 = torch.empty(5, dtype=torch.int32, device=gpu)
+    ops.sample(l.to(gpu), out2)
+    assert torch.equal(out, out2)
+
+
+@pytest.mark.parametrize("params", [dict(temp=0.8), dict(temp=1.0, top_k=5), dict(temp=0.7, top_p=0.9),
+                                    dict(temp=1.3, min_p=0.05), dict(temp=0.9, top_k=40, top_p=0.8, min_p=0.01),
+                                    dict(temp=2.0, top_k=1)])
+def test_sample_matches_the_plain_sampler(gpu, params):
+    """The same draws give the same tokens as the plain restatement of the reference's sampler,
+    except where the draw falls within float32 rounding of a boundary between two candidates."""
+    from plain.sampler_plain import PlainSampler
+    from tuff_amd.csrc import ops
+    V, R = 3001, 64
+    logits = _r(R, V, seed=41, scale=3.0)
+    plain_s = PlainSampler(seed=123, **params)
+    us, want = [], []
+    for r in range(R):
+        probe = PlainSampler(seed=123, **params)
+        probe.rng.s = list(plain_s.rng.s)
+        us.append(float(probe.rng.uniform()))
+        want.append(plain_s.sample(logits[r].numpy()))
+    out = torch.empty(R, dtype=torch.int32, device=gpu)
+    f = lambda key, default, dt: torch.full((R,), params.get(key, default), dtype=dt, device=gpu)
+    ops.sample(logits.to(gpu), out, temps=f("temp", 0.0, torch.float32), top_ks=f("top_k", 0, torch.int32),
+               top_ps=f("top_p", 1.0, torch.float32), min_ps=f("min_p", 0.0, torch.float32),
+               uniforms=torch.tensor(us, dtype=torch.float32, device=gpu))
+    got = out.cpu().tolist()
+    differ = [r for r in range(R) if got[r] != want[r]]
+    for r in differ:
+        # allowed only if the two tokens are neighbours in the sorted order and r is at their border
+        p = torch.softmax(logits[r].double() / params["temp"], 0)
+        order = torch.argsort(-p)
+        rank = {int(t): i for i, t in enumerate(order)}
+        assert abs(rank[got[r]] - rank[want[r]]) == 1, (r, got[r], want[r])
+    assert len(differ) <= 1
+
+
+def test_sample_top_k_ties_and_uniform_logits(gpu):
+    from tuff_amd.csrc import ops
+    V = 500
+    l = torch.zeros(3, V)
+    out = torch.empty(3, dtype=torch.int32, device=gpu)
+    u = torch.tensor([0.0, 0.5, 0.999999], dtype=torch.float32, device=gpu)
+    ones = torch.ones(3, device=gpu)
+    ops.sample(l.to(gpu), out, temps=ones, uniforms=u)
+    assert out.cpu().tolist() == [0, 249, 499]           # equal values are ordered by index
+    ops.sample(l.to(gpu), out, temps=ones, top_ks=torch.full((3,), 10, dtype=torch.int32, device=gpu), uniforms=u)
+    assert out.cpu().tolist() == [0, 4, 9]
+
+
+def test_repeat_penalty(gpu):
+    from tuff_amd.csrc import ops
+    l = torch.tensor([[2.0, -2.0, 1.0, 4.0]] * 2)
+    recent = torch.tensor([[0, 1, 0, 9], [3, 3, 3, 3]], dtype=torch.int32)
+    g = l.to(gpu)
+    ops.repeat_penalty(g, recent.to(gpu), torch.tensor([3, 2], dtype=torch.int32, device=gpu),
+                       torch.tensor([2.0, 1.0], device=gpu))
+    assert g.cpu().tolist() == [[0.5, -4.0, 1.0, 4.0], [2.0, -2.0, 1.0, 4.0]]

@@ -1,0 +1,143 @@
+"""The engine against the plain implementation under every way of cutting and batching:
+whole requests, a long head then 32 single tokens, portions of changing size, and up to four
+live requests mixed with so few pages that they are used again.  float32 and bfloat16."""
+import os
+
+import pytest
+import torch
+
+import util
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = [45, 70, 100, 33, 129, 64]
+
+
+def requests_for(name):
+    V = util.CONFIGS[name][0]["vocab_size"]
+    return {f"r{i}": util.rand_tokens(n, V, 100 * i + len(name)) for i, n in enumerate(LENGTHS)}
+
+
+def stored_for(dtype):
+    return "float32" if dtype == "float32" else "bfloat16"
+
+
+def make_engine(name, dtype, **kw):
+    from tuff_amd.engine.engine import Engine
+    kw.setdefault("page_size", 16)
+    kw.setdefault("max_tokens", 1024)
+    return Engine.from_folder(util.model_folder(name, stored_for(dtype)), dtype=dtype, **kw)
+
+
+def check_plan(name, dtype, plan, reqs, **kw):
+    eng = make_engine(name, dtype, **kw)
+    got = util.run_plan(eng, plan)
+    eng.manager.check()
+    assert not eng.manager.live()
+    for rid, toks in reqs.items():
+        want = util.plain_logits(name, toks, stored_for(dtype))
+        util.assert_close(dtype, got[rid], want, f"{name}/{dtype}/{rid}")
+    return eng, got
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole(gpu, name, dtype):
+    reqs = requests_for(name)
+    check_plan(name, dtype, util.plan_whole(reqs), reqs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_head_then_single_tokens(gpu, name, dtype):
+    reqs = requests_for(name)
+    check_plan(name, dtype, util.plan_tail(reqs, 32), reqs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_changing_portions(gpu, name, dtype):
+    reqs = requests_for(name)
+    check_plan(name, dtype, util.plan_chunks(reqs), reqs)
+    check_plan(name, dtype, util.plan_chunks(reqs, sizes=(2, 2, 3, 2, 29)), reqs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_with_page_reuse(gpu, name, dtype):
+    reqs = requests_for(name)
+    for seed in (0, 1):
+        plan = util.plan_mixed(reqs, seed=seed)
+        assert max(len(s["entries"]) for s in plan) >= 3          # really mixed
+        assert any(len(e["tokens"]) == 1 for s in plan if len(s["entries"]) > 1 for e in s["entries"])
+        peak = util.live_tokens_peak(plan)
+        eng, _ = check_plan(name, dtype, plan, reqs, max_tokens=peak, max_requests=4)
+        pool = eng.manager.groups[0].pool
+        assert pool.allocations > pool.num_pages, "the pool was so large that no page was used again"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_splits_agree_with_each_other(gpu, dtype):
+    """The same logits whatever the cutting: bitwise in float32 where the kernels keep one order
+    of summation per position, to rounding in bfloat16."""
+    name = "B"
+    reqs = requests_for(name)
+    eng = make_engine(name, dtype)
+    whole = util.run_plan(eng, util.plan_whole(reqs))
+    for plan in (util.plan_tail(reqs), util.plan_chunks(reqs), util.plan_mixed(reqs, seed=3)):
+        other = util.run_plan(eng, plan)
+        for rid in reqs:
+            if dtype == "float32":
+                assert torch.equal(whole[rid], other[rid]), f"{rid}: float32 logits depend on the cutting"
+            else:
+                util.assert_close_bf16(other[rid], whole[rid], rid, rms=0.02)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decode(gpu, dtype):
+    """300 tokens one by one after a short prompt: crosses key tiles and many pages."""
+    name = "A"
+    toks = util.rand_tokens(330, util.TINY_A["vocab_size"], 77)
+    reqs = {"long": toks}
+    check_plan(name, dtype, util.plan_tail(reqs, 300), reqs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens(gpu, name, dtype):
+    """Positions 0, 1, 2 fed one by one, and prompts of one and two tokens."""
+    V = util.CONFIGS[name][0]["vocab_size"]
+    reqs = {"one": util.rand_tokens(1, V, 1), "two": util.rand_tokens(2, V, 2), "three": util.rand_tokens(3, V, 3)}
+    check_plan(name, dtype, util.plan_whole(reqs), reqs)
+    check_plan(name, dtype, util.plan_tail(reqs, 3), reqs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(gpu, dtype, tmp_path):
+    """bin/trace_run as a child process gives what the engine gives in this process."""
+    name = "B"
+    reqs = requests_for(name)
+    plan = util.plan_mixed(reqs, seed=5)
+    peak = util.live_tokens_peak(plan)
+    folder = util.model_folder(name, stored_for(dtype))
+    got = util.run_trace_run(folder, dtype, plan, peak, str(tmp_path / "out"))
+    eng = make_engine(name, dtype, max_tokens=peak)
+    here = util.run_plan(eng, plan)
+    for rid, toks in reqs.items():
+        util.assert_close(dtype, got[rid], util.plain_logits(name, toks, stored_for(dtype)), rid)
+        assert torch.equal(got[rid], here[rid])
+
+
+def test_out_of_pages_leaves_everything_as_it_was(gpu):
+    from tuff_amd.cache.manager import OutOfPages
+    from tuff_amd.engine.batch import StepEntry
+    eng = make_engine("A", "float32", max_tokens=64)
+    eng.begin("a")
+    eng.begin("b")
+    eng.step([StepEntry("a", list(range(40)), [39])])
+    with pytest.raises(OutOfPages):
+        eng.step([StepEntry("a", [1], [0]), StepEntry("b", list(range(30)), [29])])
+    assert eng.length("a") == 40 and eng.length("b") == 0
+    eng.manager.check()
+    eng.step([StepEntry("a", [1], [0]), StepEntry("b", list(range(10)), [9])])
+    eng.manager.check()

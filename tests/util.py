@@ -1,0 +1,258 @@
+"""Shared helpers of the tests: tiny configurations, model folders, replay plans."""
+from __future__ import annotations
+
+import functools
+import json
+import os
+import random
+import subprocess
+import sys
+import tempfile
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# Three tiny configurations that differ in every size and option.
+TINY_A = dict(
+    architectures=["Lfm2ForCausalLM"], num_hidden_layers=4,
+    layer_types=["conv", "conv", "full_attention", "conv"],
+    hidden_size=64, num_attention_heads=4, num_key_value_heads=2,
+    block_ff_dim=192, block_auto_adjust_ff_dim=False, vocab_size=512, rope_theta=10000.0,
+    conv_L_cache=3, norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=4096)
+TINY_B = dict(
+    architectures=["Lfm2ForCausalLM"], num_hidden_layers=6,
+    layer_types=["full_attention", "conv", "conv", "full_attention", "conv", "full_attention"],
+    hidden_size=96, num_attention_heads=4, num_key_value_heads=1,
+    block_ff_dim=384, block_auto_adjust_ff_dim=True, block_multiple_of=64, vocab_size=1000,
+    rope_theta=1000000.0, conv_L_cache=4, norm_eps=1e-6, tie_word_embeddings=False,
+    max_position_embeddings=2048)
+TINY_C = dict(
+    architectures=["Lfm2ForCausalLM"], num_hidden_layers=3,
+    layer_types=["full_attention", "conv", "full_attention"],
+    hidden_size=240, num_attention_heads=3, num_key_value_heads=3,
+    block_ff_dim=328, block_auto_adjust_ff_dim=False, vocab_size=777, rope_theta=500000.0,
+    conv_L_cache=2, norm_eps=3e-6, tie_word_embeddings=True, max_position_embeddings=1024)
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 5)}
+
+_TMP = tempfile.TemporaryDirectory(prefix="tuff_amd_tests_")
+
+
+@functools.lru_cache(maxsize=None)
+def model_folder(name: str, stored: str = "bfloat16") -> str:
+    """A model folder of configuration `name` with random weights, made once per session."""
+    from tuff_amd.models.registry import config_from_dict
+    from tuff_amd.weights.random_init import write_random_model
+    raw, seed = CONFIGS[name]
+    out = os.path.join(_TMP.name, f"{name}_{stored}")
+    write_random_model(config_from_dict(raw), out, seed, getattr(torch, stored))
+    return out
+
+
+@functools.lru_cache(maxsize=None)
+def plain_model(name: str, stored: str = "bfloat16"):
+    from plain.lfm2_plain import read_model
+    return read_model(model_folder(name, stored))
+
+
+def plain_logits(name: str, tokens, stored: str = "bfloat16") -> torch.Tensor:
+    from plain.lfm2_plain import forward_logits
+    cfg, w = plain_model(name, stored)
+    return forward_logits(cfg, w, list(tokens))
+
+
+def rand_tokens(n: int, vocab: int, seed: int) -> list[int]:
+    rng = random.Random(seed)
+    return [rng.randrange(vocab) for _ in range(n)]
+
+
+# ------------------------------------------------------------------------------ plans
+# A plan is a list of steps in the format bin/trace_run reads.
+def plan_whole(reqs: dict) -> list[dict]:
+    return [{"step": i, "entries": [{"id": rid, "tokens": toks, "want": list(range(len(toks)))}], "end": [rid]}
+            for i, (rid, toks) in enumerate(reqs.items())]
+
+
+def plan_tail(reqs: dict, tail: int = 32) -> list[dict]:
+    """Most of each request in one step, its last `tail` tokens one by one."""
+    steps = []
+    for rid, toks in reqs.items():
+        head = max(1, len(toks) - tail)
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": toks[:head], "want": list(range(head))}],
+                      "end": []})
+        for j in range(head, len(toks)):
+            steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": [toks[j]], "want": [0]}], "end": []})
+        steps[-1]["end"] = [rid]
+    return steps
+
+
+def plan_chunks(reqs: dict, sizes=(7, 2, 13, 3, 2, 5, 31, 2, 64, 17)) -> list[dict]:
+    """Each request alone, in portions of changing size, down to two tokens."""
+    steps = []
+    for rid, toks in reqs.items():
+        i, k = 0, 0
+        while i < len(toks):
+            n = min(sizes[k % len(sizes)], len(toks) - i)
+            k += 1
+            steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": toks[i:i + n], "want": list(range(n))}],
+                          "end": []})
+            i += n
+        steps[-1]["end"] = [rid]
+    return steps
+
+
+def plan_mixed(reqs: dict, seed: int = 0, max_live: int = 4, decode_tail: int = 12) -> list[dict]:
+    """Up to `max_live` requests live at a time.  Each request is fed in portions of random size
+    (2..40) until `decode_tail` tokens remain, then one token a step; in any step a live request
+    may be left out.  A finished request ends and the next one starts."""
+    rng = random.Random(seed)
+    waiting = list(reqs.items())
+    live: dict = {}
+    steps = []
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            rid, toks = waiting.pop(0)
+            live[rid] = [toks, 0]
+        entries, end = [], []
+        for rid, (toks, done) in list(live.items()):
+            if len(live) > 1 and rng.random() < 0.25:
+                continue                                   # sits this step out
+            left = len(toks) - done
+            n = 1 if left <= decode_tail else min(left - decode_tail, rng.choice([2, 3, 5, 8, 16, 23, 40]))
+            entries.append({"id": rid, "tokens": toks[done:done + n], "want": list(range(n))})
+            live[rid][1] = done + n
+            if done + n == len(toks):
+                end.append(rid)
+        if not entries:
+            continue
+        for rid in end:
+            del live[rid]
+        steps.append({"step": len(steps), "entries": entries, "end": end})
+    return steps
+
+
+def live_tokens_peak(plan) -> int:
+    """Most tokens live requests hold at any time, each rounded up to 64."""
+    held, peak = {}, 0
+    for s in plan:
+        for e in s["entries"]:
+            held[e["id"]] = held.get(e["id"], 0) + len(e["tokens"])
+        peak = max(peak, sum(-(-v // 64) * 64 for v in held.values()))
+        for rid in s["end"]:
+            held.pop(rid, None)
+    return peak
+
+
+# ---------------------------------------------------------------------------- running
+def run_plan(engine, plan) -> dict:
+    """Runs a plan on an Engine in this process.  Returns {req id: float32 [n_tokens, vocab]}
+    with the logits of every wanted place (NaN rows where nothing was wanted)."""
+    from tuff_amd.engine.batch import StepEntry
+    fed: dict = {}
+    rows: dict = {}
+    for s in plan:
+        entries = []
+        for e in s["entries"]:
+            if not engine.is_live(e["id"]):
+                engine.begin(e["id"])
+                fed[e["id"]] = 0
+                rows[e["id"]] = {}
+            entries.append(StepEntry(e["id"], e["tokens"], e["want"]))
+        logits = engine.step(entries)
+        if logits is not None:
+            logits = logits.float().cpu()
+            i = 0
+            for e in s["entries"]:
+                for w in e["want"]:
+                    rows[e["id"]][fed[e["id"]] + w] = logits[i]
+                    i += 1
+        for e in s["entries"]:
+            fed[e["id"]] += len(e["tokens"])
+        for rid in s["end"]:
+            engine.end(rid)
+    out = {}
+    for rid, d in rows.items():
+        n = fed[rid]
+        V = next(iter(d.values())).shape[0]
+        t = torch.full((n, V), float("nan"))
+        for pos, row in d.items():
+            t[pos] = row
+        out[rid] = t
+    return out
+
+
+def run_trace_run(model_dir: str, dtype: str, plan, max_tokens: int, out_dir: str, extra=()) -> dict:
+    """Runs a plan through bin/trace_run as a child process and reads back its files."""
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype,
+           "--out", out_dir, "--max-tokens", str(max_tokens), *extra]
+    proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    try:
+        for s in plan:
+            proc.stdin.write(json.dumps(s) + "\n")
+            proc.stdin.flush()
+            line = proc.stdout.readline().strip()
+            assert line == f"done {s['step']}", f"trace_run answered {line!r} to step {s['step']}"
+        proc.stdin.close()
+        assert proc.wait(timeout=120) == 0
+    finally:
+        if proc.poll() is None:
+            proc.kill()
+    with open(os.path.join(model_dir, "config.json")) as f:
+        V = json.load(f)["vocab_size"]
+    fed, rows = {}, {}
+    for s in plan:
+        n_want = sum(len(e["want"]) for e in s["entries"])
+        path = os.path.join(out_dir, f"{s['step']}.f32")
+        if n_want:
+            data = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(n_want, V).copy())
+        else:
+            assert not os.path.exists(path)
+        i = 0
+        for e in s["entries"]:
+            fed.setdefault(e["id"], 0)
+            rows.setdefault(e["id"], {})
+            for w in e["want"]:
+                rows[e["id"]][fed[e["id"]] + w] = data[i]
+                i += 1
+            fed[e["id"]] += len(e["tokens"])
+    return {rid: torch.stack([d[p] for p in sorted(d)]) for rid, d in rows.items()}
+
+
+# -------------------------------------------------------------------------- comparing
+# Tolerances, fixed up front.  float32: the engine adds in another order than the float64
+# plain implementation; with logits of spread ~0.2 that is 1e-6..1e-5.  bfloat16: roundings of
+# relative size 2^-9 at ~10 places a layer add up like a random walk, ~2^-9 * sqrt(10 L) of the
+# logits' spread: 3 % for 6 layers is the bound on the RMS error, 5 sigma of it on any element.
+def assert_close_f32(got: torch.Tensor, want: torch.Tensor, what: str = ""):
+    got, want = got.double(), want.double()
+    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
+    assert torch.isfinite(got).all(), f"{what}: non-finite logits"
+    err = (got - want).abs()
+    tol = 2e-5 + 1e-4 * want.abs()
+    if not (err <= tol).all():
+        bad = torch.nonzero(err > tol)
+        first = bad[0].tolist()
+        raise AssertionError(f"{what}: {len(bad)} elements differ, first at {first} "
+                             f"(got {got[tuple(first)]:.7f}, want {want[tuple(first)]:.7f}), max err {err.max():.3e}")
+
+
+def rel_rms(got: torch.Tensor, want: torch.Tensor) -> float:
+    got, want = got.double(), want.double()
+    return float(((got - want).pow(2).mean() / want.pow(2).mean().clamp_min(1e-30)).sqrt())
+
+
+def assert_close_bf16(got: torch.Tensor, want: torch.Tensor, what: str = "", rms: float = 0.03):
+    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
+    assert torch.isfinite(got).all(), f"{what}: non-finite logits"
+    want = want.double()
+    spread = float(want.pow(2).mean().sqrt())
+    per_row = ((got.double() - want).pow(2).mean(-1).sqrt() / spread)
+    worst = int(per_row.argmax())
+    assert per_row.max() <= rms, f"{what}: row {worst} has relative RMS error {per_row.max():.4f} > {rms}"
+    mx = float((got.double() - want).abs().max()) / spread
+    assert mx <= 6 * rms, f"{what}: largest error {mx:.4f} of the spread > {6 * rms}"
+
+
+def assert_close(dtype: str, got, want, what=""):
+    (assert_close_f32 if dtype == "float32" else assert_close_bf16)(got, want, what)

@@ -1,0 +1,115 @@
+// Row-wise kernels of the residual stream: embedding gather, RMSNorm, SwiGLU gate,
+// casts and fills.  The residual stream is float32 in every mode; sums of squares
+// are taken in float32 in a fixed order.
+#include "common.h"
+
+// ------------------------------------------------------------------ embedding
+// out[t, :] = table[tokens[t], :] as float32.  Reference: one row gather per token
+// with no scale (src/lfm25_gpu.cu:725-741).
+template <typename T>
+__global__ void embed_rows_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
+                                  float* __restrict__ out, int d) {
+    const int t = blockIdx.x;
+    const long long row = tokens[t];
+    const T* src = table + row * (long long)d;
+    float* dst = out + (long long)t * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) dst[i] = to_f32(src[i]);
+}
+
+TUFF_EXPORT int tuff_embed_rows(const void* table, int table_dt, const int* tokens, float* out,
+                                int n_tokens, int d, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    dim3 grid(n_tokens), block(256);
+    if (table_dt == DT_F32)
+        hipLaunchKernelGGL(embed_rows_kernel<float>, grid, block, 0, stream, (const float*)table, tokens, out, d);
+    else
+        hipLaunchKernelGGL(embed_rows_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, tokens, out, d);
+    return launch_status();
+}
+
+// -------------------------------------------------------------------- RMSNorm
+// y_i = x_i * (1 / sqrt(mean_j x_j^2 + eps)) * w_i   (src/lfm25_gpu.cu:235,244).
+// `rows` (optional) gathers input rows: output row r is the norm of x[rows[r]].
+// Per-thread strided partial sums -> wave butterfly -> wave partials in order.
+template <typename TW, typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ w,
+                               TO* __restrict__ out, const int* __restrict__ rows, int d, float eps) {
+    __shared__ float scratch[4];
+    const int r = blockIdx.x;
+    const long long src = rows ? rows[r] : r;
+    const float* xr = x + src * (long long)d;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < d; i += 256) { const float v = xr[i]; ss += v * v; }
+    const float total = block_sum<4>(ss, scratch);
+    const float inv = 1.0f / sqrtf(total / (float)d + eps);
+    TO* o = out + (long long)r * d;
+    for (int i = threadIdx.x; i < d; i += 256) o[i] = from_f32<TO>(xr[i] * inv * to_f32(w[i]));
+}
+
+TUFF_EXPORT int tuff_rmsnorm(const float* x, const void* w, int w_dt, void* out, int out_dt,
+                             const int* rows, int n_rows, int d, float eps, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    dim3 grid(n_rows), block(256);
+#define LAUNCH(TW, TO) hipLaunchKernelGGL((rmsnorm_kernel<TW, TO>), grid, block, 0, stream, x, (const TW*)w, (TO*)out, rows, d, eps)
+    if (w_dt == DT_F32 && out_dt == DT_F32) LAUNCH(float, float);
+    else if (w_dt == DT_F32 && out_dt == DT_BF16) LAUNCH(float, bf16_t);
+    else if (w_dt == DT_BF16 && out_dt == DT_F32) LAUNCH(bf16_t, float);
+    else LAUNCH(bf16_t, bf16_t);
+#undef LAUNCH
+    return launch_status();
+}
+
+// --------------------------------------------------------------------- SwiGLU
+// act[t, f] = g / (1 + exp(-g)) * u with g = gu[t, f], u = gu[t, F + f]
+// (src/lfm25_gpu.cu:614-617), evaluated in float32.
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ act, long long n, int F) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const long long t = i / F;
+    const int f = (int)(i - t * F);
+    const float g = to_f32(gu[t * 2 * F + f]);
+    const float u = to_f32(gu[t * 2 * F + F + f]);
+    act[i] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+}
+
+TUFF_EXPORT int tuff_swiglu(const void* gu, void* act, int dt, int n_tokens, int F, hipStream_t stream) {
+    const long long n = (long long)n_tokens * F;
+    if (n <= 0) return 0;
+    dim3 grid((unsigned)ceil_div_ll(n, 256)), block(256);
+    if (dt == DT_F32) hipLaunchKernelGGL(swiglu_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)act, n, F);
+    else hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)act, n, F);
+    return launch_status();
+}
+
+// ----------------------------------------------------------------------- cast
+template <typename TI, typename TO>
+__global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, long long n) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = from_f32<TO>(to_f32(in[i]));
+}
+
+TUFF_EXPORT int tuff_cast(const void* in, int in_dt, void* out, int out_dt, long long n, hipStream_t stream) {
+    if (n <= 0) return 0;
+    dim3 grid((unsigned)ceil_div_ll(n, 256)), block(256);
+    if (in_dt == DT_F32 && out_dt == DT_BF16) hipLaunchKernelGGL((cast_kernel<float, bf16_t>), grid, block, 0, stream, (const float*)in, (bf16_t*)out, n);
+    else if (in_dt == DT_BF16 && out_dt == DT_F32) hipLaunchKernelGGL((cast_kernel<bf16_t, float>), grid, block, 0, stream, (const bf16_t*)in, (float*)out, n);
+    else if (in_dt == DT_F32) hipLaunchKernelGGL((cast_kernel<float, float>), grid, block, 0, stream, (const float*)in, (float*)out, n);
+    else hipLaunchKernelGGL((cast_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (const bf16_t*)in, (bf16_t*)out, n);
+    return launch_status();
+}
+
+// ----------------------------------------------------------------------- fill
+// Sets n 32-bit words to `value`; used instead of a memset so that a caller may
+// record it into a graph.
+__global__ void fill_u32_kernel(uint32_t* __restrict__ p, uint32_t value, long long n) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = value;
+}
+
+TUFF_EXPORT int tuff_fill_u32(void* p, uint32_t value, long long n, hipStream_t stream) {
+    if (n <= 0) return 0;
+    dim3 grid((unsigned)ceil_div_ll(n, 256)), block(256);
+    hipLaunchKernelGGL(fill_u32_kernel, grid, block, 0, stream, (uint32_t*)p, value, n);
+    return launch_status();
+}

@@ -1,0 +1,341 @@
+"""Python face of the HIP kernels: loads the compiled libraries with ctypes, checks every
+operand on the host (device, dtype, contiguity, shape) and launches on torch's current stream.
+
+There is no other implementation behind these functions: a missing library is compiled, a
+library that cannot be compiled or a tensor that is not on the GPU is an error.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Optional
+
+import torch
+
+from . import build
+
+DT_F32, DT_BF16 = 0, 1
+OUT_BF16, OUT_F32, OUT_F32_ACCUM = 0, 1, 2
+
+_c_int, _c_float, _c_void_p, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_SIGNATURES = {
+    "elementwise": {
+        "tuff_embed_rows": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+        "tuff_rmsnorm": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_float, _c_void_p],
+        "tuff_swiglu": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_cast": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_void_p],
+        "tuff_fill_u32": [_c_void_p, ctypes.c_uint32, _c_ll, _c_void_p],
+    },
+    "gemm_f32": {
+        "tuff_gemm_f32": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    },
+    "gemm_bf16": {
+        "tuff_gemm_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    },
+    "rope_kv": {
+        "tuff_qkv_post": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                          _c_void_p, _c_void_p, _c_int, _c_float,
+                          _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
+                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_kv_write": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
+                          _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    },
+    "attention": {
+        "tuff_attention_general": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
+                                   _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                   _c_float, _c_void_p],
+    },
+    "shortconv": {
+        "tuff_shortconv_fwd": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
+                               _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_shortconv_state": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                                 _c_int, _c_int, _c_int, _c_void_p],
+    },
+    "sampling": {
+        "tuff_argmax": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+        "tuff_sample": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                        _c_int, _c_int, _c_void_p],
+        "tuff_repeat_penalty": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    },
+}
+
+_libs: dict[str, ctypes.CDLL] = {}
+
+
+def load(module: str) -> ctypes.CDLL:
+    """The loaded library of a kernel module; compiled at first use if it is not built yet."""
+    lib = _libs.get(module)
+    if lib is None:
+        path = build.ensure_built(module)
+        lib = ctypes.CDLL(path)
+        for name, argtypes in _SIGNATURES.get(module, {}).items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = _c_int
+        _libs[module] = lib
+    return lib
+
+
+def loaded_modules() -> list[str]:
+    return sorted(_libs)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return DT_F32
+    if t.dtype == torch.bfloat16:
+        return DT_BF16
+    raise KernelError(f"unsupported element type {t.dtype}; kernels take float32 and bfloat16")
+
+
+def _gpu(name: str, t: torch.Tensor, dtype=None, shape=None) -> int:
+    if not isinstance(t, torch.Tensor):
+        raise KernelError(f"{name}: expected a tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise KernelError(f"{name}: tensor is on '{t.device}'; the kernels run on the GPU only "
+                          f"and there is no CPU fallback")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: tensor must be contiguous (shape {tuple(t.shape)}, stride {t.stride()})")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: expected {dtype}, got {t.dtype}")
+    if shape is not None:
+        if len(shape) != t.dim() or any(s is not None and s != g for s, g in zip(shape, t.shape)):
+            raise KernelError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
+    return t.data_ptr()
+
+
+def _opt(name, t, dtype=None, shape=None) -> Optional[int]:
+    return None if t is None else _gpu(name, t, dtype, shape)
+
+
+def _check(code: int, what: str) -> None:
+    if code != 0:
+        if code == -2:
+            raise KernelError(f"{what}: the kernel refuses these sizes")
+        raise KernelError(f"{what}: launch failed with HIP error {code}")
+
+
+# ------------------------------------------------------------------------ row kernels
+def embed_rows(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
+    n, d = out.shape
+    _check(load("elementwise").tuff_embed_rows(
+        _gpu("table", table, shape=(None, d)), _dt(table), _gpu("tokens", tokens, torch.int32, (n,)),
+        _gpu("out", out, torch.float32), n, d, _stream()), "embed_rows")
+
+
+def rmsnorm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, eps: float,
+            rows: Optional[torch.Tensor] = None) -> None:
+    n, d = out.shape
+    if rows is None:
+        _gpu("x", x, torch.float32, (n, d))
+    else:
+        _gpu("x", x, torch.float32, (None, d))
+    _check(load("elementwise").tuff_rmsnorm(
+        x.data_ptr(), _gpu("w", w, shape=(d,)), _dt(w), _gpu("out", out), _dt(out),
+        _opt("rows", rows, torch.int32, (n,)), n, d, float(eps), _stream()), "rmsnorm")
+
+
+def swiglu(gu: torch.Tensor, act: torch.Tensor) -> None:
+    n, F = act.shape
+    _check(load("elementwise").tuff_swiglu(
+        _gpu("gu", gu, act.dtype, (n, 2 * F)), _gpu("act", act), _dt(act), n, F, _stream()), "swiglu")
+
+
+def cast(inp: torch.Tensor, out: torch.Tensor) -> None:
+    if inp.numel() != out.numel():
+        raise KernelError(f"cast: {inp.numel()} elements in, {out.numel()} out")
+    _check(load("elementwise").tuff_cast(_gpu("inp", inp), _dt(inp), _gpu("out", out), _dt(out),
+                                         inp.numel(), _stream()), "cast")
+
+
+def fill_u32(t: torch.Tensor, value: int = 0) -> None:
+    """Sets every 32-bit word of `t` to `value` (t must be a 4-byte type)."""
+    if t.element_size() != 4:
+        raise KernelError("fill_u32: tensor elements must be 4 bytes wide")
+    if not t.is_cuda or not t.is_contiguous():
+        raise KernelError("fill_u32: contiguous GPU tensor required")
+    _check(load("elementwise").tuff_fill_u32(t.data_ptr(), value, t.numel(), _stream()), "fill_u32")
+
+
+# ------------------------------------------------------------------------------ GEMM
+def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out (=|+=) x @ w.T.  x [M, K], w [N, K] of one dtype; float32 operands give the true
+    float32 product, bfloat16 operands the matrix-core product with float32 accumulation.
+    `out` is float32 (stored or accumulated into) or, for bfloat16 operands, bfloat16."""
+    M, K = x.shape
+    N = w.shape[0]
+    _gpu("x", x)
+    _gpu("w", w, x.dtype, (N, K))
+    _gpu("out", out, shape=(M, N))
+    if x.dtype == torch.float32:
+        if out.dtype != torch.float32:
+            raise KernelError("gemm: float32 operands need a float32 output")
+        _check(load("gemm_f32").tuff_gemm_f32(x.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K,
+                                              int(accumulate), _stream()), "gemm_f32")
+        return
+    if x.dtype != torch.bfloat16:
+        raise KernelError(f"gemm: unsupported operand type {x.dtype}")
+    if K % 8 != 0:
+        raise KernelError(f"gemm: the bfloat16 kernels need an inner size that is a multiple of 8, got {K}")
+    if out.dtype == torch.float32:
+        mode = OUT_F32_ACCUM if accumulate else OUT_F32
+    elif out.dtype == torch.bfloat16:
+        if accumulate:
+            raise KernelError("gemm: accumulation needs a float32 output")
+        mode = OUT_BF16
+    else:
+        raise KernelError(f"gemm: unsupported output type {out.dtype}")
+    _check(load("gemm_bf16").tuff_gemm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, mode,
+                                            _stream()), "gemm_bf16")
+
+
+# ----------------------------------------------------------------- q/k/v post-processing
+def qkv_post(qkv, q_out, *, H, Hkv, hd, positions, eps=0.0, q_norm_w=None, k_norm_w=None,
+             inv_freq=None, rotary_dim=0, interleaved=False, k_out=None,
+             k_cache=None, v_cache=None, slot_mapping=None, page_size=1) -> None:
+    T = qkv.shape[0]
+    dt = qkv.dtype
+    _gpu("qkv", qkv, shape=(T, (H + 2 * Hkv) * hd))
+    _gpu("q_out", q_out, dt, (T, H * hd))
+    _opt("k_out", k_out, dt, (T, Hkv * hd))
+    if (k_cache is None) != (v_cache is None):
+        raise KernelError("qkv_post: k_cache and v_cache go together")
+    if k_cache is not None:
+        if slot_mapping is None:
+            raise KernelError("qkv_post: a cache write needs slot_mapping")
+        P = k_cache.shape[0]
+        _gpu("k_cache", k_cache, dt, (P, Hkv, page_size, hd))
+        _gpu("v_cache", v_cache, dt, (P, Hkv, page_size, hd))
+        _gpu("slot_mapping", slot_mapping, torch.int32, (T,))
+    norm_dt = DT_F32
+    if q_norm_w is not None or k_norm_w is not None:
+        if q_norm_w is None or k_norm_w is None or q_norm_w.dtype != k_norm_w.dtype:
+            raise KernelError("qkv_post: q and k norm weights go together and share a dtype")
+        _gpu("q_norm_w", q_norm_w, shape=(hd,))
+        _gpu("k_norm_w", k_norm_w, shape=(hd,))
+        norm_dt = _dt(q_norm_w)
+    if inv_freq is not None:
+        if rotary_dim <= 0 or rotary_dim > hd or rotary_dim % 2:
+            raise KernelError(f"qkv_post: rotary_dim {rotary_dim} must be even and within the head size {hd}")
+        _gpu("inv_freq", inv_freq, torch.float32, (rotary_dim // 2,))
+    _gpu("positions", positions, torch.int32, (T,))
+    if hd > 256:
+        raise KernelError(f"qkv_post: head size {hd} above 256 is not supported")
+    p = lambda t: None if t is None else t.data_ptr()
+    _check(load("rope_kv").tuff_qkv_post(
+        qkv.data_ptr(), q_out.data_ptr(), p(k_out), p(k_cache), p(v_cache), _dt(qkv),
+        p(q_norm_w), p(k_norm_w), norm_dt, float(eps), p(inv_freq), int(rotary_dim), int(interleaved),
+        positions.data_ptr(), p(slot_mapping), T, H, Hkv, hd, page_size, _stream()), "qkv_post")
+
+
+def kv_write(k, v, k_cache, v_cache, slot_mapping, *, Hkv, hd, page_size) -> None:
+    T = k.shape[0]
+    dt = k.dtype
+    _gpu("k", k, shape=(T, Hkv * hd))
+    _gpu("v", v, dt, (T, Hkv * hd))
+    P = k_cache.shape[0]
+    _gpu("k_cache", k_cache, dt, (P, Hkv, page_size, hd))
+    _gpu("v_cache", v_cache, dt, (P, Hkv, page_size, hd))
+    _gpu("slot_mapping", slot_mapping, torch.int32, (T,))
+    _check(load("rope_kv").tuff_kv_write(k.data_ptr(), v.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                         _dt(k), slot_mapping.data_ptr(), T, Hkv, hd, page_size, _stream()),
+           "kv_write")
+
+
+# -------------------------------------------------------------------------- attention
+def attention_general(q, k_cache, v_cache, out, *, block_table, req_of_token, positions,
+                      H, Hkv, hd, page_size, window=0, scale=None) -> None:
+    T = q.shape[0]
+    dt = q.dtype
+    _gpu("q", q, shape=(T, H * hd))
+    _gpu("out", out, dt, (T, H * hd))
+    P = k_cache.shape[0]
+    _gpu("k_cache", k_cache, dt, (P, Hkv, page_size, hd))
+    _gpu("v_cache", v_cache, dt, (P, Hkv, page_size, hd))
+    _gpu("block_table", block_table, torch.int32)
+    if block_table.dim() != 2:
+        raise KernelError("attention: block_table must be [requests, blocks]")
+    _gpu("req_of_token", req_of_token, torch.int32, (T,))
+    _gpu("positions", positions, torch.int32, (T,))
+    if hd > 256 or H % Hkv:
+        raise KernelError(f"attention: head size {hd} / heads {H}:{Hkv} not supported")
+    if scale is None:
+        scale = 1.0 / math.sqrt(hd)
+    _check(load("attention").tuff_attention_general(
+        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _dt(q),
+        block_table.data_ptr(), block_table.shape[1], req_of_token.data_ptr(), positions.data_ptr(),
+        T, H, Hkv, hd, page_size, int(window or 0), float(scale), _stream()), "attention_general")
+
+
+# ------------------------------------------------------------------------- short conv
+def shortconv_fwd(bcx, conv_w, state, out, *, req_of_token, q_start, state_slot, K) -> None:
+    T, d = out.shape
+    dt = out.dtype
+    _gpu("bcx", bcx, dt, (T, 3 * d))
+    _gpu("out", out)
+    _gpu("conv_w", conv_w, shape=(d, K))
+    _gpu("state", state, torch.float32, (None, K - 1, d))
+    R = q_start.shape[0]
+    _gpu("req_of_token", req_of_token, torch.int32, (T,))
+    _gpu("q_start", q_start, torch.int32, (R,))
+    _gpu("state_slot", state_slot, torch.int32, (R,))
+    _check(load("shortconv").tuff_shortconv_fwd(
+        bcx.data_ptr(), conv_w.data_ptr(), _dt(conv_w), state.data_ptr(), out.data_ptr(), _dt(out),
+        req_of_token.data_ptr(), q_start.data_ptr(), state_slot.data_ptr(), T, d, K, _stream()), "shortconv_fwd")
+
+
+def shortconv_state(bcx, state, *, q_start, q_len, state_slot, K) -> None:
+    d = state.shape[2]
+    R = q_start.shape[0]
+    _gpu("bcx", bcx, shape=(None, 3 * d))
+    _gpu("state", state, torch.float32, (None, K - 1, d))
+    _gpu("q_start", q_start, torch.int32, (R,))
+    _gpu("q_len", q_len, torch.int32, (R,))
+    _gpu("state_slot", state_slot, torch.int32, (R,))
+    _check(load("shortconv").tuff_shortconv_state(
+        bcx.data_ptr(), _dt(bcx), state.data_ptr(), q_start.data_ptr(), q_len.data_ptr(),
+        state_slot.data_ptr(), R, d, K, _stream()), "shortconv_state")
+
+
+# --------------------------------------------------------------------------- sampling
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    R, V = logits.shape
+    _check(load("sampling").tuff_argmax(_gpu("logits", logits, torch.float32), _gpu("out", out, torch.int32, (R,)),
+                                        R, V, _stream()), "argmax")
+
+
+def sample(logits, out, *, temps=None, top_ks=None, top_ps=None, min_ps=None, uniforms=None) -> None:
+    """One token per row: greedy where temps[r] <= 0 (or temps is None), else the reference's
+    chain min-p -> top-k -> top-p -> draw with the host-supplied uniform of that row."""
+    R, V = logits.shape
+    _gpu("logits", logits, torch.float32)
+    _gpu("out", out, torch.int32, (R,))
+    if temps is not None and uniforms is None:
+        raise KernelError("sample: stochastic rows need uniforms")
+    p = lambda n, t, dt: None if t is None else _gpu(n, t, dt, (R,))
+    _check(load("sampling").tuff_sample(
+        logits.data_ptr(), p("temps", temps, torch.float32), p("top_ks", top_ks, torch.int32),
+        p("top_ps", top_ps, torch.float32), p("min_ps", min_ps, torch.float32),
+        p("uniforms", uniforms, torch.float32), out.data_ptr(), R, V, _stream()), "sample")
+
+
+def repeat_penalty(logits, recent, counts, penalties) -> None:
+    """In place: each row's logits penalised once per entry of its ring of recent tokens."""
+    R, V = logits.shape
+    cap = recent.shape[1]
+    _gpu("logits", logits, torch.float32)
+    _gpu("recent", recent, torch.int32, (R, cap))
+    _gpu("counts", counts, torch.int32, (R,))
+    _gpu("penalties", penalties, torch.float32, (R,))
+    _check(load("sampling").tuff_repeat_penalty(logits.data_ptr(), recent.data_ptr(), counts.data_ptr(),
+                                                penalties.data_ptr(), R, cap, V, _stream()), "repeat_penalty")

@@ -1,0 +1,139 @@
+// After the q/k/v projection: per-head RMSNorm of q and k, rotary position encoding,
+// and the write of k and v into the paged cache, in one pass over the projected row.
+//
+// Reference: src/lfm25_gpu.cu:420-485 (norm over the head with a shared [hd] weight,
+// then half-split rotation with theta_j = base^(-2j/hd), K cached after both) and
+// :487-501 (V cached as projected).  Here theta_j comes in as a float32 table and the
+// angle pos * theta_j, its cosine and sine are float32.
+//
+// Cache layout: [page][kv_head][offset][hd]; slot = page * page_size + offset.
+#include "common.h"
+
+namespace {
+constexpr int MAX_PER_LANE = 4;            // head sizes up to 256
+
+template <typename T, typename TW>
+__global__ __launch_bounds__(WAVE) void qkv_post_kernel(
+    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_out,
+    T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const TW* __restrict__ q_norm_w, const TW* __restrict__ k_norm_w, float eps,
+    const float* __restrict__ inv_freq, int rotary_dim, int interleaved,
+    const int* __restrict__ positions, const int* __restrict__ slot_mapping,
+    int H, int Hkv, int hd, int page_size) {
+    __shared__ float vals[MAX_PER_LANE * WAVE];
+    const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const int row_width = (H + 2 * Hkv) * hd;
+    const T* src = qkv + (long long)t * row_width + (long long)head * hd;
+    const bool is_q = head < H, is_k = !is_q && head < H + Hkv;
+    const int kvh = is_q ? 0 : (is_k ? head - H : head - H - Hkv);
+
+    float v[MAX_PER_LANE];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAX_PER_LANE; ++i) {
+        const int j = lane + i * WAVE;
+        v[i] = (j < hd) ? to_f32(src[j]) : 0.f;
+        ss += v[i] * v[i];
+    }
+    const TW* nw = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
+    if (nw) {
+        const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)hd + eps);
+#pragma unroll
+        for (int i = 0; i < MAX_PER_LANE; ++i) {
+            const int j = lane + i * WAVE;
+            if (j < hd) v[i] = v[i] * inv * to_f32(nw[j]);
+        }
+    }
+    const bool rotate = inv_freq != nullptr && (is_q || is_k);
+    if (rotate) {
+#pragma unroll
+        for (int i = 0; i < MAX_PER_LANE; ++i) vals[lane + i * WAVE] = v[i];
+        __syncthreads();
+        const float pos = (float)positions[t];
+        const int half = rotary_dim / 2;
+#pragma unroll
+        for (int i = 0; i < MAX_PER_LANE; ++i) {
+            const int j = lane + i * WAVE;
+            if (j >= rotary_dim || j >= hd) continue;
+            int f, partner; bool first;
+            if (interleaved) { f = j / 2; first = (j % 2) == 0; partner = first ? j + 1 : j - 1; }
+            else { first = j < half; f = first ? j : j - half; partner = first ? j + half : j - half; }
+            const float a = pos * inv_freq[f];
+            const float c = cosf(a), s = sinf(a);
+            const float x0 = first ? vals[j] : vals[partner];
+            const float x1 = first ? vals[partner] : vals[j];
+            v[i] = first ? (x0 * c - x1 * s) : (x0 * s + x1 * c);
+        }
+    }
+    T* dst = nullptr;
+    T* dst2 = nullptr;
+    if (is_q) dst = q_out + ((long long)t * H + head) * hd;
+    else {
+        if (is_k && k_out) dst2 = k_out + ((long long)t * Hkv + kvh) * hd;
+        if (k_cache) {
+            const long long slot = slot_mapping[t];
+            if (slot >= 0) {
+                const long long page = slot / page_size, off = slot % page_size;
+                dst = (is_k ? k_cache : v_cache) + ((page * Hkv + kvh) * page_size + off) * hd;
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < MAX_PER_LANE; ++i) {
+        const int j = lane + i * WAVE;
+        if (j < hd) {
+            const T o = from_f32<T>(v[i]);
+            if (dst) dst[j] = o;
+            if (dst2) dst2[j] = o;
+        }
+    }
+}
+
+// Copies already encoded k and v rows [T, Hkv, hd] into the paged cache.
+template <typename T>
+__global__ __launch_bounds__(WAVE) void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v,
+                                                        T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                                        const int* __restrict__ slot_mapping, int Hkv, int hd, int page_size) {
+    const int t = blockIdx.x, kvh = blockIdx.y;
+    const long long slot = slot_mapping[t];
+    if (slot < 0) return;
+    const long long page = slot / page_size, off = slot % page_size;
+    const long long dst = ((page * Hkv + kvh) * page_size + off) * hd;
+    const long long src = ((long long)t * Hkv + kvh) * hd;
+    for (int j = threadIdx.x; j < hd; j += WAVE) { k_cache[dst + j] = k[src + j]; v_cache[dst + j] = v[src + j]; }
+}
+}  // namespace
+
+// dt: element type of qkv, q_out, k_out and the caches.  norm_dt: element type of the
+// norm weights.  Null q_norm_w / k_norm_w: no norm.  Null inv_freq: no rotation.
+// Null k_cache: nothing is written to the cache (then only the H query heads and, if
+// k_out is given, the key heads are processed).
+TUFF_EXPORT int tuff_qkv_post(const void* qkv, void* q_out, void* k_out, void* k_cache, void* v_cache, int dt,
+                              const void* q_norm_w, const void* k_norm_w, int norm_dt, float eps,
+                              const float* inv_freq, int rotary_dim, int interleaved,
+                              const int* positions, const int* slot_mapping,
+                              int n_tokens, int H, int Hkv, int hd, int page_size, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (hd > MAX_PER_LANE * WAVE || rotary_dim > hd || (rotary_dim % 2) != 0) return -2;
+    const int heads = k_cache ? H + 2 * Hkv : (k_out ? H + Hkv : H);
+    dim3 grid(n_tokens, heads), block(WAVE);
+#define LAUNCH(T, TW) hipLaunchKernelGGL((qkv_post_kernel<T, TW>), grid, block, 0, stream, (const T*)qkv, (T*)q_out, (T*)k_out, \
+        (T*)k_cache, (T*)v_cache, (const TW*)q_norm_w, (const TW*)k_norm_w, eps, inv_freq, rotary_dim, interleaved, \
+        positions, slot_mapping, H, Hkv, hd, page_size)
+    if (dt == DT_F32 && norm_dt == DT_F32) LAUNCH(float, float);
+    else if (dt == DT_F32) LAUNCH(float, bf16_t);
+    else if (norm_dt == DT_F32) LAUNCH(bf16_t, float);
+    else LAUNCH(bf16_t, bf16_t);
+#undef LAUNCH
+    return launch_status();
+}
+
+TUFF_EXPORT int tuff_kv_write(const void* k, const void* v, void* k_cache, void* v_cache, int dt,
+                              const int* slot_mapping, int n_tokens, int Hkv, int hd, int page_size,
+                              hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    dim3 grid(n_tokens, Hkv), block(WAVE);
+    if (dt == DT_F32) hipLaunchKernelGGL(kv_write_kernel<float>, grid, block, 0, stream, (const float*)k, (const float*)v, (float*)k_cache, (float*)v_cache, slot_mapping, Hkv, hd, page_size);
+    else hipLaunchKernelGGL(kv_write_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)k, (const bf16_t*)v, (bf16_t*)k_cache, (bf16_t*)v_cache, slot_mapping, Hkv, hd, page_size);
+    return launch_status();
+}

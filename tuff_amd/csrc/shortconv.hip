@@ -1,0 +1,99 @@
+// Gated short convolution of a mixed batch, with per-request state.
+//
+//   bcx = in_proj(h): B = bcx[0:d], C = bcx[d:2d], X = bcx[2d:3d];  u = B * X
+//   y_t = sum_{k=0}^{K-1} w[c, k] * u_{t-(K-1)+k}      (tap K-1 is the current token)
+//   out = C * y;   state <- the last K-1 rows of u
+// (src/lfm25_gpu.cu:378-397 for one token, :1056-1079 over a chunk;
+//  tools/lfm25_fp64_ref.py:118-126.)
+//
+// The convolution is a finite filter, not a recurrence: a token needs only the K-1
+// values of u before it.  Those come from earlier tokens of the same portion when they
+// are in this step, and from the request's state slot otherwise, so all tokens of a
+// step run in parallel and the sum  fma(u_2, w_2, fma(u_1, w_1, u_0 * w_0))  is the
+// same chain of operations wherever the portion was cut.  The state holds u in float32
+// (a product of two bfloat16 values is exact in float32).
+//
+// The forward kernel only reads the state; a second kernel, launched after it on the
+// same stream, rewrites each (slot, channel) column from registers.
+#include "common.h"
+
+namespace {
+constexpr int MAX_TAPS = 16;
+
+template <typename T, typename TW>
+__global__ void shortconv_fwd_kernel(const T* __restrict__ bcx, const TW* __restrict__ conv_w,
+                                     const float* __restrict__ state, T* __restrict__ out,
+                                     const int* __restrict__ req_of_token, const int* __restrict__ q_start,
+                                     const int* __restrict__ state_slot, int d, int K) {
+    const int t = blockIdx.x;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= d) return;
+    const int r = req_of_token[t];
+    const int t0 = q_start[r];
+    const int i = t - t0;
+    const float* st = state + (long long)state_slot[r] * (K - 1) * d;
+    float y = 0.f;
+    for (int k = 0; k < K; ++k) {
+        const int src = i - (K - 1) + k;
+        float u;
+        if (src >= 0) {
+            const T* row = bcx + (long long)(t0 + src) * 3 * d;
+            u = to_f32(row[c]) * to_f32(row[2 * d + c]);
+        } else {
+            u = st[(long long)(K - 1 + src) * d + c];
+        }
+        const float w = to_f32(conv_w[(long long)c * K + k]);
+        y = (k == 0) ? u * w : fmaf(u, w, y);
+    }
+    const float cg = to_f32(bcx[(long long)t * 3 * d + d + c]);
+    out[(long long)t * d + c] = from_f32<T>(cg * y);
+}
+
+template <typename T>
+__global__ void shortconv_state_kernel(const T* __restrict__ bcx, float* __restrict__ state,
+                                       const int* __restrict__ q_start, const int* __restrict__ q_len,
+                                       const int* __restrict__ state_slot, int d, int K) {
+    const int r = blockIdx.x;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= d) return;
+    const int t0 = q_start[r], n = q_len[r];
+    float* st = state + (long long)state_slot[r] * (K - 1) * d;
+    float tmp[MAX_TAPS];
+    for (int j = 0; j < K - 1; ++j) {
+        const int src = n - (K - 1) + j;
+        if (src >= 0) {
+            const T* row = bcx + (long long)(t0 + src) * 3 * d;
+            tmp[j] = to_f32(row[c]) * to_f32(row[2 * d + c]);
+        } else {
+            tmp[j] = st[(long long)(K - 1 + src) * d + c];
+        }
+    }
+    for (int j = 0; j < K - 1; ++j) st[(long long)j * d + c] = tmp[j];
+}
+}  // namespace
+
+TUFF_EXPORT int tuff_shortconv_fwd(const void* bcx, const void* conv_w, int w_dt, const float* state, void* out, int dt,
+                                   const int* req_of_token, const int* q_start, const int* state_slot,
+                                   int n_tokens, int d, int K, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (K < 2 || K - 1 > MAX_TAPS) return -2;
+    dim3 block(256), grid(n_tokens, ceil_div(d, 256));
+#define LAUNCH(T, TW) hipLaunchKernelGGL((shortconv_fwd_kernel<T, TW>), grid, block, 0, stream, (const T*)bcx, (const TW*)conv_w, \
+        state, (T*)out, req_of_token, q_start, state_slot, d, K)
+    if (dt == DT_F32 && w_dt == DT_F32) LAUNCH(float, float);
+    else if (dt == DT_F32) LAUNCH(float, bf16_t);
+    else if (w_dt == DT_F32) LAUNCH(bf16_t, float);
+    else LAUNCH(bf16_t, bf16_t);
+#undef LAUNCH
+    return launch_status();
+}
+
+TUFF_EXPORT int tuff_shortconv_state(const void* bcx, int dt, float* state, const int* q_start, const int* q_len,
+                                     const int* state_slot, int n_requests, int d, int K, hipStream_t stream) {
+    if (n_requests <= 0) return 0;
+    if (K < 2 || K - 1 > MAX_TAPS) return -2;
+    dim3 block(256), grid(n_requests, ceil_div(d, 256));
+    if (dt == DT_F32) hipLaunchKernelGGL(shortconv_state_kernel<float>, grid, block, 0, stream, (const float*)bcx, state, q_start, q_len, state_slot, d, K);
+    else hipLaunchKernelGGL(shortconv_state_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)bcx, state, q_start, q_len, state_slot, d, K);
+    return launch_status();
+}

@@ -1,0 +1,137 @@
+"""The engine: a bound model, its cache, and the one step function.
+
+`step(entries)` takes, for each request in the step, its next tokens (a portion of a prompt of
+any length, or one decoded token) and the places whose logits are wanted.  It runs exactly
+those tokens as one batch against the cache that earlier steps left and returns the float32
+logits of the wanted places.  The reference's counterparts take one token or up to eight
+consecutive tokens of its single request (src/lfm25_engine.c:434-475, :496-599).
+"""
+from __future__ import annotations
+
+import math
+from typing import Hashable, Optional, Sequence
+
+import torch
+
+from ..cache.manager import CacheLayout, CacheManager, OutOfPages
+from ..cache.storage import CacheStorage
+from ..config.base import ModelConfig
+from ..csrc import ops
+from ..models.registry import build_model, load_config
+from ..parts.base import Runtime
+from ..weights.loader import load_weights
+from ..weights.random_init import random_weights
+from .batch import StepContext, StepEntry, build_context
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
+           "fp32": torch.float32, "f32": torch.float32}
+
+
+def parse_dtype(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"the engine computes in bfloat16 or float32, not {name}")
+        return name
+    if name not in _DTYPES:
+        raise ValueError(f"unknown dtype '{name}'; choose bfloat16 or float32")
+    return _DTYPES[name]
+
+
+def require_gpu(device="cuda:0") -> torch.device:
+    if not torch.cuda.is_available():
+        raise RuntimeError("no GPU is visible: this engine runs its model on a gfx950 GPU through its "
+                           "own HIP kernels and has no CPU path")
+    return torch.device(device)
+
+
+class Engine:
+    def __init__(self, model, weights: dict, *, dtype, device="cuda:0", page_size: int = 16,
+                 max_tokens: int = 8192, max_requests: int = 8, num_pages=None, poison_cache: bool = False):
+        """max_tokens: tokens the page pool of each cache group holds (rounded up to whole
+        pages).  max_requests: state slots, i.e. requests that can be live at a time."""
+        self.device = require_gpu(device)
+        self.dtype = parse_dtype(dtype)
+        self.model = model
+        self.rt = Runtime(self.device, self.dtype)
+        for m in model.kernel_modules() + (["gemm_f32"] if self.dtype == torch.float32 else ["gemm_bf16"]):
+            ops.load(m)                      # compile or load now, not in the middle of a step
+        model.bind(weights, self.rt)
+        self.layout = CacheLayout.from_specs(model.cache_specs)
+        self.page_size = int(page_size)
+        if num_pages is None:
+            num_pages = -(-int(max_tokens) // self.page_size)
+        self.manager = CacheManager(self.layout, self.page_size, num_pages, int(max_requests))
+        self.storage = CacheStorage(self.manager, self.dtype, self.device, poison=poison_cache)
+        self.steps = 0
+
+    # ---------------------------------------------------------------- construction
+    @classmethod
+    def from_folder(cls, model_dir: str, *, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
+        dev = require_gpu(device)
+        cfg = load_config(model_dir)
+        model = build_model(cfg)
+        weights = load_weights(model_dir, model.weight_decls(), parse_dtype(dtype), dev)
+        eng = cls(model, weights, dtype=dtype, device=device, **kw)
+        eng.config = cfg
+        return eng
+
+    @classmethod
+    def from_config(cls, cfg: ModelConfig, seed: int, *, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
+        """Random weights made on the device (no folder is written)."""
+        dev = require_gpu(device)
+        model = build_model(cfg)
+        weights = random_weights(model.weight_decls(), seed, parse_dtype(dtype), dev)
+        eng = cls(model, weights, dtype=dtype, device=device, **kw)
+        eng.config = cfg
+        return eng
+
+    # -------------------------------------------------------------------- requests
+    def begin(self, req_id: Hashable) -> None:
+        slot = self.manager.admit(req_id)
+        self.storage.zero_slot(slot)
+
+    def end(self, req_id: Hashable) -> None:
+        self.manager.release(req_id)
+
+    def is_live(self, req_id) -> bool:
+        return req_id in self.manager
+
+    def length(self, req_id) -> int:
+        return self.manager.length(req_id)
+
+    # ------------------------------------------------------------------------ step
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Runs one batch.  Returns float32 logits [wanted, vocab] on the device, in the order
+        of the entries and of their `want` lists, or None if nothing is wanted.
+        Raises OutOfPages (and leaves every request as it was) if the pool is too small."""
+        entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        entries = [e for e in entries if len(e.tokens) > 0]
+        if not entries:
+            return None
+        ids = [e.req_id for e in entries]
+        if len(set(ids)) != len(ids):
+            raise ValueError("a request appears twice in one step")
+        limit = self.model.max_positions
+        V = self.model.vocab_size
+        for e in entries:                     # refuse bad input before anything is changed
+            if e.req_id not in self.manager:
+                raise ValueError(f"request {e.req_id!r} is not live: call begin() first")
+            if min(e.tokens) < 0 or max(e.tokens) >= V:
+                raise ValueError(f"request {e.req_id!r}: token id outside [0, {V})")
+            if any((not 0 <= w < len(e.tokens)) for w in e.want):
+                raise ValueError(f"request {e.req_id!r}: a wanted place is outside its {len(e.tokens)} tokens")
+        done = []
+        try:
+            for e in entries:
+                if limit is not None and self.manager.length(e.req_id) + len(e.tokens) > limit:
+                    raise ValueError(f"request {e.req_id!r} would pass the model's {limit} positions")
+                self.manager.extend(e.req_id, len(e.tokens))
+                done.append(e)
+        except Exception:
+            for e in done:
+                self.manager.truncate(e.req_id, self.manager.length(e.req_id) - len(e.tokens))
+            raise
+        ctx = build_context(entries, self.manager, self.device, self.model.vocab_size)
+        logits = self.model.forward(ctx, self.storage.views)
+        self.steps += 1
+        return logits

@@ -1,0 +1,129 @@
+"""A decoder as data: an embedding, a set of blocks, the order in which they run, a final norm
+and a head.  The run order is a list of LayerRun; it may name a block twice (each run then has
+a cache of its own) or let a run read the cache that another run writes.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Optional
+
+import torch
+
+from ..csrc import ops
+from ..parts.base import Block, FixedState, Norm, PagedKV, Runtime, WeightDecl
+
+
+@dataclasses.dataclass(frozen=True)
+class LayerRun:
+    block: int                      # index into DecoderModel.blocks
+    cache: Optional[int] = None     # cache entry this run uses (default: one of its own)
+    writes: bool = True             # False: only reads the entry, which an earlier run writes
+
+
+class DecoderModel:
+    def __init__(self, *, vocab_size: int, hidden_size: int, embedding: WeightDecl,
+                 blocks: list[Block], final_norm: Norm, head: Optional[WeightDecl] = None,
+                 schedule: Optional[list[LayerRun]] = None, max_positions: Optional[int] = None,
+                 eos_token_id: Optional[int] = None):
+        """head=None: the head is the embedding (tied), as the reference does when the file has
+        no output matrix (src/lfm25_model.c:128-131)."""
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.embedding_decl, self.head_decl = embedding, head
+        self.blocks, self.final_norm = list(blocks), final_norm
+        self.max_positions, self.eos_token_id = max_positions, eos_token_id
+        runs = schedule if schedule is not None else [LayerRun(i) for i in range(len(self.blocks))]
+        self.schedule: list[LayerRun] = []
+        next_id = 0
+        used = {r.cache for r in runs if r.cache is not None}
+        for r in runs:
+            if not 0 <= r.block < len(self.blocks):
+                raise ValueError(f"run order names block {r.block}; there are {len(self.blocks)}")
+            cache = r.cache
+            if cache is None:
+                while next_id in used:
+                    next_id += 1
+                cache = next_id
+                used.add(cache)
+            self.schedule.append(LayerRun(r.block, cache, r.writes))
+        # every cache entry has exactly one writer, which comes before its readers
+        self.cache_specs: dict[int, object] = {}
+        for r in self.schedule:
+            spec = self.blocks[r.block].mixer.cache_spec()
+            if r.writes:
+                if r.cache in self.cache_specs:
+                    raise ValueError(f"cache entry {r.cache} has two writers")
+                self.cache_specs[r.cache] = spec
+            else:
+                if r.cache not in self.cache_specs:
+                    raise ValueError(f"a run reads cache entry {r.cache} before any run writes it")
+                if self.cache_specs[r.cache] != spec:
+                    raise ValueError(f"a run reads cache entry {r.cache} of another shape: "
+                                     f"{self.cache_specs[r.cache]} vs {spec}")
+                if isinstance(spec, FixedState):
+                    raise ValueError("a fixed-size state cannot be shared between runs")
+        self.embedding: Optional[torch.Tensor] = None
+        self.head: Optional[torch.Tensor] = None
+
+    # ------------------------------------------------------------------ description
+    def weight_decls(self) -> list[WeightDecl]:
+        decls = [self.embedding_decl]
+        for b in self.blocks:
+            decls += b.weight_decls()
+        decls += self.final_norm.weight_decls()
+        if self.head_decl is not None:
+            decls.append(self.head_decl)
+        seen, out = set(), []
+        for d in decls:
+            if d.name in seen:
+                raise ValueError(f"two parts declare the tensor '{d.name}'")
+            seen.add(d.name)
+            out.append(d)
+        return out
+
+    def kernel_modules(self) -> list[str]:
+        mods = ["elementwise"]
+        for b in self.blocks:
+            mods += b.kernel_modules()
+        mods += self.final_norm.kernel_modules()
+        return sorted(set(mods))
+
+    def num_parameters(self) -> int:
+        n = 0
+        for d in self.weight_decls():
+            k = 1
+            for s in d.shape:
+                k *= s
+            n += k
+        return n
+
+    # ------------------------------------------------------------------------ bind
+    def bind(self, weights: dict[str, torch.Tensor], rt: Runtime) -> None:
+        self.rt = rt
+        self.embedding = weights[self.embedding_decl.name]
+        self.head = weights[self.head_decl.name] if self.head_decl is not None else self.embedding
+        for b in self.blocks:
+            b.bind(weights, rt)
+        self.final_norm.bind(weights, rt)
+        self._head_cast: Optional[torch.Tensor] = None
+        if self.head.dtype != rt.dtype and self.head.dtype != torch.float32:
+            raise TypeError(f"head weight of type {self.head.dtype} in a {rt.dtype} run")
+
+    # --------------------------------------------------------------------- forward
+    def forward(self, ctx, cache_views: dict[int, object]) -> Optional[torch.Tensor]:
+        """Runs the step's tokens through all layers.  Returns float32 logits
+        [len(ctx.logit_rows), vocab], or None when no logits are wanted."""
+        rt = self.rt
+        x = torch.empty(ctx.T, self.hidden_size, dtype=torch.float32, device=rt.device)
+        ops.embed_rows(self.embedding, ctx.tokens, x)
+        for run in self.schedule:
+            self.blocks[run.block].forward(x, ctx, cache_views.get(run.cache), run.writes)
+        if ctx.n_logits == 0:
+            return None
+        h = self.final_norm.forward(x, rows=ctx.logit_rows)
+        logits = torch.empty(ctx.n_logits, self.vocab_size, dtype=torch.float32, device=rt.device)
+        if h.dtype != self.head.dtype:
+            h32 = torch.empty(h.shape, dtype=torch.float32, device=rt.device)
+            ops.cast(h, h32)
+            h = h32
+        ops.gemm(h, self.head, logits)
+        return logits

@@ -1,0 +1,108 @@
+"""Grouped-query attention mixer over the paged cache.
+
+q = W_q h, k = W_k h, v = W_v h; optional per-head RMSNorm of q and k with a shared [hd]
+weight; optional position encoding; k (normed, encoded) and v (as projected) go to the cache
+at the token's slot; every token attends to the cached keys of its request up to its own
+position (within `window` if given); query head i reads kv head i // (H / Hkv); scores are
+scaled by 1/sqrt(hd); o = W_o concat(heads).
+Reference: src/lfm25_engine.c:386-405, src/lfm25_gpu.cu:420-485, :506-558.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from ..csrc import ops
+from .base import MIXERS, Mixer, PagedKV, PositionEncoding, Runtime, WeightDecl
+from .linear import Linear
+
+
+@MIXERS.register("attention")
+class AttentionMixer(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, *,
+                 names: dict[str, str], qk_norm_eps: Optional[float] = None,
+                 position: Optional[PositionEncoding] = None, window: Optional[int] = None,
+                 scale: Optional[float] = None, aliases: Optional[dict[str, tuple]] = None):
+        """names: checkpoint names of 'q', 'k', 'v', 'o' and, with qk_norm_eps, 'q_norm', 'k_norm'."""
+        if num_heads % num_kv_heads:
+            raise ValueError(f"heads {num_heads} must be a multiple of kv heads {num_kv_heads}")
+        if head_dim > 256:
+            raise ValueError(f"head size {head_dim} above 256 is not supported by the attention kernels")
+        self.d, self.H, self.Hkv, self.hd = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
+        self.eps = None if qk_norm_eps is None else float(qk_norm_eps)
+        self.position, self.window = position, (int(window) if window else None)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.hd)
+        self.names = dict(names)
+        al = aliases or {}
+        self.qkv = Linear([names["q"], names["k"], names["v"]], self.d,
+                          [self.H * self.hd, self.Hkv * self.hd, self.Hkv * self.hd],
+                          aliases=[al.get("q", ()), al.get("k", ()), al.get("v", ())])
+        self.out = Linear(names["o"], self.H * self.hd, self.d, aliases=[al.get("o", ())])
+        self._al = al
+        self.q_norm_w = self.k_norm_w = None
+
+    def weight_decls(self):
+        decls = self.qkv.weight_decls() + self.out.weight_decls()
+        if self.eps is not None:
+            decls += [WeightDecl(self.names["q_norm"], (self.hd,), "norm", aliases=self._al.get("q_norm", ())),
+                      WeightDecl(self.names["k_norm"], (self.hd,), "norm", aliases=self._al.get("k_norm", ()))]
+        if self.position is not None:
+            decls += self.position.weight_decls()
+        return decls
+
+    def kernel_modules(self):
+        mods = ["rope_kv", "attention"]
+        if self.position is not None:
+            mods += self.position.kernel_modules()
+        return mods
+
+    def cache_spec(self):
+        return PagedKV(self.Hkv, self.hd, self.window)
+
+    def bind(self, weights, rt: Runtime):
+        self.rt = rt
+        self.qkv.bind(weights, rt)
+        self.out.bind(weights, rt)
+        if self.eps is not None:
+            self.q_norm_w = weights[self.names["q_norm"]]
+            self.k_norm_w = weights[self.names["k_norm"]]
+            if self.q_norm_w.dtype != self.k_norm_w.dtype:
+                self.q_norm_w = self.q_norm_w.float()
+                self.k_norm_w = self.k_norm_w.float()
+        if self.position is not None:
+            self.position.bind(weights, rt)
+
+    def forward(self, h, ctx, cache, residual, write_cache: bool = True) -> None:
+        T = h.shape[0]
+        H, Hkv, hd = self.H, self.Hkv, self.hd
+        g = ctx.groups[cache.group]
+        qkv = self.qkv.forward(h)
+        q = self.rt.empty(T, H * hd)
+        norm = dict(eps=self.eps or 0.0, q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w)
+        tables = self.position.rotary_tables() if self.position is not None else None
+        if self.position is None or tables is not None:
+            rot = {}
+            if tables is not None:
+                rot = dict(inv_freq=tables[0], rotary_dim=tables[1], interleaved=tables[2])
+            wr = dict(k_cache=cache.k, v_cache=cache.v, slot_mapping=g.slot_mapping) if write_cache else {}
+            ops.qkv_post(qkv, q, H=H, Hkv=Hkv, hd=hd, positions=ctx.positions, page_size=cache.page_size,
+                         **norm, **rot, **wr)
+        else:
+            # a position encoding of its own: norm, then its apply(), then the cache write
+            k = self.rt.empty(T, Hkv * hd)
+            ops.qkv_post(qkv, q, H=H, Hkv=Hkv, hd=hd, positions=ctx.positions, k_out=k, **norm)
+            self.position.apply(q, k, ctx.positions)
+            if write_cache:
+                v = qkv[:, (H + Hkv) * hd:].contiguous()
+                ops.kv_write(k, v, cache.k, cache.v, g.slot_mapping, Hkv=Hkv, hd=hd, page_size=cache.page_size)
+        o = self.rt.empty(T, H * hd)
+        self.attend(q, o, ctx, cache, g)
+        self.out.forward(o, accumulate_into=residual)
+
+    def attend(self, q, o, ctx, cache, g) -> None:
+        ops.attention_general(q, cache.k, cache.v, o, block_table=g.block_table,
+                              req_of_token=ctx.req_of_token, positions=ctx.positions,
+                              H=self.H, Hkv=self.Hkv, hd=self.hd, page_size=cache.page_size,
+                              window=self.window or 0, scale=self.scale)

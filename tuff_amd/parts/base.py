@@ -1,0 +1,153 @@
+"""What a part is: the interfaces of mixers, feed-forwards, norms, position encodings and
+blocks, the declaration of their weights and caches, and the registries that name them.
+
+A part is built in two phases.  Its constructor takes sizes and constants only and allocates
+nothing, so a whole model can be described, its weights listed and its caches sized without a
+GPU.  `bind(weights, runtime)` then attaches device tensors and the compute dtype.  No part
+knows which model it is in: names of checkpoint tensors come in through `names`.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Callable, Optional
+
+import torch
+
+
+# ---------------------------------------------------------------------- declarations
+@dataclasses.dataclass(frozen=True)
+class WeightDecl:
+    """One tensor a part needs from the checkpoint."""
+    name: str                       # name in the checkpoint
+    shape: tuple
+    init: str = "normal"            # random-weights mode: "normal" N(0, 0.02) | "norm" 1 + N(0, 0.01)
+    alt_shapes: tuple = ()          # shapes that are accepted and reshaped to `shape`
+    aliases: tuple = ()             # other names the same tensor may have
+
+
+@dataclasses.dataclass(frozen=True)
+class PagedKV:
+    """Keys and values that grow by one entry a token, kept in pages.  `window`: only the
+    last `window` positions are ever read (None: all)."""
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclasses.dataclass(frozen=True)
+class FixedState:
+    """Per-request state of fixed size, float32, zero for a new request."""
+    shape: tuple
+
+
+@dataclasses.dataclass
+class Runtime:
+    """What parts need at bind time: where tensors live and in which type they compute."""
+    device: torch.device
+    dtype: torch.dtype              # torch.bfloat16 (serving) or torch.float32 (true 32-bit)
+
+    def empty(self, *shape, dtype=None) -> torch.Tensor:
+        return torch.empty(*shape, dtype=dtype or self.dtype, device=self.device)
+
+
+# -------------------------------------------------------------------------- interfaces
+class Part:
+    """Base of all parts.  `names` maps the part's own weight names to checkpoint names."""
+
+    def weight_decls(self) -> list[WeightDecl]:
+        return []
+
+    def bind(self, weights: dict[str, torch.Tensor], rt: Runtime) -> None:
+        self.rt = rt
+
+    def kernel_modules(self) -> list[str]:
+        """Kernel libraries (names of tuff_amd.csrc.build.MODULES) this part launches."""
+        return []
+
+
+class Norm(Part):
+    """forward(x float32 [T, d], rows=None) -> [T or len(rows), d] in the compute dtype."""
+
+    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Encodes positions into q and k of an attention mixer, after their norm and before the
+    cache write (the cache holds encoded keys).
+
+    Either `rotary_tables()` returns (inv_freq float32 [rotary_dim/2], rotary_dim, interleaved)
+    and the mixer applies it inside its fused kernel, or it returns None and the mixer calls
+    `apply(q [T, H*hd], k [T, Hkv*hd], positions int32 [T])`, which rewrites both in place.
+    """
+
+    def rotary_tables(self):
+        return None
+
+    def apply(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """Token mixer.  forward adds its output to `residual` (float32 [T, d]).
+
+    h: [T, d] in the compute dtype, already normed.  ctx: the step's StepContext.
+    cache: the view of this run's cache entry (PagedKVView, StateView or None).
+    write_cache=False: read the cache of another run without writing to it.
+    """
+
+    def cache_spec(self):
+        return None
+
+    def forward(self, h, ctx, cache, residual, write_cache: bool = True) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """forward(h [T, d] compute dtype, ctx, residual float32 [T, d]) adds its output."""
+
+    def forward(self, h, ctx, residual) -> None:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arrangement of norms, a mixer and a feed-forward around the residual stream.
+    forward(x float32 [T, d], ctx, cache, write_cache) updates x in place."""
+
+    mixer: Mixer
+
+    def forward(self, x, ctx, cache, write_cache: bool = True) -> None:
+        raise NotImplementedError
+
+
+# --------------------------------------------------------------------------- registries
+class Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self._items: dict[str, Callable] = {}
+
+    def register(self, name: str, item=None):
+        def put(obj):
+            if name in self._items and self._items[name] is not obj:
+                raise ValueError(f"{self.what} '{name}' is already registered")
+            self._items[name] = obj
+            return obj
+        return put if item is None else put(item)
+
+    def get(self, name: str):
+        if name not in self._items:
+            raise KeyError(f"unknown {self.what} '{name}'; registered: {sorted(self._items)}")
+        return self._items[name]
+
+    def names(self) -> list[str]:
+        return sorted(self._items)
+
+    def unregister(self, name: str) -> None:
+        self._items.pop(name, None)
+
+
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+NORMS = Registry("norm")
+POSITION_ENCODINGS = Registry("position encoding")
+BLOCKS = Registry("block arrangement")

@@ -1,0 +1,37 @@
+"""SwiGLU feed-forward: W_down (silu(W_gate h) * (W_up h)), silu(g) = g / (1 + exp(-g)).
+Reference: src/lfm25_gpu.cu:583-618, src/lfm25_engine.c:412-419.  Gate and up are one product.
+"""
+from __future__ import annotations
+
+from ..csrc import ops
+from .base import FEED_FORWARDS, FeedForward, Runtime
+from .linear import Linear
+
+
+@FEED_FORWARDS.register("swiglu")
+class SwiGLU(FeedForward):
+    def __init__(self, hidden_size: int, ffn_dim: int, *, names: dict[str, str],
+                 aliases: dict[str, tuple] | None = None):
+        """names: checkpoint names of 'gate' [F, d], 'up' [F, d], 'down' [d, F]."""
+        self.d, self.F = int(hidden_size), int(ffn_dim)
+        al = aliases or {}
+        self.gate_up = Linear([names["gate"], names["up"]], self.d, [self.F, self.F],
+                              aliases=[al.get("gate", ()), al.get("up", ())])
+        self.down = Linear(names["down"], self.F, self.d, aliases=[al.get("down", ())])
+
+    def weight_decls(self):
+        return self.gate_up.weight_decls() + self.down.weight_decls()
+
+    def kernel_modules(self):
+        return ["elementwise"]
+
+    def bind(self, weights, rt: Runtime):
+        self.rt = rt
+        self.gate_up.bind(weights, rt)
+        self.down.bind(weights, rt)
+
+    def forward(self, h, ctx, residual) -> None:
+        gu = self.gate_up.forward(h)
+        act = self.rt.empty(h.shape[0], self.F, dtype=gu.dtype)
+        ops.swiglu(gu, act)
+        self.down.forward(act, accumulate_into=residual)

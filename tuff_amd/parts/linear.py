@@ -1,0 +1,69 @@
+"""Projection y = x W^T with W [out, in] row-major, as every projection of the reference
+(`dst[row] = W[row, :] . x`, src/lfm25_gpu.cu:148-202).  Several checkpoint tensors with the
+same input can be stacked into one weight, so q/k/v or gate/up are one product.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence
+
+import torch
+
+from ..csrc import ops
+from .base import Runtime, WeightDecl
+
+
+class Linear:
+    def __init__(self, names: Sequence[str] | str, in_features: int,
+                 out_features: Sequence[int] | int, aliases: Sequence[Sequence[str]] | None = None):
+        self.names = [names] if isinstance(names, str) else list(names)
+        outs = [out_features] if isinstance(out_features, int) else list(out_features)
+        if len(outs) != len(self.names):
+            raise ValueError("one output size per stacked tensor")
+        self.in_features, self.outs = int(in_features), [int(o) for o in outs]
+        self.out_features = sum(self.outs)
+        self.aliases = [tuple(a) for a in aliases] if aliases else [()] * len(self.names)
+        self.weight: Optional[torch.Tensor] = None
+
+    def weight_decls(self) -> list[WeightDecl]:
+        return [WeightDecl(n, (o, self.in_features), "normal", aliases=a)
+                for n, o, a in zip(self.names, self.outs, self.aliases)]
+
+    def bind(self, weights: dict[str, torch.Tensor], rt: Runtime) -> None:
+        self.rt = rt
+        ws = [weights[n] for n in self.names]
+        if len(ws) == 1:
+            self.weight = ws[0]
+        else:
+            if len({w.dtype for w in ws}) != 1:
+                ws = [w.to(torch.float32) for w in ws]
+            self.weight = torch.cat(ws, dim=0).contiguous()
+        if self.weight.dtype == torch.bfloat16 and self.in_features % 8 != 0:
+            raise ValueError(f"{self.names[0]}: the bfloat16 matrix kernels need an input size that is a "
+                             f"multiple of 8, got {self.in_features}")
+
+    def forward(self, x: torch.Tensor, *, out_dtype: Optional[torch.dtype] = None,
+                accumulate_into: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        """x [T, in] in the compute dtype.  Returns a new [T, out] tensor of `out_dtype`
+        (default: the compute dtype), or adds into `accumulate_into` (float32) and returns None."""
+        w = self.weight
+        T = x.shape[0]
+        if x.dtype != w.dtype:
+            # a weight stored in 32-bit stays so: run this product in float32
+            if w.dtype != torch.float32:
+                raise TypeError(f"{self.names[0]}: activation {x.dtype} with weight {w.dtype}")
+            x32 = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+            ops.cast(x, x32)
+            x = x32
+        if accumulate_into is not None:
+            ops.gemm(x, w, accumulate_into, accumulate=True)
+            return None
+        want = out_dtype or self.rt.dtype
+        if w.dtype == torch.float32 and want != torch.float32:
+            y32 = torch.empty(T, self.out_features, dtype=torch.float32, device=x.device)
+            ops.gemm(x, w, y32)
+            y = torch.empty(T, self.out_features, dtype=want, device=x.device)
+            ops.cast(y32, y)
+            return y
+        y = torch.empty(T, self.out_features, dtype=want, device=x.device)
+        ops.gemm(x, w, y)
+        return y
