@@ -1,0 +1,105 @@
+"""The Python entry point: from prompts (token ids) to generated token ids.
+
+    llm = LLM("model_dir", dtype="bfloat16")
+    outs = llm.generate([[1, 36309]], SamplingParams(max_new_tokens=16))
+
+`generate` is the reference's run loop (prefill in portions, then one token a step until -n
+tokens, src/main.c:1743-1858) for many requests at once: scheduler -> step -> sampler.
+"""
+from __future__ import annotations
+
+import dataclasses
+import itertools
+from typing import Optional, Sequence
+
+import torch
+
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler
+from .batch import StepEntry
+from .engine import Engine
+from .scheduler import Request, Scheduler
+
+
+@dataclasses.dataclass
+class Generation:
+    request_id: object
+    prompt: list
+    token_ids: list
+    finish_reason: str
+    preemptions: int = 0
+
+
+class LLM:
+    def __init__(self, model=None, *, engine: Optional[Engine] = None, dtype="bfloat16", device="cuda:0",
+                 max_num_seqs: int = 8, max_batched_tokens: int = 2048, ctx_size: Optional[int] = None,
+                 page_size: int = 16, num_pages: Optional[int] = None, ignore_eos: bool = False):
+        """model: a folder with config.json and model.safetensors.  ctx_size (-c): the longest
+        prompt + generation of one request.  num_pages: size of the page pool; default: room for
+        max_num_seqs requests of ctx_size."""
+        if engine is None:
+            if model is None:
+                raise ValueError("give a model folder or an engine")
+            from ..models.registry import load_config
+            cfg = load_config(model)
+            limit = getattr(cfg, "max_position_embeddings", None)
+            ctx = min(ctx_size or 4096, limit or (ctx_size or 4096))
+            pages = num_pages if num_pages is not None else max_num_seqs * -(-ctx // page_size)
+            engine = Engine.from_folder(model, dtype=dtype, device=device, page_size=page_size,
+                                        num_pages=pages, max_requests=max_num_seqs)
+            ctx_size = ctx
+        self.engine = engine
+        model_limit = engine.model.max_positions
+        self.ctx_size = min(c for c in (ctx_size, model_limit) if c is not None) if (ctx_size or model_limit) else None
+        self.max_num_seqs = min(max_num_seqs, engine.manager.num_slots)
+        self.max_batched_tokens = max_batched_tokens
+        self.ignore_eos = ignore_eos
+        self.sampler = Sampler(engine.device)
+        self._ids = itertools.count()
+        self.last_stats: dict = {}
+
+    def new_scheduler(self) -> Scheduler:
+        eos = None if self.ignore_eos else self.engine.model.eos_token_id
+        return Scheduler(self.engine.manager, begin=self.engine.begin, end=self.engine.end,
+                         max_num_seqs=self.max_num_seqs, max_batched_tokens=self.max_batched_tokens,
+                         max_model_len=self.ctx_size, eos_token_id=eos)
+
+    def run(self, sched: Scheduler, on_step=None) -> None:
+        """Steps until every request of the scheduler has finished."""
+        steps = tokens = 0
+        while sched.has_unfinished():
+            batch = sched.schedule()
+            if not batch:
+                if sched.has_unfinished():
+                    raise RuntimeError("the scheduler made no progress: no request fits the cache")
+                break
+            entries = [StepEntry(s.request.id, s.tokens, [len(s.tokens) - 1] if s.samples else [])
+                       for s in batch]
+            logits = self.engine.step(entries)
+            sampling = [s.request for s in batch if s.samples]
+            sampled = {}
+            if sampling:
+                toks = self.sampler.sample(logits, [r.sampler for r in sampling])
+                sampled = {r.id: t for r, t in zip(sampling, toks)}
+            sched.update(batch, sampled)
+            steps += 1
+            tokens += sum(len(s.tokens) for s in batch)
+            if on_step is not None:
+                on_step(batch, sampled)
+        self.last_stats = {"steps": steps, "tokens_run": tokens, "preemptions": sched.num_preemptions}
+
+    def generate(self, prompts: Sequence[Sequence[int]], params=None) -> list[Generation]:
+        """prompts: token id lists.  params: one SamplingParams for all, or one per prompt."""
+        if params is None:
+            params = SamplingParams()
+        plist = [params] * len(prompts) if isinstance(params, SamplingParams) else list(params)
+        if len(plist) != len(prompts):
+            raise ValueError("one SamplingParams per prompt, or one for all")
+        sched = self.new_scheduler()
+        reqs = []
+        for prompt, p in zip(prompts, plist):
+            r = Request(next(self._ids), [int(t) for t in prompt], dataclasses.replace(p))
+            reqs.append(r)
+            sched.add(r)
+        self.run(sched)
+        return [Generation(r.id, r.prompt, list(r.output), r.finish_reason or "", r.preemptions) for r in reqs]

@@ -1,0 +1,241 @@
+"""Continuous batching above the step function.
+
+Every call to `schedule()` decides one step: requests that are decoding get their one token
+first, then prompts are continued and new requests admitted, in arrival order, while the
+token budget, the state slots and the pages last; the last prompt portion is cut to fit the
+budget.  `update()` takes the sampled tokens, finishes requests and frees what they held.
+
+When pages run out: a waiting request is simply not admitted yet.  If a running request
+cannot get the pages for its next tokens, the most recently admitted running request is
+preempted: its pages and slot are given back, and it returns to the head of the waiting queue
+to be computed again from its first token, prompt and generated tokens together (a conv state
+cannot be rebuilt from the KV cache, so recomputation is the only exact way).  Its sampler state
+is kept, so its output does not change.  A request that does not fit the pool even alone is
+finished with reason "capacity".
+
+The reference runs one request and has no scheduler; the loop shape follows its other
+backend's slot loop (src/qwen35/q35_server.c:869-1050): FIFO admission, prompt portions beside
+one decode batch, slot freed at finish.
+"""
+from __future__ import annotations
+
+import collections
+import dataclasses
+from typing import Hashable, Optional
+
+from ..cache.manager import CacheManager
+from ..sampling.params import SamplerState, SamplingParams
+
+WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
+
+
+@dataclasses.dataclass
+class Request:
+    id: Hashable
+    prompt: list
+    params: SamplingParams
+    output: list = dataclasses.field(default_factory=list)
+    status: str = WAITING
+    num_computed: int = 0            # tokens of prompt+output whose cache entries exist
+    finish_reason: Optional[str] = None
+    preemptions: int = 0
+    sampler: Optional[SamplerState] = None
+
+    def tokens(self) -> list:
+        return self.prompt + self.output
+
+    def remaining(self) -> int:
+        return len(self.prompt) + len(self.output) - self.num_computed
+
+
+@dataclasses.dataclass
+class Scheduled:
+    request: Request
+    start: int                       # first position fed in this step
+    tokens: list
+    samples: bool                    # the step reaches the request's last token: draw the next
+
+
+class Scheduler:
+    def __init__(self, manager: CacheManager, *, begin, end, max_num_seqs: int = 8,
+                 max_batched_tokens: int = 2048, max_model_len: Optional[int] = None,
+                 eos_token_id: Optional[int] = None):
+        """begin(req_id) / end(req_id): take and give back a request's cache (Engine.begin/end)."""
+        self.manager, self._begin, self._end = manager, begin, end
+        self.max_num_seqs = int(max_num_seqs)
+        self.max_batched_tokens = int(max_batched_tokens)
+        self.max_model_len = max_model_len
+        self.eos_token_id = eos_token_id
+        if self.max_batched_tokens < 1 or self.max_num_seqs < 1:
+            raise ValueError("max_batched_tokens and max_num_seqs must be positive")
+        self.waiting: collections.deque[Request] = collections.deque()
+        self.running: list[Request] = []          # in admission order
+        self.finished: list[Request] = []
+        self.num_preemptions = 0
+
+    # ------------------------------------------------------------------- requests
+    def add(self, req: Request) -> None:
+        req.params.validate()
+        if not req.prompt:
+            raise ValueError(f"request {req.id!r}: empty prompt")
+        if req.sampler is None:
+            req.sampler = SamplerState(req.params)
+        if self.max_model_len is not None and len(req.prompt) + req.params.max_new_tokens > self.max_model_len:
+            # the reference checks the same up front (ctx_fits, src/main.c:687-692, :1264-1275)
+            self._finish(req, "rejected: prompt + max_new_tokens exceeds the context length")
+            return
+        if req.params.max_new_tokens == 0:
+            self._finish(req, "length")
+            return
+        self.waiting.append(req)
+
+    def adopt(self, req: Request, num_computed: int) -> None:
+        """Takes over a request that is already live in the cache with its first
+        `num_computed` tokens computed (begin() and the steps were done by the caller)."""
+        req.params.validate()
+        if self.manager.length(req.id) != num_computed or not 0 <= num_computed < len(req.prompt) + len(req.output):
+            raise ValueError(f"request {req.id!r}: the cache holds {self.manager.length(req.id)} tokens, "
+                             f"not the {num_computed} stated")
+        if req.sampler is None:
+            req.sampler = SamplerState(req.params)
+        req.status, req.num_computed = RUNNING, num_computed
+        self.running.append(req)
+
+    def has_unfinished(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    def abort(self, req_id) -> None:
+        for r in list(self.running):
+            if r.id == req_id:
+                self.running.remove(r)
+                self._end(r.id)
+                self._finish(r, "aborted")
+                return
+        for r in list(self.waiting):
+            if r.id == req_id:
+                self.waiting.remove(r)
+                self._finish(r, "aborted")
+                return
+
+    def _finish(self, req: Request, reason: str) -> None:
+        req.status, req.finish_reason = FINISHED, reason
+        self.finished.append(req)
+
+    # ------------------------------------------------------------------- one step
+    def _fits(self, req: Request, n: int, promised: list[int]) -> bool:
+        need = self.manager.pages_needed(req.id, n)
+        back = self.manager.reclaimable(req.id)
+        return all(nd <= g.pool.num_free + b - p
+                   for nd, b, p, g in zip(need, back, promised, self.manager.groups))
+
+    def _promise(self, req: Request, n: int, promised: list[int]) -> None:
+        need = self.manager.pages_needed(req.id, n)
+        back = self.manager.reclaimable(req.id)
+        for i, (nd, b) in enumerate(zip(need, back)):
+            promised[i] += nd - b
+
+    def _preempt(self, victim: Request) -> None:
+        self.running.remove(victim)
+        self._end(victim.id)
+        victim.status, victim.num_computed = WAITING, 0
+        victim.preemptions += 1
+        self.num_preemptions += 1
+        self.waiting.appendleft(victim)
+
+    def _total_pages(self) -> list[int]:
+        return [g.pool.num_pages for g in self.manager.groups]
+
+    def schedule(self) -> list[Scheduled]:
+        budget = self.max_batched_tokens
+        promised = [0] * len(self.manager.groups)
+        out: list[Scheduled] = []
+
+        # running requests, decoding ones first, then prompts in admission order
+        order = sorted(self.running, key=lambda r: (r.remaining() != 1, self.running.index(r)))
+        for req in order:
+            if req not in self.running or budget == 0:       # preempted meanwhile / nothing left
+                continue
+            n = min(req.remaining(), budget)
+            while not self._fits(req, n, promised):
+                victim = self.running[-1]
+                if victim is req and len(self.running) == 1:
+                    # alone and still too large: shrink the portion, or give up
+                    while n > 1 and not self._fits(req, n, promised):
+                        n -= 1
+                    if not self._fits(req, n, promised):
+                        self.running.remove(req)
+                        self._end(req.id)
+                        self._finish(req, "capacity")
+                        n = 0
+                    break
+                scheduled_victim = next((s for s in out if s.request is victim), None)
+                if scheduled_victim is not None:
+                    out.remove(scheduled_victim)
+                    budget += len(scheduled_victim.tokens)
+                    promised = [0] * len(self.manager.groups)
+                    for s in out:
+                        self._promise(s.request, len(s.tokens), promised)
+                self._preempt(victim)
+                if victim is req:
+                    n = 0
+                    break
+            if n == 0:
+                continue
+            self._promise(req, n, promised)
+            toks = req.tokens()[req.num_computed:req.num_computed + n]
+            out.append(Scheduled(req, req.num_computed, toks, req.num_computed + n == len(req.prompt) + len(req.output)))
+            budget -= n
+
+        # admit waiting requests in order while slots, budget and pages last
+        while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs \
+                and self.manager.free_slots > 0:
+            req = self.waiting[0]
+            total = len(req.prompt) + req.params.max_new_tokens
+            need_alone = -(-total // self.manager.page_size)
+            windows = [g.window for g in self.manager.groups]
+            if any(w is None and need_alone > tp for w, tp in zip(windows, self._total_pages())):
+                self.waiting.popleft()
+                self._finish(req, "capacity")
+                continue
+            self._begin(req.id)
+            n = min(req.remaining(), budget)
+            if not self._fits(req, n, promised):
+                # try a shorter first portion; if not even one token fits, wait
+                while n > 1 and not self._fits(req, n, promised):
+                    n = n // 2
+                if not self._fits(req, n, promised) or self.running:
+                    self._end(req.id)
+                    break
+            self.waiting.popleft()
+            req.status = RUNNING
+            self.running.append(req)
+            self._promise(req, n, promised)
+            toks = req.tokens()[:n]
+            out.append(Scheduled(req, 0, toks, n == len(req.prompt) + len(req.output)))
+            budget -= n
+        return out
+
+    def update(self, scheduled: list[Scheduled], sampled: dict) -> list[Request]:
+        """sampled: {request id: token} for every Scheduled with samples=True.
+        Returns the requests that finished in this step."""
+        done = []
+        for s in scheduled:
+            req = s.request
+            req.num_computed += len(s.tokens)
+            if not s.samples:
+                continue
+            tok = int(sampled[req.id])
+            req.output.append(tok)
+            reason = None
+            if self.eos_token_id is not None and tok == self.eos_token_id and not req.params.ignore_eos:
+                reason = "stop"
+            elif len(req.output) >= req.params.max_new_tokens:
+                reason = "length"
+            elif self.max_model_len is not None and len(req.prompt) + len(req.output) >= self.max_model_len:
+                reason = "context"
+            if reason:
+                self.running.remove(req)
+                self._end(req.id)
+                self._finish(req, reason)
+                done.append(req)
+        return done

@@ -1,0 +1,63 @@
+"""Draws the next token of every request of a step from its logits row, on the GPU.
+
+Per request: greedy if temp <= 0 (the penalty is not applied then, as in the reference's
+fast path, src/sampler.c:102-113); else repetition penalty -> min-p -> top-k -> top-p -> draw
+with the request's own xorshift128+ generator.  The uniform is drawn on the host, one per
+stochastic row, so a request's stream does not depend on what else is in the batch.
+"""
+from __future__ import annotations
+
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from ..csrc import ops
+from .params import SamplerState
+
+
+class Sampler:
+    def __init__(self, device):
+        self.device = device
+
+    def sample(self, logits: torch.Tensor, states: Sequence[SamplerState]) -> list[int]:
+        """logits: float32 [R, vocab] on the device (changed in place where a penalty applies);
+        states: the R requests' sampler states, in row order.  Returns R token ids and records
+        them in the states' rings."""
+        R = logits.shape[0]
+        if R != len(states):
+            raise ValueError(f"{R} logits rows for {len(states)} requests")
+        if R == 0:
+            return []
+        out = torch.empty(R, dtype=torch.int32, device=self.device)
+        stochastic = [s.params.temp > 0.0 for s in states]
+        if not any(stochastic):
+            ops.sample(logits, out)
+        else:
+            f32 = np.zeros((5, R), dtype=np.float32)      # temp, top_p, min_p, uniform, penalty
+            top_k = np.zeros(R, dtype=np.int32)
+            for r, s in enumerate(states):
+                p = s.params
+                f32[0, r], f32[1, r], f32[2, r], f32[4, r] = p.temp, p.top_p, p.min_p, 1.0
+                top_k[r] = p.top_k
+                if stochastic[r]:
+                    f32[3, r] = s.rng.uniform()
+                    f32[4, r] = p.repeat_penalty
+            dev = torch.from_numpy(f32).to(self.device)
+            penalised = [r for r, s in enumerate(states)
+                         if stochastic[r] and s.params.repeat_penalty > 1.0 and s.count > 0]
+            if penalised:
+                cap = max(states[r].cap for r in penalised)
+                recent = np.zeros((R, cap), dtype=np.int32)
+                counts = np.zeros(R, dtype=np.int32)
+                for r in penalised:
+                    recent[r, :states[r].count] = states[r].recent[:states[r].count]
+                    counts[r] = states[r].count
+                ops.repeat_penalty(logits, torch.from_numpy(recent).to(self.device),
+                                   torch.from_numpy(counts).to(self.device), dev[4].contiguous())
+            ops.sample(logits, out, temps=dev[0].contiguous(), top_ks=torch.from_numpy(top_k).to(self.device),
+                       top_ps=dev[1].contiguous(), min_ps=dev[2].contiguous(), uniforms=dev[3].contiguous())
+        tokens = out.cpu().tolist()
+        for s, t in zip(states, tokens):
+            s.accept(t)
+        return tokens
