@@ -132,7 +132,7 @@ def test_qkv_post(gpu, H, Hkv, hd, ps, dt):
     j = torch.arange(hd // 2, dtype=torch.float64)
     inv_freq = (base ** (-2 * j / hd)).float()
     kc = torch.zeros(n_pages, Hkv, ps, hd, dtype=dt, device=gpu)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(n_pages, Hkv, hd, ps, dtype=dt, device=gpu)
     q = torch.empty(T, H * hd, dtype=dt, device=gpu)
     ops.qkv_post(qkv.to(gpu), q, H=H, Hkv=Hkv, hd=hd, positions=pos.to(gpu), eps=eps, q_norm_w=qw.to(gpu),
                  k_norm_w=kw.to(gpu), inv_freq=inv_freq.to(gpu), rotary_dim=hd, k_cache=kc, v_cache=vc,
@@ -145,7 +145,7 @@ def test_qkv_post(gpu, H, Hkv, hd, ps, dt):
     tol = 2e-4 if dt == torch.float32 else 2 ** -7
     assert (q.cpu().double().reshape(T, H, hd) - want_q).abs().max() <= tol * float(want_q.abs().max())
     got_k = kc.cpu().double().permute(0, 2, 1, 3).reshape(n_pages * ps, Hkv, hd)[slots.long()]
-    got_v = vc.cpu().double().permute(0, 2, 1, 3).reshape(n_pages * ps, Hkv, hd)[slots.long()]
+    got_v = vc.cpu().double().permute(0, 3, 1, 2).reshape(n_pages * ps, Hkv, hd)[slots.long()]
     assert (got_k - want_k).abs().max() <= tol * float(want_k.abs().max())
     assert torch.equal(got_v, vs)
     # nothing else in the cache was touched
@@ -187,7 +187,7 @@ def _paged_case(gpu, dt, H, Hkv, hd, ps, lens, window, seed=0):
     n_pages = sum(n_blocks) + 3
     perm = torch.randperm(n_pages, generator=g).tolist()
     kc = _r(n_pages, Hkv, ps, hd, seed=seed + 1, dtype=dt)
-    vc = _r(n_pages, Hkv, ps, hd, seed=seed + 2, dtype=dt)
+    vc = _r(n_pages, Hkv, hd, ps, seed=seed + 2, dtype=dt)           # V pages are [kv_head][hd][offset]
     maxb = max(n_blocks) + 1
     table = torch.full((len(lens), maxb), -1, dtype=torch.int32)
     Ks, Vs = [], []
@@ -195,7 +195,7 @@ def _paged_case(gpu, dt, H, Hkv, hd, ps, lens, window, seed=0):
         pages = [perm.pop() for _ in range(nb)]
         table[r, :nb] = torch.tensor(pages, dtype=torch.int32)
         Ks.append(kc[pages].permute(0, 2, 1, 3).reshape(nb * ps, Hkv, hd).double())
-        Vs.append(vc[pages].permute(0, 2, 1, 3).reshape(nb * ps, Hkv, hd).double())
+        Vs.append(vc[pages].permute(0, 3, 1, 2).reshape(nb * ps, Hkv, hd).double())
     req, pos = [], []
     for r, n in enumerate(lens):
         for p in sorted({0, n // 2, max(0, n - 2), n - 1}):
@@ -226,6 +226,62 @@ def test_attention_general(gpu, H, Hkv, hd, ps, dt, window):
         assert (got - want).abs().max() <= tol * max(1.0, float(want.abs().max())), (t, int(req[t]), int(pos[t]))
 
 
+@pytest.mark.parametrize("H,Hkv,hd,ps", [(4, 2, 16, 16), (4, 1, 24, 16), (3, 3, 80, 16), (2, 1, 256, 32),
+                                          (32, 8, 64, 16), (8, 2, 128, 64), (32, 1, 64, 16), (5, 5, 40, 48)])
+@pytest.mark.parametrize("window", [0, 37, 300])
+def test_attention_mfma(gpu, H, Hkv, hd, ps, window):
+    """A mixed step: a decoded token deep in a long request, a prompt portion in the middle of
+    another, a whole short prompt, a first token.  Stale pages hold NaN."""
+    from tuff_amd.csrc import ops
+    dt = torch.bfloat16
+    # (tokens already in the cache, tokens of this step)
+    reqs = [(699, 1), (230, 50), (0, 33), (0, 1), (255, 3), (511, 2)]
+    n_blocks = [-(-(past + n) // ps) for past, n in reqs]
+    n_pages = sum(n_blocks) + 2
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(7)).tolist()
+    kc = torch.full((n_pages, Hkv, ps, hd), float("nan"), dtype=dt)
+    vc = torch.full((n_pages, Hkv, hd, ps), float("nan"), dtype=dt)
+    maxb = max(n_blocks)
+    table = torch.full((len(reqs), maxb), -1, dtype=torch.int32)
+    Ks, Vs, q_start, q_len, pos = [], [], [], [], []
+    for r, ((past, n), nb_) in enumerate(zip(reqs, n_blocks)):
+        pages = [perm.pop() for _ in range(nb_)]
+        table[r, :nb_] = torch.tensor(pages, dtype=torch.int32)
+        K = _r(past + n, Hkv, hd, seed=50 + r, dtype=dt)
+        V = _r(past + n, Hkv, hd, seed=70 + r, dtype=dt)
+        for t in range(past + n):
+            kc[pages[t // ps], :, t % ps, :] = K[t]
+            vc[pages[t // ps], :, :, t % ps] = V[t]
+        Ks.append(K.double())
+        Vs.append(V.double())
+        q_start.append(len(pos))
+        q_len.append(n)
+        pos += list(range(past, past + n))
+    T = len(pos)
+    q = _r(T, H * hd, seed=90, dtype=dt)
+    scale = 1 / math.sqrt(hd)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
+    for nb in ([1, 2, 4] if hd <= 128 else [1, 2]):
+        blk_req, blk_col0 = ops.query_blocks(q_len, H // Hkv, nb)
+        out = torch.full((T, H * hd), float("nan"), dtype=dt, device=gpu)
+        ops.attention_mfma(q.to(gpu), kc.to(gpu), vc.to(gpu), out, block_table=table.to(gpu),
+                           blk_req=torch.from_numpy(blk_req).to(gpu), blk_col0=torch.from_numpy(blk_col0).to(gpu), nb=nb,
+                           q_start=i32(q_start), q_len=i32(q_len), positions=i32(pos), H=H, Hkv=Hkv, hd=hd,
+                           page_size=ps, max_ctx_len=700, window=window)
+        got = out.cpu().double().reshape(T, H, hd)
+        assert torch.isfinite(got).all(), nb
+        if nb == 1:
+            first = got
+        else:
+            assert torch.equal(got, first), "the result depends on the column blocking"
+        t = 0
+        for r, (past, n) in enumerate(reqs):
+            for j in range(n):
+                want = _attention_reference(q[t].double().reshape(H, hd), Ks[r], Vs[r], past + j, window, scale)
+                assert (got[t] - want).abs().max() <= 2 ** -6 * max(1.0, float(want.abs().max())), (nb, r, j)
+                t += 1
+
+
 def test_attention_finds_a_far_key(gpu):
     """One key among hundreds matches the query: the output must be that key's value row,
     wherever the key sits (first position, a page's edge, a tile's edge, the last position)."""
@@ -235,7 +291,7 @@ def test_attention_finds_a_far_key(gpu):
     for dt in (torch.float32, torch.bfloat16):
         for hot in (0, 15, 16, 63, 64, 447, 448, 699):
             kc = _r(n // ps + 1, 1, ps, hd, seed=3, scale=0.05, dtype=dt)
-            vc = _r(n // ps + 1, 1, ps, hd, seed=4, dtype=dt)
+            vc = _r(n // ps + 1, 1, hd, ps, seed=4, dtype=dt)
             q = torch.zeros(1, hd, dtype=dt)
             q[0, 5] = 30.0
             kc[hot // ps, 0, hot % ps, 5] = 30.0                     # score 900/sqrt(32) = 159 above the rest
@@ -245,7 +301,7 @@ def test_attention_finds_a_far_key(gpu):
                                   req_of_token=torch.zeros(1, dtype=torch.int32, device=gpu),
                                   positions=torch.tensor([n - 1], dtype=torch.int32, device=gpu),
                                   H=1, Hkv=1, hd=hd, page_size=ps)
-            assert torch.equal(out.cpu()[0], vc[hot // ps, 0, hot % ps]), (dt, hot)
+            assert torch.equal(out.cpu()[0], vc[hot // ps, 0, :, hot % ps]), (dt, hot)
 
 
 def test_attention_window_edge(gpu):
@@ -254,11 +310,11 @@ def test_attention_window_edge(gpu):
     hd, ps, W, pos = 16, 16, 40, 100
     for edge, seen in ((pos - W + 1, True), (pos - W, False)):
         kc = torch.zeros(8, 1, ps, hd)
-        vc = torch.zeros(8, 1, ps, hd)
+        vc = torch.zeros(8, 1, hd, ps)
         q = torch.zeros(1, hd)
         q[0, 0] = 20.0
         kc[edge // ps, 0, edge % ps, 0] = 20.0
-        vc[edge // ps, 0, edge % ps, :] = 1.0
+        vc[edge // ps, 0, :, edge % ps] = 1.0
         out = torch.empty(1, hd, device=gpu)
         ops.attention_general(q.to(gpu), kc.to(gpu), vc.to(gpu), out,
                               block_table=torch.arange(8, dtype=torch.int32, device=gpu)[None],

@@ -1,6 +1,8 @@
 """The tensors behind the cache manager's book-keeping.
 
-Per PagedKV entry: K and V as [num_pages, kv_heads, page_size, head_dim] in the compute dtype
+Per PagedKV entry: K as [num_pages, kv_heads, page_size, head_dim] and V transposed within the
+page, [num_pages, kv_heads, head_dim, page_size] (the matrix cores read both with the summed
+index contiguous), in the compute dtype
 (bfloat16 in serving, float32 in the 32-bit path; the reference keeps float32 rows
 [layer][kv_head][pos][hd], src/lfm25_gpu.cu:480-483).  Per FixedState entry: one float32
 tensor [num_slots, *shape].  Pages are not cleared when they are handed out again: nothing
@@ -41,13 +43,14 @@ class CacheStorage:
             gi = layout.group_of_entry[e]
             n = manager.groups[gi].pool.num_pages
             shape = (n, spec.num_kv_heads, ps, spec.head_dim)
+            vshape = (n, spec.num_kv_heads, spec.head_dim, ps)
             if poison:
                 # stale reads show up as NaN in the logits
                 k = torch.full(shape, float("nan"), dtype=dtype, device=device)
-                v = torch.full(shape, float("nan"), dtype=dtype, device=device)
+                v = torch.full(vshape, float("nan"), dtype=dtype, device=device)
             else:
                 k = torch.empty(shape, dtype=dtype, device=device)
-                v = torch.empty(shape, dtype=dtype, device=device)
+                v = torch.empty(vshape, dtype=dtype, device=device)
             self.views[e] = PagedKVView(k, v, gi, ps, spec.window)
         for e, spec in layout.states.items():
             st = torch.zeros((manager.num_slots,) + tuple(spec.shape), dtype=torch.float32, device=device)

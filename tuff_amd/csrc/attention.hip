@@ -11,6 +11,8 @@
 // aligned to absolute positions (0, 64, 128, ...), so the order of every sum depends
 // only on the token's position, not on how the sequence was cut into steps.
 //
+// Cache layout: K [page][kv_head][offset][hd], V [page][kv_head][hd][offset].
+//
 // This is the general kernel: any head size up to 256, any page size, float32 or
 // bfloat16 cache.  One wave per (token, head): lanes are keys for q.k, lanes are
 // channels for p.v.
@@ -49,8 +51,9 @@ __global__ __launch_bounds__(WAVE) void attention_general_kernel(
         long long base = 0;
         if (valid) {
             const long long page = table[kt / page_size];
-            base = ((page * Hkv + kvh) * page_size + (kt % page_size)) * (long long)hd;
-            const T* krow = k_cache + base;
+            const long long head_base = (page * Hkv + kvh) * page_size * (long long)hd;
+            base = head_base + (kt % page_size);          // V: [hd][page_size], this key's column
+            const T* krow = k_cache + head_base + (long long)(kt % page_size) * hd;
             float d = 0.f;
             for (int j = 0; j < hd; ++j) d = fmaf(qs[j], to_f32(krow[j]), d);
             s = d * scale;
@@ -70,11 +73,11 @@ __global__ __launch_bounds__(WAVE) void attention_general_kernel(
         for (int jj = 0; jj < n_keys; ++jj) {
             const float pj = ps[jj];
             if (pj == 0.f) continue;                 // masked (below the window) or underflowed
-            const T* vrow = v_cache + voff[jj];
+            const T* vcol = v_cache + voff[jj];
 #pragma unroll
             for (int i = 0; i < MAX_PER_LANE; ++i) {
                 const int j = lane + i * WAVE;
-                if (j < hd) acc[i] = fmaf(pj, to_f32(vrow[j]), acc[i]);
+                if (j < hd) acc[i] = fmaf(pj, to_f32(vcol[(long long)j * page_size]), acc[i]);
             }
         }
     }

@@ -1,0 +1,270 @@
+// Paged attention on the gfx950 matrix cores, bfloat16 cache, for prompt portions and decoded
+// tokens alike.
+//
+// Work is cut the same way whatever the batch: the keys of a request are split into partitions
+// of 256 positions (0..255, 256..511, ...).  One wave takes one partition, one kv head and one
+// block of query columns (a column = one query head of one token; all columns of a block share
+// the request and the kv head).  It produces, per column, the running maximum m, the sum l and
+// the unnormalised output o of that partition, in float32.  A second kernel merges a token's
+// partitions in ascending order.  Since the columns of a matrix product do not influence each
+// other, a token's result does not depend on how the sequence was cut into steps or on what
+// else was in the batch.
+//
+// Inside a wave (S^T = K Q^T, O^T = V^T P^T, all with v_mfma_f32_16x16x32_bf16):
+//  * 32 keys a step, as two blocks of 16.  A operand of S^T: K rows [key][hd], 16 bytes a lane.
+//    B operand: Q [column][hd], loaded once.
+//  * The result tile gives lane (column = l % 16, group g = l / 16) the scores of keys
+//    4g..4g+3 of each block.  After masking, running max and exp these eight values are,
+//    as they lie, the lane's part of the B operand P^T of the second product if the product's
+//    summed index is numbered k = 8g + i  <->  key (i < 4 ? 4g + i : 16 + 4g + i - 4).  The
+//    A operand V^T follows the same numbering: two 8-byte loads from the transposed V page.
+//  * No LDS, no transposes, no barriers.
+//
+// Cache layout: K [page][kv_head][offset][hd], V [page][kv_head][hd][offset]; the page size
+// must be a multiple of 16 and the head size a multiple of 8 (the host falls back to the
+// general kernel otherwise).
+#include "common.h"
+#include <math.h>
+
+namespace {
+constexpr int PART = 256;
+
+__device__ __forceinline__ f32x4 mfma32(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+template <int HDP, int NB>
+__global__ __launch_bounds__(WAVE) void attn_partition_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    float* __restrict__ ws_o, float* __restrict__ ws_ml,
+    const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ blk_req, const int* __restrict__ blk_col0,
+    const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ positions,
+    int H, int Hkv, int hd, int page_size, int window, float scale, int n_parts) {
+    constexpr int KC = HDP / 32;          // 32-wide chunks of the head dimension
+    constexpr int DB = HDP / 16;          // 16-wide blocks of output channels
+    const int part = blockIdx.x, qb = blockIdx.y, kvh = blockIdx.z;
+    const int lane = threadIdx.x, n16 = lane % 16, g = lane / 16;
+    const int G = H / Hkv;
+    const int r = blk_req[qb], col0 = blk_col0[qb];
+    const int t0 = q_start[r], ncols = q_len[r] * G;
+    const int* table = block_table + (long long)r * max_blocks;
+
+    // the block's range of keys
+    const int last_col = min(ncols, col0 + NB * 16) - 1;
+    const int pos_max = positions[t0 + last_col / G];
+    const int lo_min = window > 0 ? max(0, positions[t0 + col0 / G] - window + 1) : 0;
+    const int key_begin = part * PART;
+    if (key_begin > pos_max || key_begin + PART <= lo_min) return;
+    const int key_end = min(key_begin + PART, pos_max + 1);
+
+    // this lane's columns
+    int pos_c[NB], lo_c[NB];
+    long long qrow[NB];                    // row of the column in q / in the work space; -1: no column
+    bf16x8 qf[NB][KC];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int c = col0 + nb * 16 + n16;
+        const bool valid = c < ncols;
+        const int tok = t0 + (valid ? c / G : 0);
+        const int head = kvh * G + (valid ? c % G : 0);
+        pos_c[nb] = valid ? positions[tok] : -1;
+        lo_c[nb] = (valid && window > 0) ? max(0, pos_c[nb] - window + 1) : 0;
+        qrow[nb] = valid ? (long long)tok * H + head : -1;
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc) {
+            const int k = kc * 32 + g * 8;
+            bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+            qf[nb][kc] = (valid && k < hd) ? *(const bf16x8*)(q + qrow[nb] * hd + k) : z;
+        }
+    }
+
+    float m_run[NB], l_run[NB];
+    f32x4 o[DB][NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        m_run[nb] = -INFINITY;
+        l_run[nb] = 0.f;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) o[db][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    for (int key0 = key_begin; key0 < key_end; key0 += 32) {
+        // ---- S^T = K Q^T for two blocks of 16 keys
+        f32x4 s[2][NB];
+        long long vbase[2];                // start of the block's 16 positions in the V page, or -1
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            const int kbs = key0 + kb * 16;
+            const bool live = kbs <= pos_max && kbs + 15 >= lo_min;
+            vbase[kb] = -1;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) s[kb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (live) {
+                const long long page = table[kbs / page_size];
+                const int off0 = kbs % page_size;
+                const long long head_base = (page * Hkv + kvh) * (long long)page_size * hd;
+                vbase[kb] = head_base + off0;
+                const bf16_t* krow = k_cache + head_base + (long long)(off0 + n16) * hd;
+#pragma unroll
+                for (int kc = 0; kc < KC; ++kc) {
+                    const int k = kc * 32 + g * 8;
+                    bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+                    const bf16x8 kf = (k < hd) ? *(const bf16x8*)(krow + k) : z;
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) s[kb][nb] = mfma32(kf, qf[nb][kc], s[kb][nb]);
+                }
+            }
+        }
+        // ---- mask, running maximum, exp; P^T stays in registers as the next B operand
+        bf16x8 pf[NB];
+        float corr[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            float v[8];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int key = key0 + kb * 16 + 4 * g + e;
+                    const bool ok = vbase[kb] >= 0 && key <= pos_c[nb] && key >= lo_c[nb];
+                    const float x = ok ? s[kb][nb][e] * scale : -INFINITY;
+                    v[kb * 4 + e] = x;
+                    mx = fmaxf(mx, x);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+            const float m_new = fmaxf(m_run[nb], mx);
+            const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+            corr[nb] = __expf(m_run[nb] - m_safe);          // 0 while nothing was seen yet
+            float sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float p = __expf(v[i] - m_safe);
+                sum += p;
+                pf[nb][i] = (bf16_t)p;
+            }
+            l_run[nb] = l_run[nb] * corr[nb] + sum;
+            m_run[nb] = m_new;
+        }
+        // ---- O^T = O^T * corr + V^T P^T
+        const bool tail = key0 + 31 > pos_max;             // keys beyond pos_max were never written
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            const int dim = db * 16 + n16;
+            bf16x8 vf = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (dim < hd) {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+                    if (vbase[kb] < 0) continue;
+                    const bf16x4 x = *(const bf16x4*)(v_cache + vbase[kb] + (long long)dim * page_size + 4 * g);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const bool written = !tail || (key0 + kb * 16 + 4 * g + e <= pos_max);
+                        vf[kb * 4 + e] = written ? x[e] : (bf16_t)0.f;
+                    }
+                }
+            }
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                f32x4 acc = o[db][nb];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] *= corr[nb];
+                o[db][nb] = mfma32(vf, pf[nb], acc);
+            }
+        }
+    }
+
+    // ---- the partition's result per column
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        float l = l_run[nb];
+        l += __shfl_xor(l, 16, WAVE);
+        l += __shfl_xor(l, 32, WAVE);
+        if (qrow[nb] < 0) continue;
+        const long long slot = qrow[nb] * n_parts + part;
+        if (g == 0) { ws_ml[slot * 2] = m_run[nb]; ws_ml[slot * 2 + 1] = l; }
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            const int dim = db * 16 + 4 * g;
+            if (dim < hd) *(f32x4*)(ws_o + slot * hd + dim) = o[db][nb];
+        }
+    }
+}
+
+// Merges the partitions of one (token, head) in ascending order and writes the bfloat16 row.
+__global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+                                                            bf16_t* __restrict__ out, const int* __restrict__ positions,
+                                                            int H, int hd, int window, int n_parts) {
+    const long long row = blockIdx.x;                      // token * H + head
+    const int lane = threadIdx.x;
+    const int pos = positions[row / H];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    float M = -INFINITY, L = 0.f;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int p = lo / PART; p <= pos / PART; ++p) {
+        const long long slot = row * n_parts + p;
+        const float m = ws_ml[slot * 2], l = ws_ml[slot * 2 + 1];
+        if (!(l > 0.f)) continue;
+        const float M_new = fmaxf(M, m);
+        const float a = __expf(M - M_new), b = __expf(m - M_new);
+        L = L * a + l * b;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int d = lane + i * WAVE;
+            if (d < hd) acc[i] = acc[i] * a + ws_o[slot * hd + d] * b;
+        }
+        M = M_new;
+    }
+    const float inv = 1.0f / L;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int d = lane + i * WAVE;
+        if (d < hd) out[row * hd + d] = (bf16_t)(acc[i] * inv);
+    }
+}
+
+template <int HDP, int NB>
+void launch_partition(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, float* ws_o,
+                      float* ws_ml, const int* bt, int max_blocks, const int* blk_req, const int* blk_col0,
+                      const int* q_start, const int* q_len, const int* positions, int H, int Hkv, int hd, int ps,
+                      int window, float scale, int n_parts) {
+    hipLaunchKernelGGL((attn_partition_kernel<HDP, NB>), grid, dim3(WAVE), 0, stream, q, kc, vc, ws_o, ws_ml, bt, max_blocks,
+                       blk_req, blk_col0, q_start, q_len, positions, H, Hkv, hd, ps, window, scale, n_parts);
+}
+}  // namespace
+
+// Query blocks are listed by the host: block b holds the columns blk_col0[b] .. +16*nb-1 of request
+// blk_req[b] (a request's columns are numbered (token - q_start) * G + head within the kv group).
+// ws_o: float32 [n_tokens * H * n_parts * hd], ws_ml: float32 [n_tokens * H * n_parts * 2].
+// n_parts >= ceil((largest position + 1) / 256).  nb: 1, 2 or 4 column blocks a wave.
+TUFF_EXPORT int tuff_attention_mfma(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                    float* ws_o, float* ws_ml, const int* block_table, int max_blocks,
+                                    const int* blk_req, const int* blk_col0, int n_qblocks, int nb,
+                                    const int* q_start, const int* q_len, const int* positions,
+                                    int n_tokens, int H, int Hkv, int hd, int page_size, int window, float scale,
+                                    int n_parts, hipStream_t stream) {
+    if (n_tokens <= 0 || n_qblocks <= 0) return 0;
+    if (hd > 256 || hd % 8 != 0 || page_size % 16 != 0 || Hkv <= 0 || H % Hkv != 0 || n_parts < 1) return -2;
+    if (Hkv > 65535 || n_qblocks > 65535) return -2;
+    const bf16_t* Q = (const bf16_t*)q;
+    const bf16_t* K = (const bf16_t*)k_cache;
+    const bf16_t* V = (const bf16_t*)v_cache;
+    dim3 grid(n_parts, n_qblocks, Hkv);
+#define GO(HDP, NB) launch_partition<HDP, NB>(grid, stream, Q, K, V, ws_o, ws_ml, block_table, max_blocks, blk_req, blk_col0, \
+                                              q_start, q_len, positions, H, Hkv, hd, page_size, window, scale, n_parts)
+#define BY_NB(HDP) do { if (nb == 1) GO(HDP, 1); else if (nb == 2) GO(HDP, 2); else if (nb == 4) GO(HDP, 4); else return -2; } while (0)
+    if (hd <= 32) BY_NB(32);
+    else if (hd <= 64) BY_NB(64);
+    else if (hd <= 96) BY_NB(96);
+    else if (hd <= 128) BY_NB(128);
+    else { if (nb == 1) GO(256, 1); else if (nb == 2) GO(256, 2); else return -2; }
+#undef BY_NB
+#undef GO
+    int rc = launch_status();
+    if (rc) return rc;
+    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)((long long)n_tokens * H)), dim3(WAVE), 0, stream,
+                       (const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, H, hd, window, n_parts);
+    return launch_status();
+}

@@ -29,6 +29,7 @@ MODULES = {
     "gemm_bf16": "gemm_bf16.hip",
     "rope_kv": "rope_kv.hip",
     "attention": "attention.hip",
+    "attention_mfma": "attention_mfma.hip",
     "shortconv": "shortconv.hip",
     "sampling": "sampling.hip",
 }
@@ -54,7 +55,7 @@ def _writable_dir() -> str:
             continue
         try:
             os.makedirs(d, exist_ok=True)
-            probe = os.path.join(d, f".probe_{os.getpid()}")
+            probe = os.path.join(d, f".probe_{os.getpid()}_{threading.get_ident()}")
             with open(probe, "w"):
                 pass
             os.unlink(probe)

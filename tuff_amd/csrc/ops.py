@@ -51,6 +51,11 @@ _SIGNATURES = {
                                    _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                    _c_float, _c_void_p],
     },
+    "attention_mfma": {
+        "tuff_attention_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                                _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p,
+                                _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p],
+    },
     "shortconv": {
         "tuff_shortconv_fwd": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
@@ -215,7 +220,7 @@ def qkv_post(qkv, q_out, *, H, Hkv, hd, positions, eps=0.0, q_norm_w=None, k_nor
             raise KernelError("qkv_post: a cache write needs slot_mapping")
         P = k_cache.shape[0]
         _gpu("k_cache", k_cache, dt, (P, Hkv, page_size, hd))
-        _gpu("v_cache", v_cache, dt, (P, Hkv, page_size, hd))
+        _gpu("v_cache", v_cache, dt, (P, Hkv, hd, page_size))
         _gpu("slot_mapping", slot_mapping, torch.int32, (T,))
     norm_dt = DT_F32
     if q_norm_w is not None or k_norm_w is not None:
@@ -245,7 +250,7 @@ def kv_write(k, v, k_cache, v_cache, slot_mapping, *, Hkv, hd, page_size) -> Non
     _gpu("v", v, dt, (T, Hkv * hd))
     P = k_cache.shape[0]
     _gpu("k_cache", k_cache, dt, (P, Hkv, page_size, hd))
-    _gpu("v_cache", v_cache, dt, (P, Hkv, page_size, hd))
+    _gpu("v_cache", v_cache, dt, (P, Hkv, hd, page_size))
     _gpu("slot_mapping", slot_mapping, torch.int32, (T,))
     _check(load("rope_kv").tuff_kv_write(k.data_ptr(), v.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                          _dt(k), slot_mapping.data_ptr(), T, Hkv, hd, page_size, _stream()),
@@ -261,7 +266,7 @@ def attention_general(q, k_cache, v_cache, out, *, block_table, req_of_token, po
     _gpu("out", out, dt, (T, H * hd))
     P = k_cache.shape[0]
     _gpu("k_cache", k_cache, dt, (P, Hkv, page_size, hd))
-    _gpu("v_cache", v_cache, dt, (P, Hkv, page_size, hd))
+    _gpu("v_cache", v_cache, dt, (P, Hkv, hd, page_size))
     _gpu("block_table", block_table, torch.int32)
     if block_table.dim() != 2:
         raise KernelError("attention: block_table must be [requests, blocks]")
@@ -275,6 +280,65 @@ def attention_general(q, k_cache, v_cache, out, *, block_table, req_of_token, po
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _dt(q),
         block_table.data_ptr(), block_table.shape[1], req_of_token.data_ptr(), positions.data_ptr(),
         T, H, Hkv, hd, page_size, int(window or 0), float(scale), _stream()), "attention_general")
+
+
+ATTN_PARTITION = 256        # keys a partition of the matrix-core attention kernel covers
+
+
+def attention_mfma_supported(dtype, hd: int, page_size: int) -> bool:
+    return dtype == torch.bfloat16 and hd % 8 == 0 and hd <= 256 and page_size % 16 == 0
+
+
+def attention_mfma(q, k_cache, v_cache, out, *, block_table, blk_req, blk_col0, nb, q_start, q_len, positions,
+                   H, Hkv, hd, page_size, max_ctx_len, window=0, scale=None) -> None:
+    """Matrix-core attention over the paged bfloat16 cache.  blk_req / blk_col0 list the query
+    blocks (see query_blocks()); max_ctx_len bounds every position + 1 of the step."""
+    T = q.shape[0]
+    if not attention_mfma_supported(q.dtype, hd, page_size):
+        raise KernelError(f"attention_mfma: needs bfloat16, a head size that is a multiple of 8 (got {hd}) "
+                          f"and a page size that is a multiple of 16 (got {page_size})")
+    _gpu("q", q, torch.bfloat16, (T, H * hd))
+    _gpu("out", out, torch.bfloat16, (T, H * hd))
+    P = k_cache.shape[0]
+    _gpu("k_cache", k_cache, torch.bfloat16, (P, Hkv, page_size, hd))
+    _gpu("v_cache", v_cache, torch.bfloat16, (P, Hkv, hd, page_size))
+    _gpu("block_table", block_table, torch.int32)
+    R = q_start.shape[0]
+    if block_table.dim() != 2 or block_table.shape[0] != R:
+        raise KernelError("attention_mfma: block_table must be [requests, blocks]")
+    n_parts = max(1, -(-int(max_ctx_len) // ATTN_PARTITION))
+    if block_table.shape[1] * page_size < int(max_ctx_len):
+        raise KernelError("attention_mfma: block_table is narrower than the longest context")
+    nblk = blk_req.shape[0]
+    _gpu("blk_req", blk_req, torch.int32, (nblk,))
+    _gpu("blk_col0", blk_col0, torch.int32, (nblk,))
+    _gpu("q_start", q_start, torch.int32, (R,))
+    _gpu("q_len", q_len, torch.int32, (R,))
+    _gpu("positions", positions, torch.int32, (T,))
+    if nb not in (1, 2, 4) or (hd > 128 and nb == 4) or H % Hkv:
+        raise KernelError(f"attention_mfma: unsupported column blocking nb={nb} for head size {hd}")
+    if scale is None:
+        scale = 1.0 / math.sqrt(hd)
+    ws_o = torch.empty(T * H * n_parts * hd, dtype=torch.float32, device=q.device)
+    ws_ml = torch.empty(T * H * n_parts * 2, dtype=torch.float32, device=q.device)
+    _check(load("attention_mfma").tuff_attention_mfma(
+        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), ws_o.data_ptr(), ws_ml.data_ptr(),
+        block_table.data_ptr(), block_table.shape[1], blk_req.data_ptr(), blk_col0.data_ptr(), nblk, nb,
+        q_start.data_ptr(), q_len.data_ptr(), positions.data_ptr(), T, H, Hkv, hd, page_size,
+        int(window or 0), float(scale), n_parts, _stream()), "attention_mfma")
+
+
+def query_blocks(q_len, G: int, nb: int):
+    """Host lists of query blocks for attention_mfma: for request r with q_len[r] tokens the
+    columns (token, head in group) are cut into blocks of 16 * nb.  Returns (blk_req, blk_col0)
+    as int32 numpy arrays."""
+    import numpy as np
+    q_len = np.asarray(q_len, dtype=np.int64)
+    per = -(-(q_len * G) // (16 * nb))
+    blk_req = np.repeat(np.arange(len(q_len)), per).astype(np.int32)
+    starts = np.concatenate([[0], np.cumsum(per)])[:-1]
+    blk_col0 = ((np.arange(int(per.sum())) - np.repeat(starts, per)) * 16 * nb).astype(np.int32)
+    return blk_req, blk_col0
 
 
 # ------------------------------------------------------------------------- short conv

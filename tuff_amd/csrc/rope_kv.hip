@@ -6,7 +6,9 @@
 // :487-501 (V cached as projected).  Here theta_j comes in as a float32 table and the
 // angle pos * theta_j, its cosine and sine are float32.
 //
-// Cache layout: [page][kv_head][offset][hd]; slot = page * page_size + offset.
+// Cache layout, slot = page * page_size + offset:
+//   K [page][kv_head][offset][hd]      a key's channels are contiguous (q.k runs over hd)
+//   V [page][kv_head][hd][offset]      a channel's positions are contiguous (p.v runs over keys)
 #include "common.h"
 
 namespace {
@@ -67,6 +69,7 @@ __global__ __launch_bounds__(WAVE) void qkv_post_kernel(
     }
     T* dst = nullptr;
     T* dst2 = nullptr;
+    long long dst_stride = 1;
     if (is_q) dst = q_out + ((long long)t * H + head) * hd;
     else {
         if (is_k && k_out) dst2 = k_out + ((long long)t * Hkv + kvh) * hd;
@@ -74,7 +77,9 @@ __global__ __launch_bounds__(WAVE) void qkv_post_kernel(
             const long long slot = slot_mapping[t];
             if (slot >= 0) {
                 const long long page = slot / page_size, off = slot % page_size;
-                dst = (is_k ? k_cache : v_cache) + ((page * Hkv + kvh) * page_size + off) * hd;
+                const long long head_base = (page * Hkv + kvh) * page_size * hd;
+                if (is_k) dst = k_cache + head_base + off * hd;
+                else { dst = v_cache + head_base + off; dst_stride = page_size; }
             }
         }
     }
@@ -83,7 +88,7 @@ __global__ __launch_bounds__(WAVE) void qkv_post_kernel(
         const int j = lane + i * WAVE;
         if (j < hd) {
             const T o = from_f32<T>(v[i]);
-            if (dst) dst[j] = o;
+            if (dst) dst[j * dst_stride] = o;
             if (dst2) dst2[j] = o;
         }
     }
@@ -98,9 +103,12 @@ __global__ __launch_bounds__(WAVE) void kv_write_kernel(const T* __restrict__ k,
     const long long slot = slot_mapping[t];
     if (slot < 0) return;
     const long long page = slot / page_size, off = slot % page_size;
-    const long long dst = ((page * Hkv + kvh) * page_size + off) * hd;
+    const long long head_base = (page * Hkv + kvh) * page_size * hd;
     const long long src = ((long long)t * Hkv + kvh) * hd;
-    for (int j = threadIdx.x; j < hd; j += WAVE) { k_cache[dst + j] = k[src + j]; v_cache[dst + j] = v[src + j]; }
+    for (int j = threadIdx.x; j < hd; j += WAVE) {
+        k_cache[head_base + off * hd + j] = k[src + j];
+        v_cache[head_base + (long long)j * page_size + off] = v[src + j];
+    }
 }
 }  // namespace
 

@@ -53,7 +53,7 @@ class AttentionMixer(Mixer):
         return decls
 
     def kernel_modules(self):
-        mods = ["rope_kv", "attention"]
+        mods = ["rope_kv", "attention", "attention_mfma"]
         if self.position is not None:
             mods += self.position.kernel_modules()
         return mods
@@ -102,6 +102,24 @@ class AttentionMixer(Mixer):
         self.out.forward(o, accumulate_into=residual)
 
     def attend(self, q, o, ctx, cache, g) -> None:
+        G = self.H // self.Hkv
+        if ops.attention_mfma_supported(q.dtype, self.hd, cache.page_size):
+            if ctx.max_q_len == 1:
+                nb = 1 if G <= 16 else (2 if G <= 32 else 4)
+            else:
+                nb = 4 if self.hd <= 128 else 2
+            key = ("query_blocks", G, nb)
+            blocks = ctx.host.get(key)
+            if blocks is None:
+                blk_req, blk_col0 = ops.query_blocks(ctx.host["q_len"], G, nb)
+                blocks = (torch.from_numpy(blk_req).to(q.device), torch.from_numpy(blk_col0).to(q.device))
+                ctx.host[key] = blocks
+            ops.attention_mfma(q, cache.k, cache.v, o, block_table=g.block_table, blk_req=blocks[0],
+                               blk_col0=blocks[1], nb=nb, q_start=ctx.q_start, q_len=ctx.q_len,
+                               positions=ctx.positions, H=self.H, Hkv=self.Hkv, hd=self.hd,
+                               page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len,
+                               window=self.window or 0, scale=self.scale)
+            return
         ops.attention_general(q, cache.k, cache.v, o, block_table=g.block_table,
                               req_of_token=ctx.req_of_token, positions=ctx.positions,
                               H=self.H, Hkv=self.Hkv, hd=self.hd, page_size=cache.page_size,
