@@ -1,0 +1,246 @@
+"""The scheduler's decisions (CPU), against a fake step function that checks what it is fed."""
+import hashlib
+
+import pytest
+
+from tuff_amd.cache.manager import CacheLayout, CacheManager
+from tuff_amd.engine.scheduler import Request, Scheduler
+from tuff_amd.parts.base import FixedState, PagedKV
+from tuff_amd.sampling.params import SamplingParams
+
+V = 1000
+
+
+def next_token(history) -> int:
+    """A stand-in model: the next token is a hash of everything before it."""
+    return int.from_bytes(hashlib.sha256(repr(list(history)).encode()).digest()[:4], "little") % V
+
+
+class FakeExecutor:
+    """Holds a real CacheManager; 'runs' a step by extending it and checks that every request is
+    fed its tokens in order, from the position its cache holds."""
+
+    def __init__(self, num_pages=64, page_size=4, num_slots=4, window=None):
+        lay = CacheLayout.from_specs({0: PagedKV(1, 8, window), 1: FixedState((2, 4))})
+        self.manager = CacheManager(lay, page_size, num_pages, num_slots)
+        self.fed = {}
+        self.begun = 0
+
+    def begin(self, rid):
+        self.manager.admit(rid)
+        self.fed[rid] = []
+        self.begun += 1
+
+    def end(self, rid):
+        self.manager.release(rid)
+        del self.fed[rid]
+
+    def step(self, batch):
+        out = {}
+        for s in batch:
+            rid = s.request.id
+            assert s.start == len(self.fed[rid]) == self.manager.length(rid), "fed out of order"
+            self.manager.extend(rid, len(s.tokens))         # must never fail: the scheduler promised
+            self.fed[rid] += list(s.tokens)
+            if s.samples:
+                out[rid] = next_token(self.fed[rid])
+        self.manager.check()
+        return out
+
+
+def run(sched, ex, max_steps=10000):
+    steps = []
+    while sched.has_unfinished():
+        batch = sched.schedule()
+        assert batch, "the scheduler stalled"
+        assert sum(len(s.tokens) for s in batch) <= sched.max_batched_tokens
+        assert len({s.request.id for s in batch}) == len(batch)
+        sched.update(batch, ex.step(batch))
+        steps.append(batch)
+        assert len(steps) < max_steps
+    return steps
+
+
+def make(ex, **kw):
+    kw.setdefault("max_num_seqs", 4)
+    kw.setdefault("max_batched_tokens", 16)
+    return Scheduler(ex.manager, begin=ex.begin, end=ex.end, **kw)
+
+
+def expected_output(prompt, n):
+    hist, out = list(prompt), []
+    for _ in range(n):
+        t = next_token(hist)
+        out.append(t)
+        hist.append(t)
+    return out
+
+
+def test_one_request_prompt_in_portions_then_decode():
+    ex = FakeExecutor()
+    sched = make(ex, max_batched_tokens=8)
+    req = Request("a", list(range(21)), SamplingParams(max_new_tokens=5))
+    sched.add(req)
+    steps = run(sched, ex)
+    assert [len(b[0].tokens) for b in steps] == [8, 8, 5, 1, 1, 1, 1]       # cut under the budget
+    assert [b[0].samples for b in steps] == [False, False, True, True, True, True, True]
+    assert req.output == expected_output(range(21), 5) and req.finish_reason == "length"
+    assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == 64
+
+
+def test_decodes_go_first_and_prompts_share_the_rest_of_the_budget():
+    ex = FakeExecutor()
+    sched = make(ex, max_batched_tokens=10)
+    a = Request("a", list(range(4)), SamplingParams(max_new_tokens=6))
+    b = Request("b", list(range(100, 125)), SamplingParams(max_new_tokens=2))
+    sched.add(a)
+    sched.add(b)
+    first = sched.schedule()
+    assert [(s.request.id, len(s.tokens)) for s in first] == [("a", 4), ("b", 6)]
+    sched.update(first, ex.step(first))
+    second = sched.schedule()
+    assert [(s.request.id, len(s.tokens), s.samples) for s in second] == [("a", 1, True), ("b", 9, False)]
+    sched.update(second, ex.step(second))
+    run(sched, ex)
+    assert a.output == expected_output(range(4), 6) and b.output == expected_output(range(100, 125), 2)
+
+
+def test_admission_is_fifo_and_bounded_by_slots_and_max_num_seqs():
+    ex = FakeExecutor(num_slots=2)
+    sched = make(ex, max_num_seqs=3, max_batched_tokens=64)
+    reqs = [Request(i, [i] * 3, SamplingParams(max_new_tokens=3)) for i in range(5)]
+    for r in reqs:
+        sched.add(r)
+    first = sched.schedule()
+    assert [s.request.id for s in first] == [0, 1]                       # two slots only
+    sched.update(first, ex.step(first))
+    steps = run(sched, ex)
+    order = []
+    for b in [first] + steps:
+        for s in b:
+            if s.start == 0 and s.request.id not in order:
+                order.append(s.request.id)
+    assert order == [0, 1, 2, 3, 4]
+    assert all(r.output == expected_output([r.id] * 3, 3) for r in reqs)
+
+
+def test_finish_reasons():
+    ex = FakeExecutor()
+    sched = make(ex, max_model_len=12, eos_token_id=next_token([5, 6, 7]))
+    stop = Request("stop", [5, 6, 7], SamplingParams(max_new_tokens=5))
+    ignore = Request("ignore", [5, 6, 7], SamplingParams(max_new_tokens=2, ignore_eos=True))
+    too_long = Request("long", list(range(10)), SamplingParams(max_new_tokens=3))
+    ctx = Request("ctx", list(range(10)), SamplingParams(max_new_tokens=2))
+    zero = Request("zero", [1], SamplingParams(max_new_tokens=0))
+    for r in (stop, ignore, too_long, ctx, zero):
+        sched.add(r)
+    run(sched, ex)
+    assert stop.finish_reason == "stop" and len(stop.output) == 1
+    assert ignore.finish_reason == "length" and len(ignore.output) == 2
+    assert too_long.finish_reason.startswith("rejected") and too_long.output == []
+    assert ctx.finish_reason in ("length", "context") and len(ctx.output) == 2
+    assert zero.finish_reason == "length" and zero.output == []
+    with pytest.raises(ValueError, match="empty prompt"):
+        sched.add(Request("e", [], SamplingParams()))
+
+
+def test_pages_run_out_preempt_the_latest_and_recompute_with_unchanged_output():
+    """Pool of 12 pages of 4 tokens; three requests that each grow to 28 tokens (7 pages) cannot
+    all stay: the most recently admitted running request is preempted, comes back later and is
+    computed again from its first token.  Every output equals the unconstrained one."""
+    prompts = {"a": list(range(8)), "b": list(range(50, 58)), "c": list(range(90, 98))}
+    ex = FakeExecutor(num_pages=12, page_size=4)
+    sched = make(ex, max_batched_tokens=32)
+    reqs = {k: Request(k, p, SamplingParams(max_new_tokens=20)) for k, p in prompts.items()}
+    for r in reqs.values():
+        sched.add(r)
+    steps = run(sched, ex)
+    assert sched.num_preemptions >= 1
+    assert reqs["c"].preemptions >= 1 and reqs["a"].preemptions == 0      # the latest admitted goes first
+    for k, p in prompts.items():
+        assert reqs[k].output == expected_output(p, 20), k
+        assert reqs[k].finish_reason == "length"
+    # a preempted request restarts at position 0 with prompt and generated tokens together
+    restarts = [s for b in steps for s in b if s.request.id == "c" and s.start == 0]
+    assert len(restarts) >= 2
+    fed_c = sum(len(s.tokens) for b in steps for s in b if s.request.id == "c")
+    assert fed_c > len(prompts["c"]) + 19                                   # tokens were computed again
+    after = [s for b in steps[[i for i, b in enumerate(steps) if restarts[-1] in b][0]:] for s in b if s.request.id == "c"]
+    assert [s.start for s in after] == [sum(len(x.tokens) for x in after[:i]) for i in range(len(after))]
+    assert any(s.start < len(prompts["c"]) < s.start + len(s.tokens) and not s.samples or
+               (s.start + len(s.tokens) > len(prompts["c"]) and len(s.tokens) > 1) for s in after)
+    assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == 12
+
+
+def test_waiting_request_is_not_admitted_into_a_full_pool():
+    ex = FakeExecutor(num_pages=6, page_size=4)
+    sched = make(ex, max_batched_tokens=64)
+    a = Request("a", list(range(20)), SamplingParams(max_new_tokens=3))      # 5 pages, 6 at the end
+    b = Request("b", list(range(8)), SamplingParams(max_new_tokens=2))
+    sched.add(a)
+    sched.add(b)
+    first = sched.schedule()
+    assert [s.request.id for s in first] == ["a"]                          # b would not fit beside a
+    sched.update(first, ex.step(first))
+    run(sched, ex)
+    assert a.output == expected_output(range(20), 3) and b.output == expected_output(range(8), 2)
+    assert b.preemptions == 0
+
+
+def test_request_larger_than_the_pool_is_finished_with_capacity():
+    ex = FakeExecutor(num_pages=4, page_size=4)
+    sched = make(ex)
+    big = Request("big", list(range(30)), SamplingParams(max_new_tokens=4))
+    ok = Request("ok", list(range(6)), SamplingParams(max_new_tokens=4))
+    sched.add(big)
+    sched.add(ok)
+    run(sched, ex)
+    assert big.finish_reason == "capacity" and big.output == []
+    assert ok.output == expected_output(range(6), 4)
+    assert ex.manager.live() == []
+
+
+def test_sliding_window_group_needs_fewer_pages():
+    """With a window of 8 a request of 60 tokens runs in a pool of 5 pages of 4."""
+    ex = FakeExecutor(num_pages=5, page_size=4, window=8)
+    sched = make(ex, max_batched_tokens=4)
+    r = Request("w", list(range(40)), SamplingParams(max_new_tokens=20))
+    sched.add(r)
+    run(sched, ex)
+    assert r.output == expected_output(range(40), 20) and r.preemptions == 0
+    assert ex.manager.groups[0].pool.allocations > 5
+
+
+def test_abort_gives_everything_back():
+    ex = FakeExecutor()
+    sched = make(ex)
+    a = Request("a", list(range(10)), SamplingParams(max_new_tokens=50))
+    b = Request("b", list(range(10)), SamplingParams(max_new_tokens=50))
+    sched.add(a)
+    sched.add(b)
+    for _ in range(3):
+        batch = sched.schedule()
+        sched.update(batch, ex.step(batch))
+    sched.abort("a")
+    assert a.finish_reason == "aborted" and ex.manager.live() == ["b"]
+    sched.abort("b")
+    assert not sched.has_unfinished() and ex.manager.groups[0].pool.num_free == 64 and ex.manager.free_slots == 4
+
+
+def test_seeded_sampling_state_survives_preemption():
+    """The per-request generator is not reset by a preemption: draws continue where they were."""
+    from tuff_amd.sampling.params import SamplerState
+    p = SamplingParams(temp=0.8, seed=11, max_new_tokens=4)
+    r = Request("x", [1, 2], p)
+    ex = FakeExecutor()
+    sched = make(ex)
+    sched.add(r)
+    first = [r.sampler.rng.uniform() for _ in range(2)]
+    sched._preempt_for_test = None
+    fresh = SamplerState(p)
+    assert first == [fresh.rng.uniform() for _ in range(2)]
+    nxt = fresh.rng.uniform()
+    sched.running.append(sched.waiting.popleft())
+    ex.begin("x")
+    sched._preempt(r)
+    assert r.sampler.rng.uniform() == nxt and r.num_computed == 0 and sched.waiting[0] is r
