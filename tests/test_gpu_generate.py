@@ -1,0 +1,189 @@
+"""Generation through the entry points: greedy and seeded temperature sampling of several
+requests at once against the plain implementation, preemption, the command line."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import util
+from plain import lfm2_plain as plain
+from plain.sampler_plain import PlainSampler
+
+pytestmark = pytest.mark.gpu
+
+
+def plain_generate(name, prompt, n, stored, sampler=None):
+    """Token by token with the plain model; returns ids and, for greedy, the top-1/top-2 margins."""
+    cfg, w = util.plain_model(name, stored)
+    ids, out, margins = list(prompt), [], []
+    for _ in range(n):
+        row = plain.forward_logits(cfg, w, ids)[-1]
+        if sampler is None:
+            top = torch.topk(row, 2).values
+            margins.append(float(top[0] - top[1]))
+            t = int(torch.nonzero(row == row.max())[0])
+        else:
+            t = sampler.sample(row.float().numpy())
+            margins.append(None)
+        out.append(t)
+        ids.append(t)
+    return out, margins
+
+
+def agree_up_to_near_ties(got, want, margins, tie):
+    """Equal until the first step at which the plain model's top two logits are closer than `tie`
+    (cf. tools/lfm25_gate.py:54-73: the greedy prefix is cut at the first near-tie)."""
+    for i, (g, w) in enumerate(zip(got, want)):
+        if g != w:
+            assert margins[i] < tie, f"step {i}: got {g}, plain {w}, margin {margins[i]:.2e}"
+            return i
+    return len(want)
+
+
+@pytest.mark.parametrize("dtype,stored,tie", [("float32", "float32", 2e-5), ("bfloat16", "bfloat16", 2e-2)])
+def test_greedy_generation_tiny_a(gpu, dtype, stored, tie):
+    """Tiny A: prompts of 7, 13 and 21 tokens, 16 greedy tokens each, all at once."""
+    from tuff_amd.engine.llm import LLM
+    from tuff_amd.sampling.params import SamplingParams
+    V = util.TINY_A["vocab_size"]
+    prompts = [util.rand_tokens(n, V, 10 + n) for n in (7, 13, 21)]
+    llm = LLM(util.model_folder("A", stored), dtype=dtype, max_num_seqs=4, max_batched_tokens=16, ctx_size=128)
+    outs = llm.generate(prompts, SamplingParams(max_new_tokens=16))
+    total = 0
+    for p, o in zip(prompts, outs):
+        want, margins = plain_generate("A", p, 16, stored)
+        assert len(o.token_ids) == 16 and o.finish_reason == "length"
+        total += agree_up_to_near_ties(o.token_ids, want, margins, tie)
+    assert total >= 24                       # most of the 48 tokens are compared, not cut away by ties
+    assert not llm.engine.manager.live()
+
+
+def test_seeded_temperature_sampling_tiny_b(gpu):
+    """Tiny B: prompts of 1, 5, 33, 64 and 100 tokens; temperature 0.8 with per-request seeds next to
+    greedy requests, in float32, equal to the plain model with the plain sampler."""
+    from tuff_amd.engine.llm import LLM
+    from tuff_amd.sampling.params import SamplingParams
+    V = util.TINY_B["vocab_size"]
+    prompts = [util.rand_tokens(n, V, 20 + n) for n in (1, 5, 33, 64, 100)]
+    params = [SamplingParams(temp=0.8, seed=100 + i, max_new_tokens=12) if i % 2 == 0 else SamplingParams(max_new_tokens=12)
+              for i in range(5)]
+    llm = LLM(util.model_folder("B", "float32"), dtype="float32", max_num_seqs=4, max_batched_tokens=48, ctx_size=160)
+    outs = llm.generate(prompts, params)
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        sampler = PlainSampler(temp=0.8, seed=100 + i) if i % 2 == 0 else None
+        want, margins = plain_generate("B", p, 12, "float32", sampler)
+        if sampler is None:
+            agree_up_to_near_ties(o.token_ids, want, margins, 2e-5)
+        else:
+            assert o.token_ids == want, i
+    # the same seeds again, one request at a time: the stream does not depend on the batch
+    for i in (0, 2):
+        alone = llm.generate([prompts[i]], params[i])[0]
+        assert alone.token_ids == outs[i].token_ids
+
+
+def test_sampling_options_through_the_entry_point(gpu):
+    from tuff_amd.engine.llm import LLM
+    from tuff_amd.sampling.params import SamplingParams
+    V = util.TINY_A["vocab_size"]
+    prompt = util.rand_tokens(9, V, 3)
+    llm = LLM(util.model_folder("A", "float32"), dtype="float32", ctx_size=64)
+    greedy = llm.generate([prompt], SamplingParams(max_new_tokens=8))[0].token_ids
+    top1 = llm.generate([prompt], SamplingParams(temp=3.0, top_k=1, seed=5, max_new_tokens=8))[0].token_ids
+    assert top1 == greedy                                                     # top-k 1 is greedy whatever the draw
+    cold = llm.generate([prompt], SamplingParams(temp=1e-4, seed=5, max_new_tokens=8))[0].token_ids
+    assert cold == greedy                                                     # temperature -> 0+ is greedy
+    p = SamplingParams(temp=1.5, top_k=50, top_p=0.9, min_p=0.01, repeat_penalty=1.3, seed=9, max_new_tokens=10)
+    a = llm.generate([prompt], p)[0].token_ids
+    b = llm.generate([prompt], p)[0].token_ids
+    assert a == b and a != greedy
+    want, _ = plain_generate("A", prompt, 10, "float32",
+                             PlainSampler(temp=1.5, top_k=50, top_p=0.9, min_p=0.01, repeat_penalty=1.3, seed=9))
+    assert a == want
+
+
+def test_preemption_does_not_change_the_output(gpu):
+    """So few pages that running requests are preempted and computed again: same tokens."""
+    from tuff_amd.engine.llm import LLM
+    from tuff_amd.sampling.params import SamplingParams
+    V = util.TINY_A["vocab_size"]
+    prompts = [util.rand_tokens(n, V, 40 + n) for n in (30, 28, 26)]
+    params = [SamplingParams(temp=0.9, seed=7, max_new_tokens=40), SamplingParams(max_new_tokens=40),
+              SamplingParams(temp=0.5, seed=8, max_new_tokens=40)]
+    roomy = LLM(util.model_folder("A", "float32"), dtype="float32", max_num_seqs=4, ctx_size=128)
+    want = [o.token_ids for o in roomy.generate(prompts, params)]
+    assert roomy.last_stats["preemptions"] == 0
+    tight = LLM(util.model_folder("A", "float32"), dtype="float32", max_num_seqs=4, ctx_size=128, num_pages=9)
+    outs = tight.generate(prompts, params)
+    assert tight.last_stats["preemptions"] >= 1
+    assert [o.token_ids for o in outs] == want
+    assert sum(o.preemptions for o in outs) == tight.last_stats["preemptions"]
+    tight.engine.manager.check()
+    assert not tight.engine.manager.live()
+
+
+def test_eos_stops_a_request(gpu):
+    from tuff_amd.engine.llm import LLM
+    from tuff_amd.sampling.params import SamplingParams
+    V = util.TINY_A["vocab_size"]
+    prompt = util.rand_tokens(11, V, 9)
+    llm = LLM(util.model_folder("A", "float32"), dtype="float32", ctx_size=64)
+    free = llm.generate([prompt], SamplingParams(max_new_tokens=10))[0].token_ids
+    llm.engine.model.eos_token_id = free[3]
+    out = llm.generate([prompt], SamplingParams(max_new_tokens=10))[0]
+    cut = free.index(free[3]) + 1
+    assert out.token_ids == free[:cut] and out.finish_reason == "stop"
+    out = llm.generate([prompt], SamplingParams(max_new_tokens=10, ignore_eos=True))[0]
+    assert out.token_ids == free and out.finish_reason == "length"
+
+
+def _tuff(*args):
+    return subprocess.run([sys.executable, os.path.join(util.ROOT, "bin", "tuff"), *args],
+                          capture_output=True, text=True, timeout=300)
+
+
+def test_command_line(gpu, tmp_path):
+    folder = util.model_folder("A", "float32")
+    prompt = util.rand_tokens(9, util.TINY_A["vocab_size"], 3)
+    ids = ",".join(map(str, prompt))
+    want, margins = plain_generate("A", prompt, 12, "float32")
+    # --dump-tokens: ids on stdout, one a line
+    p = _tuff("--model", folder, "--prompt-ids", ids, "--dump-tokens", "-n", "12", "--dtype", "fp32")
+    assert p.returncode == 0, p.stderr
+    got = [int(x) for x in p.stdout.split()]
+    assert agree_up_to_near_ties(got, want, margins, 2e-5) == 12
+    # prompt from a file, fed in portions of 4: same tokens
+    f = tmp_path / "p.txt"
+    f.write_text(" ".join(map(str, prompt)))
+    p2 = _tuff("--model", folder, "--prompt-ids", str(f), "--dump-tokens", "-n", "12", "--dtype", "fp32", "--prefill-batch", "4")
+    assert p2.returncode == 0 and p2.stdout == p.stdout
+    # --teacher-force with --dump-logits: agreement 12/12 and the file holds the plain logits
+    ref = tmp_path / "ref.txt"
+    ref.write_text("\n".join(map(str, got)))
+    out = tmp_path / "logits.bin"
+    p3 = _tuff("--model", folder, "--prompt-ids", ids, "--teacher-force", str(ref), "--dump-logits", str(out),
+               "--tf-batch", "4", "-n", "12", "--dtype", "fp32")
+    assert p3.returncode == 0, p3.stderr
+    assert "12/12" in p3.stderr
+    raw = out.read_bytes()
+    assert raw[:8] == b"CLBRLGT1"
+    n, V = np.frombuffer(raw[8:16], dtype="<u4")
+    assert (n, V) == (12, 512)
+    rows = torch.from_numpy(np.frombuffer(raw[16:], dtype="<f4").reshape(12, 512).copy())
+    full = util.plain_logits("A", prompt + got[:-1], "float32")[len(prompt) - 1:]
+    util.assert_close_f32(rows, full, "teacher-forced logits")
+    # a wrong reference is reported with exit code 1
+    ref.write_text("\n".join(map(str, [got[0], (got[1] + 1) % 512] + got[2:])))
+    p4 = _tuff("--model", folder, "--prompt-ids", ids, "--teacher-force", str(ref), "-n", "12", "--dtype", "fp32")
+    assert p4.returncode == 1 and "top-1 agreement" in p4.stderr and "12/12" not in p4.stderr
+    # timed mode prints the speed line; usage errors give 2; a broken model gives 1
+    p5 = _tuff("--model", folder, "--prompt-ids", ids, "-n", "8", "--warmup", "2", "--runs", "2")
+    assert p5.returncode == 0 and "Pipeline Generation Speed" in p5.stdout, p5.stderr
+    assert _tuff("--model", folder).returncode == 2
+    assert _tuff("--model", folder, "--prompt-ids", ids, "-n", "5000").returncode == 2
+    assert _tuff("--model", str(tmp_path), "--prompt-ids", ids).returncode == 1
+    assert _tuff("--model", folder, "--inspect").returncode == 0

@@ -1,0 +1,303 @@
+"""Each part alone on the GPU against its plain counterpart, at sizes of its own, and a toy
+mixer with state of its own that is registered, built and stepped from this file."""
+import dataclasses
+import math
+from typing import ClassVar
+
+import pytest
+import torch
+
+import util
+from plain import lfm2_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+
+def _r(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * scale
+
+
+class Harness:
+    """Runs one mixer (or any callable taking h, ctx, cache, residual) over requests cut into steps."""
+
+    def __init__(self, gpu, dtype, cache_spec, page_size=16, pages=64):
+        from tuff_amd.cache.manager import CacheLayout, CacheManager
+        from tuff_amd.cache.storage import CacheStorage
+        from tuff_amd.parts.base import Runtime
+        self.gpu, self.dtype = gpu, dtype
+        self.rt = Runtime(gpu, dtype)
+        self.mgr = CacheManager(CacheLayout.from_specs({0: cache_spec}), page_size, pages, 4)
+        self.storage = CacheStorage(self.mgr, dtype, gpu, poison=True)
+
+    def run(self, forward, inputs: dict, cuts: dict, d_out: int):
+        """inputs: {rid: [n, d] float tensor}; cuts: {rid: [portion sizes]}; all requests advance together."""
+        from tuff_amd.engine.batch import StepEntry, build_context
+        done = {rid: 0 for rid in inputs}
+        outs = {rid: [] for rid in inputs}
+        for rid in inputs:
+            slot = self.mgr.admit(rid)
+            self.storage.zero_slot(slot)
+        step = 0
+        while any(done[r] < inputs[r].shape[0] for r in inputs):
+            entries, rows = [], []
+            for rid, x in inputs.items():
+                if step < len(cuts[rid]):
+                    n = cuts[rid][step]
+                    self.mgr.extend(rid, n)
+                    entries.append(StepEntry(rid, [0] * n, []))
+                    rows.append(x[done[rid]:done[rid] + n])
+            ctx = build_context(entries, self.mgr, self.gpu, 1)
+            h = torch.cat(rows).to(self.gpu, self.dtype).contiguous()
+            residual = torch.zeros(h.shape[0], d_out, device=self.gpu)
+            forward(h, ctx, self.storage.views.get(0), residual)
+            t = 0
+            for e in entries:
+                outs[e.req_id].append(residual[t:t + len(e.tokens)].cpu())
+                done[e.req_id] += len(e.tokens)
+                t += len(e.tokens)
+            step += 1
+        return {rid: torch.cat(v).double() for rid, v in outs.items()}
+
+
+def tol(dtype):
+    return 2e-5 if dtype == torch.float32 else 3e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("d,H,Hkv,hd,window,theta", [(48, 3, 1, 16, None, 1e4), (80, 2, 2, 40, 21, 1e6), (64, 8, 2, 8, None, 50.0)])
+def test_attention_mixer_alone(gpu, dtype, d, H, Hkv, hd, window, theta):
+    from tuff_amd.parts.attention import AttentionMixer
+    from tuff_amd.parts.rope import Rotary
+    names = {k: k for k in ("q", "k", "v", "o", "q_norm", "k_norm")}
+    mixer = AttentionMixer(d, H, Hkv, hd, names=names, qk_norm_eps=1e-6, position=Rotary(hd, theta), window=window)
+    w = {"q": _r(H * hd, d, seed=1, scale=0.3), "k": _r(Hkv * hd, d, seed=2, scale=0.3), "v": _r(Hkv * hd, d, seed=3, scale=0.3),
+         "o": _r(d, H * hd, seed=4, scale=0.3), "q_norm": 1 + _r(hd, seed=5, scale=0.1), "k_norm": 1 + _r(hd, seed=6, scale=0.1)}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    hs = Harness(gpu, dtype, mixer.cache_spec())
+    mixer.bind({k: v.to(gpu) for k, v in w.items()}, hs.rt)
+    inputs = {"a": _r(70, d, seed=7).to(dtype).float(), "b": _r(37, d, seed=8).to(dtype).float()}
+    got = hs.run(mixer.forward, inputs, {"a": [33, 1, 1, 30, 5], "b": [2, 20, 15]}, d)
+    wd = {k: v.double() for k, v in w.items()}
+    for rid, x in inputs.items():
+        want = plain.attention(x.double(), wd["q"], wd["k"], wd["v"], wd["o"], wd["q_norm"], wd["k_norm"],
+                               n_head=H, n_kv=Hkv, eps=1e-6, base=theta)
+        if window:                       # the plain function is full attention: redo it with the window
+            T = x.shape[0]
+            pos = torch.arange(T)
+            q = plain.rope_neox(plain.rms_norm((x.double() @ wd["q"].T).reshape(T, H, hd), wd["q_norm"], 1e-6), pos, theta)
+            k = plain.rope_neox(plain.rms_norm((x.double() @ wd["k"].T).reshape(T, Hkv, hd), wd["k_norm"], 1e-6), pos, theta)
+            v = (x.double() @ wd["v"].T).reshape(T, Hkv, hd)
+            k, v = k.repeat_interleave(H // Hkv, 1), v.repeat_interleave(H // Hkv, 1)
+            s = torch.einsum("thd,shd->hts", q, k) / math.sqrt(hd)
+            i, j = torch.arange(T)[:, None], torch.arange(T)[None, :]
+            s = s.masked_fill(~((j <= i) & (j > i - window)), float("-inf"))
+            want = torch.einsum("hts,shd->thd", torch.softmax(s, -1), v).reshape(T, H * hd) @ wd["o"].T
+        assert (got[rid] - want).abs().max() <= tol(dtype) * float(want.abs().max()), rid
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_mixer_without_norm_or_position_is_plain_attention(gpu, dtype):
+    """No rotation, no norm, one head: the library's causal attention."""
+    from tuff_amd.parts.attention import AttentionMixer
+    d = hd = 32
+    mixer = AttentionMixer(d, 1, 1, hd, names={k: k for k in "qkvo"})
+    w = {k: _r(d, d, seed=i, scale=0.2).to(dtype) for i, k in enumerate("qkvo")}
+    hs = Harness(gpu, dtype, mixer.cache_spec())
+    mixer.bind({k: v.to(gpu) for k, v in w.items()}, hs.rt)
+    x = _r(50, d, seed=9).to(dtype).float()
+    got = hs.run(mixer.forward, {"a": x}, {"a": [17, 33]}, d)["a"]
+    xd = x.double()
+    q, k, v = (xd @ w[n].double().T for n in "qkv")
+    o = torch.nn.functional.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)[0]
+    want = o @ w["o"].double().T
+    assert (got - want).abs().max() <= tol(dtype) * float(want.abs().max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("d,K", [(40, 3), (72, 5)])
+def test_shortconv_mixer_alone(gpu, dtype, d, K):
+    from tuff_amd.parts.shortconv import ShortConvMixer
+    mixer = ShortConvMixer(d, K, names={"in_proj": "i", "conv": "c", "out_proj": "o"})
+    w = {"i": _r(3 * d, d, seed=1, scale=0.3).to(dtype), "c": _r(d, K, seed=2, scale=0.5).to(dtype),
+         "o": _r(d, d, seed=3, scale=0.3).to(dtype)}
+    hs = Harness(gpu, dtype, mixer.cache_spec())
+    mixer.bind({k: v.to(gpu) for k, v in w.items()}, hs.rt)
+    inputs = {"a": _r(30, d, seed=4).to(dtype).float(), "b": _r(9, d, seed=5).to(dtype).float()}
+    got = hs.run(mixer.forward, inputs, {"a": [1, 1, 20, 2, 6], "b": [5, 1, 3]}, d)
+    for rid, x in inputs.items():
+        want = plain.short_conv(x.double(), w["i"].double(), w["c"].double(), w["o"].double())
+        assert (got[rid] - want).abs().max() <= tol(dtype) * float(want.abs().max()), rid
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu_norm_and_block_alone(gpu, dtype):
+    from tuff_amd.parts.base import Runtime
+    from tuff_amd.parts.block import PreNormBlock
+    from tuff_amd.parts.ffn import SwiGLU
+    from tuff_amd.parts.norm import RMSNorm
+    from tuff_amd.parts.shortconv import ShortConvMixer
+    d, F, K, eps = 56, 104, 3, 1e-4
+    rt = Runtime(gpu, dtype)
+    w = {"g": _r(F, d, seed=1, scale=0.3), "u": _r(F, d, seed=2, scale=0.3), "dn": _r(d, F, seed=3, scale=0.3),
+         "n1": 1 + _r(d, seed=4, scale=0.1), "n2": 1 + _r(d, seed=5, scale=0.1),
+         "i": _r(3 * d, d, seed=6, scale=0.3), "c": _r(d, K, seed=7, scale=0.5), "o": _r(d, d, seed=8, scale=0.3)}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    wg = {k: v.to(gpu) for k, v in w.items()}
+    wd = {k: v.double() for k, v in w.items()}
+    x = _r(13, d, seed=9)
+    # norm
+    norm = RMSNorm(d, eps, "n1")
+    norm.bind(wg, rt)
+    h = norm.forward(x.to(gpu))
+    want_h = plain.rms_norm(x.double(), wd["n1"], eps)
+    assert h.dtype == dtype and (h.cpu().double() - want_h).abs().max() <= tol(dtype) * float(want_h.abs().max())
+    # feed-forward
+    ffn = SwiGLU(d, F, names={"gate": "g", "up": "u", "down": "dn"})
+    ffn.bind(wg, rt)
+    res = x.to(gpu).clone()
+    ffn.forward(h, None, res)
+    want = x.double() + plain.swiglu(h.cpu().double(), wd["g"], wd["u"], wd["dn"])
+    assert (res.cpu().double() - want).abs().max() <= tol(dtype) * float(want.abs().max())
+    # the block: x += mixer(norm1 x); x += ffn(norm2 x)
+    block = PreNormBlock(RMSNorm(d, eps, "n1"), ShortConvMixer(d, K, names={"in_proj": "i", "conv": "c", "out_proj": "o"}),
+                         RMSNorm(d, eps, "n2"), SwiGLU(d, F, names={"gate": "g", "up": "u", "down": "dn"}))
+    assert sorted(dd.name for dd in block.weight_decls()) == sorted(w)
+    hs = Harness(gpu, dtype, block.mixer.cache_spec())
+    block.bind(wg, hs.rt)
+
+    def fwd(h_in, ctx, cache, residual):
+        residual.copy_(h_in.float())
+        block.forward(residual, ctx, cache)
+    got = hs.run(fwd, {"a": x.to(dtype).float()}, {"a": [4, 9]}, d)["a"]
+    xd = x.to(dtype).double()
+    y = xd + plain.short_conv(plain.rms_norm(xd, wd["n1"], eps), wd["i"], wd["c"], wd["o"])
+    y = y + plain.swiglu(plain.rms_norm(y, wd["n2"], eps), wd["g"], wd["u"], wd["dn"])
+    assert (got - y).abs().max() <= tol(dtype) * float(y.abs().max())
+
+
+def test_position_encoding_of_its_own_goes_through_apply(gpu):
+    """A position encoding that is not rotary: the mixer norms, calls apply(), then writes the cache."""
+    from tuff_amd.parts.attention import AttentionMixer
+    from tuff_amd.parts.base import PositionEncoding
+
+    class SignFlip(PositionEncoding):
+        """Negates q and k at odd positions (q.k of two odd or two even positions is unchanged)."""
+        calls = 0
+
+        def apply(self, q, k, positions):
+            SignFlip.calls += 1
+            sign = (1 - 2 * (positions % 2)).to(q.dtype)[:, None]
+            q.mul_(sign)
+            k.mul_(sign)
+    d = hd = 16
+    w = {k: _r(d, d, seed=i, scale=0.4) for i, k in enumerate("qkvo")}
+    x = _r(12, d, seed=5)
+    outs = []
+    for pos in (SignFlip(), None):
+        mixer = AttentionMixer(d, 1, 1, hd, names={k: k for k in "qkvo"}, position=pos)
+        hs = Harness(gpu, torch.float32, mixer.cache_spec())
+        mixer.bind({k: v.to(gpu) for k, v in w.items()}, hs.rt)
+        outs.append(hs.run(mixer.forward, {"a": x}, {"a": [5, 7]}, d)["a"])
+    assert SignFlip.calls == 2
+    xd = x.double()
+    q, k, v = (xd @ w[n].double().T for n in "qkv")
+    sign = (1 - 2 * (torch.arange(12) % 2)).double()[:, None]
+    o = torch.nn.functional.scaled_dot_product_attention((q * sign)[None], (k * sign)[None], v[None], is_causal=True)[0]
+    assert (outs[0] - o @ w["o"].double().T).abs().max() < 1e-5
+    assert (outs[0] - outs[1]).abs().max() > 1e-3
+
+
+# ---------------------------------------------------------------------- a toy mixer
+def test_toy_mixer_with_state_is_registered_built_and_stepped(gpu):
+    """A leaky running sum s_t = a * s_{t-1} + h_t (state [d] per request), out = W s_t, defined
+    here, put into an architecture of its own, run through Engine.step in different cuttings."""
+    from tuff_amd.config.base import ModelConfig
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.models import registry
+    from tuff_amd.models.decoder import DecoderModel
+    from tuff_amd.parts.base import MIXERS, FixedState, Mixer, WeightDecl
+    from tuff_amd.parts.block import PreNormBlock
+    from tuff_amd.parts.ffn import SwiGLU
+    from tuff_amd.parts.norm import RMSNorm
+
+    class LeakySum(Mixer):
+        def __init__(self, d, decay, name):
+            self.d, self.decay, self.name = d, decay, name
+
+        def weight_decls(self):
+            return [WeightDecl(self.name, (self.d, self.d))]
+
+        def cache_spec(self):
+            return FixedState((self.d,))
+
+        def bind(self, weights, rt):
+            self.rt, self.w = rt, weights[self.name].float()
+
+        def forward(self, h, ctx, cache, residual, write_cache=True):
+            hf = h.float()
+            slots = ctx.state_slot.tolist()
+            t = 0
+            for r, n in enumerate(ctx.host["q_len"].tolist()):
+                s = cache.state[slots[r]].clone()
+                for i in range(n):
+                    s = self.decay * s + hf[t + i]
+                    residual[t + i] += s @ self.w.T
+                if write_cache:
+                    cache.state[slots[r]] = s
+                t += n
+
+    @dataclasses.dataclass
+    class ToyConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyLeakyForCausalLM"
+        vocab_size: int
+        hidden_size: int
+        num_hidden_layers: int
+        decay: float
+        ffn: int
+
+    def build(cfg):
+        blocks = [PreNormBlock(RMSNorm(cfg.hidden_size, 1e-5, f"l{i}.n1"),
+                               MIXERS.get("leaky_sum")(cfg.hidden_size, cfg.decay, f"l{i}.mix"),
+                               RMSNorm(cfg.hidden_size, 1e-5, f"l{i}.n2"),
+                               SwiGLU(cfg.hidden_size, cfg.ffn, names={"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"}))
+                  for i in range(cfg.num_hidden_layers)]
+        return DecoderModel(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size,
+                            embedding=WeightDecl("emb", (cfg.vocab_size, cfg.hidden_size)), blocks=blocks,
+                            final_norm=RMSNorm(cfg.hidden_size, 1e-5, "fn"))
+
+    MIXERS.register("leaky_sum", LeakySum)
+    registry.register_architecture("ToyLeakyForCausalLM", ToyConfig, build)
+    try:
+        cfg = registry.config_from_dict({"architectures": ["ToyLeakyForCausalLM"], "vocab_size": 97, "hidden_size": 24,
+                                         "num_hidden_layers": 2, "decay": 0.7, "ffn": 40})
+        from tuff_amd.weights.random_init import random_weights
+        model = registry.build_model(cfg)
+        w32 = random_weights(model.weight_decls(), 3, torch.float32, "cpu")
+        eng = Engine(model, {k: v.to(gpu) for k, v in w32.items()}, dtype="float32", max_tokens=256)
+        assert eng.layout.states and not eng.layout.paged
+        reqs = {"a": util.rand_tokens(19, 97, 1), "b": util.rand_tokens(8, 97, 2)}
+        whole = util.run_plan(eng, util.plan_whole(reqs))
+        single = util.run_plan(eng, util.plan_tail(reqs, 100))
+        mixed = util.run_plan(eng, util.plan_mixed(reqs, seed=1, decode_tail=3))
+        for rid in reqs:
+            assert (whole[rid] - single[rid]).abs().max() < 1e-5
+            assert (whole[rid] - mixed[rid]).abs().max() < 1e-5
+        # against a plain loop over the same weights
+        w = {k: v.double() for k, v in w32.items()}
+        for rid, toks in reqs.items():
+            x = w["emb"][toks]
+            for i in range(2):
+                h = plain.rms_norm(x, w[f"l{i}.n1"], 1e-5)
+                s = torch.zeros(24, dtype=torch.float64)
+                rows = []
+                for t in range(h.shape[0]):
+                    s = 0.7 * s + h[t]
+                    rows.append(s @ w[f"l{i}.mix"].T)
+                x = x + torch.stack(rows)
+                x = x + plain.swiglu(plain.rms_norm(x, w[f"l{i}.n2"], 1e-5), w[f"l{i}.g"], w[f"l{i}.u"], w[f"l{i}.d"])
+            want = plain.rms_norm(x, w["fn"], 1e-5) @ w["emb"].T
+            util.assert_close_f32(whole[rid], want, rid)
+    finally:
+        MIXERS.unregister("leaky_sum")
+        registry.unregister_architecture("ToyLeakyForCausalLM")
