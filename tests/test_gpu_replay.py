@@ -141,3 +141,45 @@ def test_out_of_pages_leaves_everything_as_it_was(gpu):
     eng.manager.check()
     eng.step([StepEntry("a", [1], [0]), StepEntry("b", list(range(10)), [9])])
     eng.manager.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_decode_steps_equal_eager_steps(gpu, dtype):
+    """Steps of single tokens are recorded into a graph and replayed.  Every replay, with eager
+    steps of other shapes and synchronisations in between, gives exactly what an engine without
+    graphs gives; a context that outgrows the recorded table width gets a new recording."""
+    name = "A"
+    V = util.TINY_A["vocab_size"]
+    reqs = {"x": util.rand_tokens(1050, V, 1), "y": util.rand_tokens(120, V, 2), "z": util.rand_tokens(40, V, 3)}
+    steps = []
+    def add(entries, end=()):
+        steps.append({"step": len(steps), "entries": entries, "end": list(end)})
+    fed = {k: 0 for k in reqs}
+    def portion(rid, n):
+        t = reqs[rid][fed[rid]:fed[rid] + n]
+        fed[rid] += n
+        return {"id": rid, "tokens": t, "want": [len(t) - 1]}
+    add([portion("x", 1000), portion("y", 50)])
+    for i in range(45):
+        if i == 10:
+            add([portion("z", 20)])                                  # an eager step of another shape in between
+        if i == 20:
+            add([portion("x", 1), portion("y", 1), portion("z", 5)])  # mixed: not recorded
+        add([portion("x", 1), portion("y", 1)] + ([portion("z", 1)] if 12 <= i < 20 else []))
+    add([portion("x", 1)], end=["x", "y", "z"])
+    assert fed["x"] > 1024                                            # x crossed the 64-block table width
+    eager = make_engine(name, dtype, max_tokens=2048, use_graphs=False)
+    want = util.run_plan(eager, steps)
+    eng = make_engine(name, dtype, max_tokens=2048)
+    assert eng.use_graphs
+    got = util.run_plan(eng, steps)
+    assert eng.graph_replays >= 30 and len(eng._graphs) >= 3
+    assert eager.graph_replays == 0
+    for rid in reqs:
+        a, b = got[rid], want[rid]
+        mask = ~torch.isnan(b[:, 0])
+        assert torch.equal(torch.isnan(a[:, 0]), torch.isnan(b[:, 0]))
+        assert torch.equal(a[mask], b[mask]), rid
+    full = util.plain_logits(name, reqs["y"][:fed["y"]], stored_for(dtype))
+    mask = ~torch.isnan(got["y"][:, 0])
+    util.assert_close(dtype, got["y"][mask], full[mask], "y")

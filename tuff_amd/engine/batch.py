@@ -1,11 +1,13 @@
 """The description of one step as the kernels read it: a flat list of tokens with, per token,
 its position and request, and, per request, where its tokens start, its state slot and its
-block tables.  Everything goes to the device in one copy.
+block tables.  Everything is packed into one int32 buffer and goes to the device in one copy;
+the device tensors are views into that buffer, so a recorded graph can be replayed after the
+buffer alone was refreshed.
 """
 from __future__ import annotations
 
 import dataclasses
-from typing import Hashable, Sequence
+from typing import Hashable, Optional, Sequence
 
 import numpy as np
 import torch
@@ -41,28 +43,51 @@ class StepContext:
     groups: list[GroupContext]
     # host-side facts kernels may be chosen by
     max_q_len: int = 1
-    max_ctx_len: int = 1
-    host: dict = dataclasses.field(default_factory=dict)
+    max_ctx_len: int = 1           # an upper bound of every position + 1 of the step
+    host: dict = dataclasses.field(default_factory=dict)     # 'q_len', 'ctx_len' (numpy) and what parts cache
 
 
-def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int) -> StepContext:
-    """`manager` has already been extended by every entry's tokens."""
+@dataclasses.dataclass
+class PackedStep:
+    """A step on the host: the int32 buffer and where its pieces lie."""
+    buf: np.ndarray
+    offs: np.ndarray
+    T: int
+    R: int
+    n_logits: int
+    n_groups: int
+    max_blocks: int
+    max_q_len: int
+    max_ctx_len: int
+    q_len: np.ndarray
+    ctx_len: np.ndarray
+
+    def shape_key(self):
+        return (self.T, self.R, self.n_logits, self.n_groups, self.max_blocks)
+
+
+def pack_step(entries: Sequence[StepEntry], manager, vocab_size: int,
+              max_blocks: Optional[int] = None) -> PackedStep:
+    """`manager` has already been extended by every entry's tokens.  max_blocks: width of the
+    block tables (default: the longest table of the step)."""
     R = len(entries)
     T = sum(len(e.tokens) for e in entries)
     n_groups = len(manager.groups)
-    max_blocks = max(1, max(len(manager.block_table(e.req_id, g)) for e in entries for g in range(n_groups))
-                     if n_groups else 1)
+    longest = max([len(manager.block_table(e.req_id, g)) for e in entries for g in range(n_groups)] + [1])
+    if max_blocks is None:
+        max_blocks = longest
+    elif max_blocks < longest:
+        raise ValueError(f"block tables need {longest} entries, {max_blocks} given")
     n_logits = sum(len(e.want) for e in entries)
     ps = manager.page_size
-    # one int32 buffer: [tokens | positions | req_of_token | q_start | q_len | ctx_len | slot |
-    #                    logit_rows | per group: slot_mapping, block_table]
+    # [tokens | positions | req_of_token | q_start | q_len | ctx_len | slot | logit_rows |
+    #  per group: slot_mapping, block_table]
     sizes = [T, T, T, R, R, R, R, n_logits] + [T, R * max_blocks] * n_groups
     offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
     buf = np.zeros(int(offs[-1]), dtype=np.int32)
     tokens, positions, req_of = (buf[offs[i]:offs[i + 1]] for i in range(3))
     q_start, q_len, ctx_len, slot, rows = (buf[offs[i]:offs[i + 1]] for i in range(3, 8))
-    t = 0
-    li = 0
+    t = li = 0
     max_q = max_ctx = 1
     for r, e in enumerate(entries):
         n = len(e.tokens)
@@ -93,12 +118,24 @@ def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int
             sm[t:t + n] = pages * ps + pos % ps
         t += n
         max_q, max_ctx = max(max_q, n), max(max_ctx, total)
-    host = torch.from_numpy(buf)
-    dev = host.pin_memory().to(device, non_blocking=True) if buf.size else host.to(device)
+    return PackedStep(buf, offs, T, R, n_logits, n_groups, max_blocks, max_q, max_ctx, q_len.copy(), ctx_len.copy())
+
+
+def context_on(dev: torch.Tensor, p: PackedStep, max_ctx_len: Optional[int] = None) -> StepContext:
+    """Views of the device buffer `dev` (same layout as p.buf) as a StepContext."""
+    offs = p.offs
     sl = lambda i: dev[int(offs[i]):int(offs[i + 1])]
-    groups = [GroupContext(block_table=sl(9 + 2 * g).view(R, max_blocks), slot_mapping=sl(8 + 2 * g))
-              for g in range(n_groups)]
-    return StepContext(T=T, R=R, n_logits=n_logits, tokens=sl(0), positions=sl(1), req_of_token=sl(2),
+    groups = [GroupContext(block_table=sl(9 + 2 * g).view(p.R, p.max_blocks), slot_mapping=sl(8 + 2 * g))
+              for g in range(p.n_groups)]
+    return StepContext(T=p.T, R=p.R, n_logits=p.n_logits, tokens=sl(0), positions=sl(1), req_of_token=sl(2),
                        q_start=sl(3), q_len=sl(4), ctx_len=sl(5), state_slot=sl(6), logit_rows=sl(7),
-                       groups=groups, max_q_len=max_q, max_ctx_len=max_ctx,
-                       host={"q_len": q_len.copy(), "ctx_len": ctx_len.copy()})
+                       groups=groups, max_q_len=p.max_q_len,
+                       max_ctx_len=max_ctx_len if max_ctx_len is not None else p.max_ctx_len,
+                       host={"q_len": p.q_len, "ctx_len": p.ctx_len})
+
+
+def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int) -> StepContext:
+    p = pack_step(entries, manager, vocab_size)
+    host = torch.from_numpy(p.buf)
+    dev = host.pin_memory().to(device, non_blocking=True) if p.buf.size else host.to(device)
+    return context_on(dev, p)

@@ -21,7 +21,7 @@ from ..models.registry import build_model, load_config
 from ..parts.base import Runtime
 from ..weights.loader import load_weights
 from ..weights.random_init import random_weights
-from .batch import StepContext, StepEntry, build_context
+from .batch import StepContext, StepEntry, build_context, context_on, pack_step
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
            "fp32": torch.float32, "f32": torch.float32}
@@ -46,7 +46,8 @@ def require_gpu(device="cuda:0") -> torch.device:
 
 class Engine:
     def __init__(self, model, weights: dict, *, dtype, device="cuda:0", page_size: int = 16,
-                 max_tokens: int = 8192, max_requests: int = 8, num_pages=None, poison_cache: bool = False):
+                 max_tokens: int = 8192, max_requests: int = 8, num_pages=None, poison_cache: bool = False,
+                 use_graphs: bool = True):
         """max_tokens: tokens the page pool of each cache group holds (rounded up to whole
         pages).  max_requests: state slots, i.e. requests that can be live at a time."""
         self.device = require_gpu(device)
@@ -63,6 +64,10 @@ class Engine:
         self.manager = CacheManager(self.layout, self.page_size, num_pages, int(max_requests))
         self.storage = CacheStorage(self.manager, self.dtype, self.device, poison=poison_cache)
         self.steps = 0
+        # steps of single decoded tokens are recorded into graphs, one per (batch size, table width)
+        self.use_graphs = bool(use_graphs) and model.graph_safe()
+        self._graphs: dict = {}
+        self.graph_replays = 0
 
     # ---------------------------------------------------------------- construction
     @classmethod
@@ -131,7 +136,70 @@ class Engine:
             for e in done:
                 self.manager.truncate(e.req_id, self.manager.length(e.req_id) - len(e.tokens))
             raise
-        ctx = build_context(entries, self.manager, self.device, self.model.vocab_size)
-        logits = self.model.forward(ctx, self.storage.views)
         self.steps += 1
-        return logits
+        if self.use_graphs and all(len(e.tokens) == 1 for e in entries):
+            return self._decode_step(entries)
+        ctx = build_context(entries, self.manager, self.device, self.model.vocab_size)
+        return self.model.forward(ctx, self.storage.views)
+
+    # --------------------------------------------------------------- recorded decode
+    GRAPH_TABLE_BUCKET = 64          # block tables of recorded steps are padded to multiples of this
+    MAX_GRAPHS = 12
+
+    def _decode_step(self, entries) -> Optional[torch.Tensor]:
+        """A step of single tokens.  The first step of a shape runs eagerly on persistent
+        buffers and is then recorded; later steps of that shape refresh the buffer and replay.
+        Everything a kernel's launch depends on (batch size, table width, number of key
+        partitions) is part of the shape; positions, tokens, tables and slots are data."""
+        longest = max([len(self.manager.block_table(e.req_id, g)) for e in entries
+                       for g in range(len(self.manager.groups))] + [1])
+        width = -(-longest // self.GRAPH_TABLE_BUCKET) * self.GRAPH_TABLE_BUCKET
+        p = pack_step(entries, self.manager, self.model.vocab_size, max_blocks=width)
+        key = p.shape_key()
+        g = self._graphs.get(key)
+        if g is None:
+            if len(self._graphs) >= self.MAX_GRAPHS:
+                self._graphs.pop(next(iter(self._graphs)))
+            g = _RecordedStep(p, self.device, width * self.page_size)
+            self._graphs[key] = g
+            g.refresh(p)
+            logits = self.model.forward(g.ctx, self.storage.views)
+            try:
+                g.record(lambda: self.model.forward(g.ctx, self.storage.views))
+            except Exception as e:                         # noqa: BLE001 - recording is an optimisation
+                import sys
+                print(f"[tuff_amd] recording the decode step failed ({type(e).__name__}: {e}); "
+                      f"continuing without graphs", file=sys.stderr)
+                self.use_graphs = False
+                self._graphs.clear()
+            return logits
+        self._graphs[key] = self._graphs.pop(key)           # most recently used last
+        g.refresh(p)
+        g.graph.replay()
+        self.graph_replays += 1
+        return g.logits
+
+
+class _RecordedStep:
+    """Persistent buffers of one step shape and the graph recorded over them."""
+
+    def __init__(self, p, device, max_ctx_len: int):
+        self.pinned = torch.empty(p.buf.size, dtype=torch.int32, pin_memory=True)
+        self.dev = torch.empty(p.buf.size, dtype=torch.int32, device=device)
+        self.ctx = context_on(self.dev, p, max_ctx_len=max_ctx_len)
+        self.copied = torch.cuda.Event()
+        self.graph = None
+        self.logits = None
+
+    def refresh(self, p) -> None:
+        self.copied.synchronize()                           # the last copy out of `pinned` is done
+        self.pinned.numpy()[:] = p.buf
+        self.dev.copy_(self.pinned, non_blocking=True)
+        self.copied.record()
+
+    def record(self, forward) -> None:
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.logits = forward()
+        self.graph = graph

@@ -87,6 +87,9 @@ class DecoderModel:
         mods += self.final_norm.kernel_modules()
         return sorted(set(mods))
 
+    def graph_safe(self) -> bool:
+        return all(b.graph_safe for b in self.blocks) and self.final_norm.graph_safe
+
     def num_parameters(self) -> int:
         n = 0
         for d in self.weight_decls():

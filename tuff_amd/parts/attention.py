@@ -43,6 +43,10 @@ class AttentionMixer(Mixer):
         self._al = al
         self.q_norm_w = self.k_norm_w = None
 
+    @property
+    def graph_safe(self):
+        return self.position is None or self.position.graph_safe
+
     def weight_decls(self):
         decls = self.qkv.weight_decls() + self.out.weight_decls()
         if self.eps is not None:

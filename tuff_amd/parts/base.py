@@ -64,6 +64,10 @@ class Part:
         """Kernel libraries (names of tuff_amd.csrc.build.MODULES) this part launches."""
         return []
 
+    #: True if forward() only launches kernels on the current stream and reads nothing back to
+    #: the host, so that a step through this part can be recorded into a graph and replayed.
+    graph_safe = False
+
 
 class Norm(Part):
     """forward(x float32 [T, d], rows=None) -> [T or len(rows), d] in the compute dtype."""

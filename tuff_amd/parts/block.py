@@ -22,6 +22,10 @@ class PreNormBlock(Block):
     def _parts(self):
         return [p for p in (self.norm1, self.mixer, self.norm2, self.ffn) if p is not None]
 
+    @property
+    def graph_safe(self):
+        return all(p.graph_safe for p in self._parts())
+
     def weight_decls(self):
         return [d for p in self._parts() for d in p.weight_decls()]
 

@@ -10,6 +10,8 @@ from .linear import Linear
 
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, ffn_dim: int, *, names: dict[str, str],
                  aliases: dict[str, tuple] | None = None):
         """names: checkpoint names of 'gate' [F, d], 'up' [F, d], 'down' [d, F]."""

@@ -11,6 +11,8 @@ from .base import NORMS, Norm, Runtime, WeightDecl
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, dim: int, eps: float, name: str, aliases: tuple = ()):
         self.dim, self.eps, self.name, self.aliases = int(dim), float(eps), name, tuple(aliases)
         self.weight: Optional[torch.Tensor] = None

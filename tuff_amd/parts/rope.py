@@ -14,6 +14,8 @@ from .base import POSITION_ENCODINGS, PositionEncoding, Runtime
 
 @POSITION_ENCODINGS.register("rotary")
 class Rotary(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, head_dim: int, base: float, rotary_dim: Optional[int] = None,
                  interleaved: bool = False):
         self.head_dim, self.base = int(head_dim), float(base)

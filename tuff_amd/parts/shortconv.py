@@ -18,6 +18,8 @@ MAX_KERNEL = 17      # the state kernel keeps K-1 <= 16 rows in registers
 
 @MIXERS.register("shortconv")
 class ShortConvMixer(Mixer):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, kernel_size: int, *, names: dict[str, str],
                  aliases: dict[str, tuple] | None = None):
         """names: checkpoint names of 'in_proj' [3d, d], 'conv' [d, K], 'out_proj' [d, d]."""
