@@ -38,7 +38,9 @@ def test_gemm_f32(gpu, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 16, 8), (5, 1000, 96), (17, 33, 40), (64, 777, 240), (65, 130, 136),
-                                   (200, 300, 328), (300, 64, 2048), (128, 128, 64), (2, 2048, 8192)])
+                                   (200, 300, 328), (300, 64, 2048), (128, 128, 64), (2, 2048, 8192),
+                                   (33, 100, 2048), (64, 2048, 8192), (20, 64, 1024), (48, 200, 512), (16, 24, 4096),
+                                   (8, 6144, 2048)])
 def test_gemm_bf16(gpu, M, N, K):
     from tuff_amd.csrc import ops
     x, w = _r(M, K, seed=4, dtype=torch.bfloat16), _r(N, K, seed=5, dtype=torch.bfloat16)
@@ -54,6 +56,15 @@ def test_gemm_bf16(gpu, M, N, K):
     acc = y0.to(gpu)
     ops.gemm(x.to(gpu), w.to(gpu), acc, accumulate=True)
     assert (acc.cpu().double() - (want + y0.double())).abs().max() <= 1e-5 * scale + 1e-6 * K
+    # the same call again gives the same bits (split-K partials are added in a fixed order), and
+    # among M <= 16 a row does not depend on the other rows of the call
+    again = torch.empty(M, N, device=gpu)
+    ops.gemm(x.to(gpu), w.to(gpu), again)
+    assert torch.equal(again, f32)
+    if 1 < M <= 16:
+        one = torch.empty(1, N, device=gpu)
+        ops.gemm(x[M - 1:].to(gpu), w.to(gpu), one)
+        assert torch.equal(one[0], f32[M - 1])
 
 
 def test_gemm_refuses_what_it_cannot_do(gpu):

@@ -1,16 +1,20 @@
 // bfloat16 matrix products on the gfx950 matrix cores:  Y[M,N] (=|+=) X[M,K] * W[N,K]^T,
 // X and W bfloat16 with K contiguous, products accumulated in float32.
 //
-// Two kernels, chosen by M on the host:
-//  * gemm_bf16_tiled   M > 64: 128x128 block tiles staged through LDS (compute bound);
-//  * gemm_bf16_skinny  M <= 64: weights streamed once from HBM straight into MFMA
-//    operands, K split over the four waves of a workgroup and summed in wave order
-//    (bandwidth bound).
-// Both use v_mfma_f32_16x16x32_bf16.  Lane l of a wave supplies row (l % 16) of an
-// operand tile and eight consecutive k at 8 * (l / 16); it receives rows
-// 4 * (l / 16) + 0..3, column (l % 16) of the 16x16 result.
-// Within one kernel the order in which the products of an output element are added
-// depends on K alone, never on M, N or the position of the row in the call.
+// Three kernels, chosen by M on the host:
+//  * tiled     M > 64: 128x128 block tiles staged through LDS (compute bound);
+//  * skinny64  16 < M <= 64: a workgroup owns 64 rows of W, one MFMA column tile a wave; the
+//    activations of a K chunk are staged once in LDS for all four waves (bandwidth bound);
+//  * skinny16  M <= 16: a workgroup owns 16 rows of W; its four waves split K (bandwidth bound).
+// The skinny kernels stream each weight byte once from HBM straight into MFMA operands.  Where
+// N alone gives too little parallelism to fill 256 CUs, skinny16 uses more waves a workgroup
+// (8 or 16, partials added in wave order through LDS) and skinny64 splits K over workgroups
+// (partial tiles in a work space, added in slice order by a second kernel).  The cut depends
+// on N and K only, never on M, so the order of additions is fixed.
+//
+// All use v_mfma_f32_16x16x32_bf16.  Lane l of a wave supplies row (l % 16) of an operand tile
+// and eight consecutive k at 8 * (l / 16); it receives rows 4 * (l / 16) + 0..3, column (l % 16)
+// of the 16x16 result.
 #include "common.h"
 
 enum : int { OUT_BF16 = 0, OUT_F32 = 1, OUT_F32_ACCUM = 2 };
@@ -118,63 +122,216 @@ __global__ __launch_bounds__(TNT) void gemm_bf16_tiled_kernel(const bf16_t* __re
         }
 }
 
-// ----------------------------------------------------------------- skinny kernel
-// One workgroup owns 16 rows of W (16 output columns) and all M <= 16*MT rows of X.
-// Wave w takes the k-chunks w, w+4, w+8, ... of 128 elements; in a chunk a lane reads
-// 64 contiguous bytes of its W row (and of each X row) and issues four MFMAs.  The four
-// wave partials are added in wave order 0,1,2,3 through LDS.
-constexpr int SK_CHUNK = 128, SK_NT = 256;
+// ----------------------------------------------------------------- skinny kernels
+constexpr int SK_CHUNK = 128;
 
-template <int MT, int MODE>
-__global__ __launch_bounds__(SK_NT) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
-                                                                 void* __restrict__ Y, int M, int N, int K) {
-    __shared__ float red[4][MT][WAVE][4];
+// M <= 16.  grid: tiles of 16 columns.  The NW waves of a workgroup split K: wave w takes the
+// chunks w, w + NW, w + 2 NW, ... of 128; in a chunk the wave reads 256 bytes of each of its 16 W
+// rows (and X rows) with four loads of 16 rows x 64 contiguous bytes and issues four MFMAs.  Loads run one chunk ahead.  The wave partials
+// are added in wave order through LDS.  NW is chosen from N and K only.
+template <int NW, int MODE>
+__global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+                                                                       void* __restrict__ Y, int M, int N, int K) {
+    __shared__ float red[NW][WAVE][4];
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
     const int r16 = lane % 16, g = lane / 16;
     const long long n0 = (long long)blockIdx.x * 16;
+    const int nchunks = (K + SK_CHUNK - 1) / SK_CHUNK;
+
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    bf16x8 a0[4], b0[4], a1[4], b1[4];
+    auto load = [&](int c, bf16x8* a, bf16x8* b) {
+        // instruction j of the wave reads bytes 64 j .. 64 j + 63 of the chunk of each of its 16 rows
+        const int kb = c * SK_CHUNK + g * 8;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[j] = load8(W, n0 + r16, N, kb + j * 32, K);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) a[j] = load8(X, r16, M, kb + j * 32, K);
+    };
+    // Workgroups start at different chunks (a rotation by the tile index), so that at any moment
+    // the chip reads from all columns of W and not from one: rows are a multiple of the DRAM
+    // channel interleave apart.  The order of a tile's additions still depends on N and K only.
+    const int rot = (int)((blockIdx.x * 5u) % (unsigned)nchunks);
+    auto chunk_of = [&](int i) { int c = i + rot; return c >= nchunks ? c - nchunks : c; };
+    int i = wave;
+    if (i < nchunks) load(chunk_of(i), a0, b0);
+    for (; i < nchunks; i += 2 * NW) {
+        const bool more = i + NW < nchunks;
+        if (more) load(chunk_of(i + NW), a1, b1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc = mfma16(a0[j], b0[j], acc);
+        if (more) {
+            if (i + 2 * NW < nchunks) load(chunk_of(i + 2 * NW), a0, b0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc = mfma16(a1[j], b1[j], acc);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) red[wave][lane][e] = acc[e];
+    __syncthreads();
+    if (tid < 256) {
+        // thread -> (lane l, element e) of the 16x16 tile; the wave partials in wave order
+        const int e = tid % 4, l = tid / 4;
+        float v = red[0][l][e];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) v += red[w][l][e];
+        const long long row = (l / 16) * 4 + e, col = n0 + (l % 16);
+        if (row < M && col < N) store_out<MODE>(Y, row * N + col, v);
+    }
+}
+
+// 16 < M <= 64.  grid (tiles of 64 columns, K slices).  Wave w owns columns 16w..16w+15 of the
+// tile and all MT row tiles.  The X rows of a K chunk (128 wide) go through LDS once for the
+// four waves, double buffered; W goes from HBM to registers one chunk ahead.  With more than
+// one K slice the partial tiles go to a work space and a second kernel adds them in slice order.
+constexpr int SK_NT = 256;
+constexpr int XS_STRIDE = SK_CHUNK + 8;             // bf16 elements; 272 bytes: conflict-free 16-byte reads
+
+template <int MT, int MODE>
+__global__ __launch_bounds__(SK_NT) void gemm_bf16_skinny64_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+                                                                   void* __restrict__ Y, int M, int N, int K, int chunks_per_slice,
+                                                                   float* __restrict__ ws) {
+    __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16 * XS_STRIDE];
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const int r16 = lane % 16, g = lane / 16;
+    const int tile = blockIdx.x, slice = blockIdx.y, n_slices = gridDim.y;
+    const long long nrow = (long long)tile * 64 + wave * 16 + r16;       // this lane's W row
+    const int nchunks = (K + SK_CHUNK - 1) / SK_CHUNK;
+    const int c_begin = slice * chunks_per_slice, c_end = min(nchunks, c_begin + chunks_per_slice);
 
     f32x4 acc[MT];
 #pragma unroll
     for (int i = 0; i < MT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int nchunks = (K + SK_CHUNK - 1) / SK_CHUNK;
-    for (int c = wave; c < nchunks; c += 4) {
-        const int kb = c * SK_CHUNK + g * 32;
-        bf16x8 b[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) b[j] = load8(W, n0 + r16, N, kb + j * 8, K);
+    // X chunk: MT*16 rows x 16 pieces of 16 bytes = MT*256 pieces, MT a thread
+    bf16x8 xr[MT], b0[4], b1[4];
+    auto load_x = [&](int c) {
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
-            bf16x8 a[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) a[j] = load8(X, i * 16 + r16, M, kb + j * 8, K);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc[i] = mfma16(a[j], b[j], acc[i]);
+            const int id = tid + i * SK_NT;
+            xr[i] = load8(X, id / 16, M, c * SK_CHUNK + (id % 16) * 8, K);
         }
+    };
+    auto store_x = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const int id = tid + i * SK_NT;
+            *(bf16x8*)(&xs[buf][(id / 16) * XS_STRIDE + (id % 16) * 8]) = xr[i];
+        }
+    };
+    auto load_w = [&](int c, bf16x8* b) {
+        const int kb = c * SK_CHUNK + g * 8;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[j] = load8(W, nrow, N, kb + j * 32, K);
+    };
+    auto compute = [&](int buf, const bf16x8* b) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bf16x8 a = *(const bf16x8*)(&xs[buf][(i * 16 + r16) * XS_STRIDE + j * 32 + g * 8]);
+                acc[i] = mfma16(a, b[j], acc[i]);
+            }
+    };
+
+    if (c_begin < c_end) {
+        load_x(c_begin);
+        load_w(c_begin, b0);
+        store_x(0);
+    }
+    __syncthreads();
+    for (int c = c_begin; c < c_end; c += 2) {
+        // chunk c from buffer 0 / b0, chunk c+1 from buffer 1 / b1
+        const bool more1 = c + 1 < c_end, more2 = c + 2 < c_end;
+        if (more1) { load_x(c + 1); load_w(c + 1, b1); }
+        compute(0, b0);
+        if (more1) store_x(1);
+        __syncthreads();
+        if (more1) {
+            if (more2) { load_x(c + 2); load_w(c + 2, b0); }
+            compute(1, b1);
+            if (more2) store_x(0);
+            __syncthreads();
+        }
+    }
+
+    const long long col = (long long)tile * 64 + wave * 16 + r16;
+    if (col >= N) return;
+    if (n_slices > 1) {
+        // partial tile of this slice: ws[slice][row][col]
+        float* mine = ws + (long long)slice * (MT * 16) * N;
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) mine[(long long)(i * 16 + g * 4 + e) * N + col] = acc[i][e];
+        return;
     }
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) red[wave][i][lane][e] = acc[i][e];
-    __syncthreads();
-    // 256 threads share the MT*64*4 sums: element id -> (i, lane, e)
-    for (int id = tid; id < MT * WAVE * 4; id += SK_NT) {
-        const int e = id % 4, l = (id / 4) % WAVE, i = id / (4 * WAVE);
-        const float v = ((red[0][i][l][e] + red[1][i][l][e]) + red[2][i][l][e]) + red[3][i][l][e];
-        const long long row = i * 16 + (l / 16) * 4 + e, col = n0 + (l % 16);
-        if (row < M && col < N) store_out<MODE>(Y, row * N + col, v);
+        for (int e = 0; e < 4; ++e) {
+            const long long row = i * 16 + g * 4 + e;
+            if (row < M) store_out<MODE>(Y, row * N + col, acc[i][e]);
+        }
+}
+
+// Y (=|+=) sum over slices, in slice order, of ws[slice][row][col]; rows_padded rows a slice.
+template <int MODE>
+__global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* __restrict__ Y, int M, int N, int rows_padded,
+                                     int n_slices) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (long long)M * N) return;
+    float v = 0.f;
+    for (int s = 0; s < n_slices; ++s) v += ws[(long long)s * rows_padded * N + i];
+    store_out<MODE>(Y, i, v);
+}
+
+struct SkinnyPlan { int tiles, waves, slices, chunks_per_slice; long long ws_floats; };
+
+// How a skinny product is cut.  Depends on N and K (and on which of the two kernels M selects).
+SkinnyPlan plan_skinny(int M, int N, int K) {
+    const int nchunks = ceil_div(K, SK_CHUNK);
+    SkinnyPlan p;
+    p.slices = 1; p.chunks_per_slice = nchunks; p.ws_floats = 0; p.waves = 4;
+    if (M <= 16) {
+        p.tiles = ceil_div(N, 16);
+        // enough waves in flight to cover the latency of HBM, at least one chunk a wave
+        while (p.waves < 16 && p.tiles * p.waves < 3072 && nchunks >= 2 * p.waves) p.waves *= 2;
+    } else {
+        const int mt = ceil_div(M, 16);
+        p.tiles = ceil_div(N, 64);
+        int s = ceil_div(512, p.tiles);
+        s = max(1, min(s, nchunks / 2));
+        p.chunks_per_slice = ceil_div(nchunks, s);
+        p.slices = ceil_div(nchunks, p.chunks_per_slice);
+        p.ws_floats = p.slices > 1 ? (long long)p.slices * mt * 16 * N : 0;
     }
+    return p;
 }
 
 template <int MODE>
-int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, hipStream_t stream) {
-    if (M <= 64) {
-        dim3 grid(ceil_div(N, 16)), block(SK_NT);
+int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, float* ws, hipStream_t stream) {
+    if (M <= 16) {
+        const SkinnyPlan p = plan_skinny(M, N, K);
+        dim3 grid(p.tiles);
+        if (p.waves == 4) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<4, MODE>), grid, dim3(256), 0, stream, X, W, Y, M, N, K);
+        else if (p.waves == 8) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<8, MODE>), grid, dim3(512), 0, stream, X, W, Y, M, N, K);
+        else hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<16, MODE>), grid, dim3(1024), 0, stream, X, W, Y, M, N, K);
+    } else if (M <= 64) {
+        const SkinnyPlan p = plan_skinny(M, N, K);
+        dim3 grid(p.tiles, p.slices), block(SK_NT);
+        if (p.slices > 1 && !ws) return -4;
+#define GO(MT) hipLaunchKernelGGL((gemm_bf16_skinny64_kernel<MT, MODE>), grid, block, 0, stream, X, W, Y, M, N, K, p.chunks_per_slice, ws)
         const int mt = ceil_div(M, 16);
-        if (mt == 1) hipLaunchKernelGGL((gemm_bf16_skinny_kernel<1, MODE>), grid, block, 0, stream, X, W, Y, M, N, K);
-        else if (mt == 2) hipLaunchKernelGGL((gemm_bf16_skinny_kernel<2, MODE>), grid, block, 0, stream, X, W, Y, M, N, K);
-        else if (mt == 3) hipLaunchKernelGGL((gemm_bf16_skinny_kernel<3, MODE>), grid, block, 0, stream, X, W, Y, M, N, K);
-        else hipLaunchKernelGGL((gemm_bf16_skinny_kernel<4, MODE>), grid, block, 0, stream, X, W, Y, M, N, K);
+        if (mt == 2) GO(2); else if (mt == 3) GO(3); else GO(4);
+#undef GO
+        if (p.slices > 1) {
+            int rc = launch_status();
+            if (rc) return rc;
+            const long long n = (long long)M * N;
+            hipLaunchKernelGGL((splitk_reduce_kernel<MODE>), dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, stream,
+                               (const float*)ws, Y, M, N, mt * 16, p.slices);
+        }
     } else {
         dim3 grid(ceil_div(N, TBN), ceil_div(M, TBM)), block(TNT);
         hipLaunchKernelGGL((gemm_bf16_tiled_kernel<MODE>), grid, block, 0, stream, X, W, Y, M, N, K);
@@ -183,15 +340,23 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
 }
 }  // namespace
 
+// Work space a product of this shape needs: *ws_floats float32 for partial tiles (0: none).
+TUFF_EXPORT int tuff_gemm_bf16_workspace(int M, int N, int K, long long* ws_floats) {
+    *ws_floats = 0;
+    if (M > 64 || M <= 16 || N <= 0) return 0;
+    *ws_floats = plan_skinny(M, N, K).ws_floats;
+    return 0;
+}
+
 // K must be a multiple of 8 (16-byte operand loads); the host wrapper refuses other K.
 TUFF_EXPORT int tuff_gemm_bf16(const void* X, const void* W, void* Y, int M, int N, int K, int mode,
-                               hipStream_t stream) {
+                               float* ws, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (K % 8 != 0) return -2;
     const bf16_t* x = (const bf16_t*)X;
     const bf16_t* w = (const bf16_t*)W;
-    if (mode == OUT_BF16) return launch_mode<OUT_BF16>(x, w, Y, M, N, K, stream);
-    if (mode == OUT_F32) return launch_mode<OUT_F32>(x, w, Y, M, N, K, stream);
-    if (mode == OUT_F32_ACCUM) return launch_mode<OUT_F32_ACCUM>(x, w, Y, M, N, K, stream);
+    if (mode == OUT_BF16) return launch_mode<OUT_BF16>(x, w, Y, M, N, K, ws, stream);
+    if (mode == OUT_F32) return launch_mode<OUT_F32>(x, w, Y, M, N, K, ws, stream);
+    if (mode == OUT_F32_ACCUM) return launch_mode<OUT_F32_ACCUM>(x, w, Y, M, N, K, ws, stream);
     return -3;
 }

@@ -36,7 +36,8 @@ _SIGNATURES = {
         "tuff_gemm_f32": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
     "gemm_bf16": {
-        "tuff_gemm_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_gemm_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
+        "tuff_gemm_bf16_workspace": [_c_int, _c_int, _c_int, ctypes.POINTER(_c_ll)],
     },
     "rope_kv": {
         "tuff_qkv_post": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
@@ -200,8 +201,26 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         mode = OUT_BF16
     else:
         raise KernelError(f"gemm: unsupported output type {out.dtype}")
+    ws_floats = _gemm_workspace(M, N, K)
+    ws = torch.empty(ws_floats, dtype=torch.float32, device=x.device) if ws_floats else None
     _check(load("gemm_bf16").tuff_gemm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, mode,
-                                            _stream()), "gemm_bf16")
+                                            None if ws is None else ws.data_ptr(), _stream()), "gemm_bf16")
+
+
+_plans: dict = {}
+
+
+def _gemm_workspace(M: int, N: int, K: int) -> int:
+    """float32 elements of work space a bfloat16 product of this shape needs (0: none)."""
+    if M <= 16 or M > 64:
+        return 0
+    key = (M, N, K)
+    n = _plans.get(key)
+    if n is None:
+        a = _c_ll(0)
+        load("gemm_bf16").tuff_gemm_bf16_workspace(M, N, K, ctypes.byref(a))
+        n = _plans[key] = int(a.value)
+    return n
 
 
 # ----------------------------------------------------------------- q/k/v post-processing
