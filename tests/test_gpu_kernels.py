@@ -67,6 +67,56 @@ def test_gemm_bf16(gpu, M, N, K):
         assert torch.equal(one[0], f32[M - 1])
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 32, 64), (8, 512, 240), (16, 6144, 2048), (5, 200, 96), (64, 384, 256),
+                                   (40, 2050, 2048), (300, 130, 136), (2048, 512, 128)])
+def test_gemm_bf16_swiglu_epilogue(gpu, M, N, K):
+    """Rows of w are gate and up rows interleaved; the output is silu(gate) * up."""
+    from tuff_amd.csrc import ops
+    x, w = _r(M, K, seed=4, dtype=torch.bfloat16), _r(N, K, seed=5, dtype=torch.bfloat16)
+    y = x.double() @ w.double().T
+    g, u = y[:, 0::2], y[:, 1::2]
+    want = g / (1 + torch.exp(-g)) * u
+    out = torch.empty(M, N // 2, device=gpu, dtype=torch.bfloat16)
+    ops.gemm(x.to(gpu), w.to(gpu), out, swiglu=True)
+    assert (out.cpu().double() - want).abs().max() <= 2 ** -8 * float(want.abs().max()) + 1e-4 * K ** 0.5
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 16, 64), (8, 6144, 2048), (16, 130, 240), (3, 1000, 96), (7, 65536, 2048), (2, 48, 8192)])
+@pytest.mark.parametrize("use_rows", [False, True])
+def test_gemm_with_the_norm_inside(gpu, M, N, K, use_rows):
+    """y = rmsnorm(x) w^T in one kernel equals the norm kernel followed by the product, to the
+    rounding of the bfloat16 operand, and is close to the float64 value."""
+    from tuff_amd.csrc import ops
+    n_x = M + 3 if use_rows else M
+    x = _r(n_x, K, seed=1, scale=2.0)
+    nw = 1 + _r(K, seed=2, scale=0.1)
+    w = _r(N, K, seed=3, scale=0.05, dtype=torch.bfloat16)
+    rows = torch.randperm(n_x, generator=torch.Generator().manual_seed(4))[:M].to(torch.int32) if use_rows else None
+    xs = x[rows.long()] if use_rows else x
+    eps = 1e-5
+    want = plain.rms_norm(xs.double(), nw.double(), eps) @ w.double().T
+    out = torch.empty(M, N, device=gpu)
+    ops.gemm_normed(x.to(gpu), nw.to(gpu), eps, w.to(gpu), out, rows=None if rows is None else rows.to(gpu))
+    scale = float(want.abs().max())
+    assert (out.cpu().double() - want).abs().max() <= 2 ** -7 * scale
+    # accumulate and swiglu epilogues
+    y0 = _r(M, N, seed=6)
+    acc = y0.to(gpu)
+    ops.gemm_normed(x.to(gpu), nw.to(gpu), eps, w.to(gpu), acc, rows=None if rows is None else rows.to(gpu), accumulate=True)
+    assert (acc.cpu().double() - (want + y0.double())).abs().max() <= 2 ** -7 * scale
+    sw = torch.empty(M, N // 2, device=gpu, dtype=torch.bfloat16)
+    ops.gemm_normed(x.to(gpu), nw.to(gpu), eps, w.to(gpu), sw, rows=None if rows is None else rows.to(gpu), swiglu=True)
+    g, u = want[:, 0::2], want[:, 1::2]
+    ref = g / (1 + torch.exp(-g)) * u
+    assert (sw.cpu().double() - ref).abs().max() <= 2 ** -6 * max(float(ref.abs().max()), scale * 0.1)
+    # a row does not depend on the other rows of the call
+    if M > 1:
+        one = torch.empty(1, N, device=gpu)
+        r1 = (rows[M - 1:] if use_rows else torch.tensor([M - 1], dtype=torch.int32)).to(gpu)
+        ops.gemm_normed(x.to(gpu), nw.to(gpu), eps, w.to(gpu), one, rows=r1)
+        assert torch.equal(one[0], out[M - 1])
+
+
 def test_gemm_refuses_what_it_cannot_do(gpu):
     from tuff_amd.csrc import ops
     x = torch.zeros(2, 12, dtype=torch.bfloat16, device=gpu)
@@ -75,8 +125,12 @@ def test_gemm_refuses_what_it_cannot_do(gpu):
         ops.gemm(x, w, torch.empty(2, 4, device=gpu))
     with pytest.raises(ops.KernelError, match="no CPU fallback"):
         ops.gemm(torch.zeros(2, 8), torch.zeros(4, 8), torch.zeros(2, 4))
+    x16 = torch.zeros(2, 16, dtype=torch.bfloat16, device=gpu)
+    w16 = torch.zeros(4, 16, dtype=torch.bfloat16, device=gpu)
     with pytest.raises(ops.KernelError, match="expected shape"):
-        ops.gemm(x, w, torch.empty(3, 4, device=gpu))
+        ops.gemm(x16, w16, torch.empty(3, 4, device=gpu))
+    with pytest.raises(ops.KernelError, match="at most 16 rows"):
+        ops.gemm_normed(torch.zeros(17, 16, device=gpu), torch.ones(16, device=gpu), 1e-5, w16, torch.empty(17, 4, device=gpu))
 
 
 # ------------------------------------------------------------------------- row kernels
@@ -387,6 +441,27 @@ def test_shortconv(gpu, d, K, dt):
         assert (got - want).abs().max() <= tol * float(want.abs().max())
         assert (state[int(slots[r])].cpu().double() - want_state).abs().max() <= 1e-6
     assert (state[1] == 0).all() and (state[3] == 0).all()       # other requests' slots untouched
+
+
+@pytest.mark.parametrize("d,K", [(64, 3), (96, 4), (240, 2), (300, 7)])
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_shortconv_single_token_kernel_equals_the_general_pair(gpu, d, K, dt):
+    from tuff_amd.csrc import ops
+    R = 5
+    w = _r(d, K, seed=20, dtype=dt).to(gpu)
+    slots = torch.tensor([3, 0, 6, 1, 4], dtype=torch.int32, device=gpu)
+    s1 = _r(8, K - 1, d, seed=21).to(gpu)
+    s2 = s1.clone()
+    ar = torch.arange(R, dtype=torch.int32, device=gpu)
+    ones = torch.ones(R, dtype=torch.int32, device=gpu)
+    for step in range(4):
+        bcx = _r(R, 3 * d, seed=30 + step, dtype=dt).to(gpu)
+        o1 = torch.empty(R, d, dtype=dt, device=gpu)
+        o2 = torch.empty(R, d, dtype=dt, device=gpu)
+        ops.shortconv_fwd(bcx, w, s1, o1, req_of_token=ar, q_start=ar, state_slot=slots, K=K)
+        ops.shortconv_state(bcx, s1, q_start=ar, q_len=ones, state_slot=slots, K=K)
+        ops.shortconv_decode(bcx, w, s2, o2, state_slot=slots, K=K)
+        assert torch.equal(o1, o2) and torch.equal(s1, s2), step
 
 
 def test_shortconv_last_tap_is_the_current_token(gpu):

@@ -114,6 +114,7 @@ class _Request:
     slot: int
     length: int = 0
     tables: list = dataclasses.field(default_factory=list)     # per group: page id or FREED per block
+    arrays: dict = dataclasses.field(default_factory=dict)     # per group: the table as int32 array, while current
 
 
 class CacheManager:
@@ -188,6 +189,9 @@ class CacheManager:
         r = self._req(req_id)
         out = []
         for gi, g in enumerate(self.groups):
+            if g.window is None:
+                out.append(0)
+                continue
             lo = self._first_needed_block(g, r.length)
             out.append(sum(1 for p in r.tables[gi][:lo] if p != FREED))
         return out
@@ -207,6 +211,7 @@ class CacheManager:
             lo = self._first_needed_block(g, r.length)
             gone = [p for p in r.tables[gi][:lo] if p != FREED]
             if gone:
+                r.arrays.pop(gi, None)
                 g.pool.free(gone)
                 for b in range(min(lo, len(r.tables[gi]))):
                     r.tables[gi][b] = FREED
@@ -216,7 +221,9 @@ class CacheManager:
                 raise OutOfPages(f"request {req_id!r}: {n} pages wanted, {g.pool.num_free} free "
                                  f"of {g.pool.num_pages} (window {g.window})")
         for gi, (n, g) in enumerate(zip(need, self.groups)):
-            r.tables[gi].extend(g.pool.alloc(n))
+            if n:
+                r.arrays.pop(gi, None)
+                r.tables[gi].extend(g.pool.alloc(n))
         r.length += n_new
 
     def truncate(self, req_id, length: int) -> None:
@@ -230,6 +237,7 @@ class CacheManager:
             extra = [p for p in r.tables[gi][keep:] if p != FREED]
             g.pool.free(extra)
             del r.tables[gi][keep:]
+        r.arrays.clear()
         r.length = length
 
     def release(self, req_id) -> None:
@@ -243,6 +251,15 @@ class CacheManager:
     # ------------------------------------------------------------------ lookups
     def block_table(self, req_id, group: int) -> list[int]:
         return self._req(req_id).tables[group]
+
+    def block_table_array(self, req_id, group: int):
+        """The block table as an int32 numpy array (kept until the table changes)."""
+        import numpy as np
+        r = self._req(req_id)
+        a = r.arrays.get(group)
+        if a is None:
+            a = r.arrays[group] = np.asarray(r.tables[group], dtype=np.int32)
+        return a
 
     def slot_of_position(self, req_id, group: int, pos: int) -> int:
         page = self._req(req_id).tables[group][pos // self.page_size]

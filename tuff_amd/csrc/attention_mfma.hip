@@ -18,7 +18,8 @@
 //    as they lie, the lane's part of the B operand P^T of the second product if the product's
 //    summed index is numbered k = 8g + i  <->  key (i < 4 ? 4g + i : 16 + 4g + i - 4).  The
 //    A operand V^T follows the same numbering: two 8-byte loads from the transposed V page.
-//  * No LDS, no transposes, no barriers.
+//  * No LDS, no transposes, no barriers; K rows and V columns of the next step are loaded
+//    while the current step computes.
 //
 // Cache layout: K [page][kv_head][offset][hd], V [page][kv_head][hd][offset]; the page size
 // must be a multiple of 16 and the head size a multiple of 8 (the host falls back to the
@@ -89,28 +90,56 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
         for (int db = 0; db < DB; ++db) o[db][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    for (int key0 = key_begin; key0 < key_end; key0 += 32) {
-        // ---- S^T = K Q^T for two blocks of 16 keys
-        f32x4 s[2][NB];
-        long long vbase[2];                // start of the block's 16 positions in the V page, or -1
+    // One step covers 32 keys as two blocks of 16.  A step's K rows and V columns are loaded
+    // into registers a step ahead of their use (where the head size leaves room for it).
+    // Large tiles (head size x columns) leave no registers for that: they load as they go.
+    constexpr bool AHEAD = HDP * NB <= 256;
+    struct Tile {
+        bf16x8 kf[2][AHEAD ? KC : 1];
+        bf16x4 vx[2][AHEAD ? DB : 1];
+        long long base[2];                 // (page, kv head) start in both caches
+        int off0[2];
+        bool live[2];
+    };
+    auto k_frag = [&](long long base, int off0, int kc) {
+        const int k = kc * 32 + g * 8;
+        bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+        return (k < hd) ? *(const bf16x8*)(k_cache + base + (long long)(off0 + n16) * hd + k) : z;
+    };
+    auto v_frag = [&](long long base, int off0, int db) {
+        const int dim = db * 16 + n16;
+        bf16x4 z = {0, 0, 0, 0};
+        return (dim < hd) ? *(const bf16x4*)(v_cache + base + off0 + 4 * g + (long long)dim * page_size) : z;
+    };
+    auto load_tile = [&](int key0, Tile& t) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
             const int kbs = key0 + kb * 16;
-            const bool live = kbs <= pos_max && kbs + 15 >= lo_min;
-            vbase[kb] = -1;
+            t.live[kb] = kbs <= pos_max && kbs + 15 >= lo_min;
+            if (!t.live[kb]) continue;
+            const long long page = table[kbs / page_size];
+            t.off0[kb] = kbs % page_size;
+            t.base[kb] = (page * Hkv + kvh) * (long long)page_size * hd;
+            if constexpr (AHEAD) {
+#pragma unroll
+                for (int kc = 0; kc < KC; ++kc) t.kf[kb][kc] = k_frag(t.base[kb], t.off0[kb], kc);
+#pragma unroll
+                for (int db = 0; db < DB; ++db) t.vx[kb][db] = v_frag(t.base[kb], t.off0[kb], db);
+            }
+        }
+    };
+    auto compute = [&](int key0, const Tile& t) {
+        // ---- S^T = K Q^T for two blocks of 16 keys
+        f32x4 s[2][NB];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) s[kb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (live) {
-                const long long page = table[kbs / page_size];
-                const int off0 = kbs % page_size;
-                const long long head_base = (page * Hkv + kvh) * (long long)page_size * hd;
-                vbase[kb] = head_base + off0;
-                const bf16_t* krow = k_cache + head_base + (long long)(off0 + n16) * hd;
+            if (t.live[kb]) {
 #pragma unroll
                 for (int kc = 0; kc < KC; ++kc) {
-                    const int k = kc * 32 + g * 8;
-                    bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-                    const bf16x8 kf = (k < hd) ? *(const bf16x8*)(krow + k) : z;
+                    bf16x8 kf;
+                    if constexpr (AHEAD) kf = t.kf[kb][kc]; else kf = k_frag(t.base[kb], t.off0[kb], kc);
 #pragma unroll
                     for (int nb = 0; nb < NB; ++nb) s[kb][nb] = mfma32(kf, qf[nb][kc], s[kb][nb]);
                 }
@@ -128,7 +157,7 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int key = key0 + kb * 16 + 4 * g + e;
-                    const bool ok = vbase[kb] >= 0 && key <= pos_c[nb] && key >= lo_c[nb];
+                    const bool ok = t.live[kb] && key <= pos_c[nb] && key >= lo_c[nb];
                     const float x = ok ? s[kb][nb][e] * scale : -INFINITY;
                     v[kb * 4 + e] = x;
                     mx = fmaxf(mx, x);
@@ -152,18 +181,16 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
         const bool tail = key0 + 31 > pos_max;             // keys beyond pos_max were never written
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-            const int dim = db * 16 + n16;
             bf16x8 vf = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (dim < hd) {
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb) {
-                    if (vbase[kb] < 0) continue;
-                    const bf16x4 x = *(const bf16x4*)(v_cache + vbase[kb] + (long long)dim * page_size + 4 * g);
+            for (int kb = 0; kb < 2; ++kb) {
+                if (!t.live[kb]) continue;
+                bf16x4 x;
+                if constexpr (AHEAD) x = t.vx[kb][db]; else x = v_frag(t.base[kb], t.off0[kb], db);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const bool written = !tail || (key0 + kb * 16 + 4 * g + e <= pos_max);
-                        vf[kb * 4 + e] = written ? x[e] : (bf16_t)0.f;
-                    }
+                for (int e = 0; e < 4; ++e) {
+                    const bool written = !tail || (key0 + kb * 16 + 4 * g + e <= pos_max);
+                    vf[kb * 4 + e] = written ? x[e] : (bf16_t)0.f;
                 }
             }
 #pragma unroll
@@ -173,6 +200,26 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
                 for (int e = 0; e < 4; ++e) acc[e] *= corr[nb];
                 o[db][nb] = mfma32(vf, pf[nb], acc);
             }
+        }
+    };
+
+    if constexpr (AHEAD) {
+        Tile t0, t1;
+        load_tile(key_begin, t0);
+        for (int key0 = key_begin; key0 < key_end; key0 += 64) {
+            const bool more = key0 + 32 < key_end;
+            if (more) load_tile(key0 + 32, t1);
+            compute(key0, t0);
+            if (more) {
+                if (key0 + 64 < key_end) load_tile(key0 + 64, t0);
+                compute(key0 + 32, t1);
+            }
+        }
+    } else {
+        Tile t0;
+        for (int key0 = key_begin; key0 < key_end; key0 += 32) {
+            load_tile(key0, t0);
+            compute(key0, t0);
         }
     }
 
@@ -193,35 +240,50 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
     }
 }
 
-// Merges the partitions of one (token, head) in ascending order and writes the bfloat16 row.
+// Merges the partitions of one (token, head) and writes the bfloat16 row:
+//   M = max_p m_p;  w_p = exp(m_p - M);  out = (sum_p w_p o_p) / (sum_p w_p l_p),
+// the sums over p in a fixed order (ascending p for the output, a fixed butterfly for the
+// denominator), so the result depends on the token's position only.
+constexpr int COMBINE_MAX_PARTS = 2048;
+
 __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                                             bf16_t* __restrict__ out, const int* __restrict__ positions,
                                                             int H, int hd, int window, int n_parts) {
+    __shared__ float wts[COMBINE_MAX_PARTS];
     const long long row = blockIdx.x;                      // token * H + head
     const int lane = threadIdx.x;
     const int pos = positions[row / H];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    float M = -INFINITY, L = 0.f;
+    const int p_lo = lo / PART, np = pos / PART - p_lo + 1;
+    const float* ml = ws_ml + (row * n_parts + p_lo) * 2;
+    float M = -INFINITY;
+    for (int i = lane; i < np; i += WAVE) M = fmaxf(M, ml[i * 2 + 1] > 0.f ? ml[i * 2] : -INFINITY);
+    M = wave_max(M);
+    float L = 0.f;
+    for (int i = lane; i < np; i += WAVE) {
+        const float l = ml[i * 2 + 1];
+        const float w = l > 0.f ? __expf(ml[i * 2] - M) : 0.f;
+        wts[i] = w;
+        L += w * l;
+    }
+    L = wave_sum(L);
+    __syncthreads();
+    const float* o = ws_o + (row * n_parts + p_lo) * hd;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int p = lo / PART; p <= pos / PART; ++p) {
-        const long long slot = row * n_parts + p;
-        const float m = ws_ml[slot * 2], l = ws_ml[slot * 2 + 1];
-        if (!(l > 0.f)) continue;
-        const float M_new = fmaxf(M, m);
-        const float a = __expf(M - M_new), b = __expf(m - M_new);
-        L = L * a + l * b;
+#pragma unroll 4
+    for (int i = 0; i < np; ++i) {
+        const float w = wts[i];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int d = lane + i * WAVE;
-            if (d < hd) acc[i] = acc[i] * a + ws_o[slot * hd + d] * b;
+        for (int j = 0; j < 4; ++j) {
+            const int d = lane + j * WAVE;
+            if (d < hd) acc[j] = fmaf(w, o[(long long)i * hd + d], acc[j]);
         }
-        M = M_new;
     }
     const float inv = 1.0f / L;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int d = lane + i * WAVE;
-        if (d < hd) out[row * hd + d] = (bf16_t)(acc[i] * inv);
+    for (int j = 0; j < 4; ++j) {
+        const int d = lane + j * WAVE;
+        if (d < hd) out[row * hd + d] = (bf16_t)(acc[j] * inv);
     }
 }
 
@@ -247,7 +309,7 @@ TUFF_EXPORT int tuff_attention_mfma(const void* q, const void* k_cache, const vo
                                     int n_parts, hipStream_t stream) {
     if (n_tokens <= 0 || n_qblocks <= 0) return 0;
     if (hd > 256 || hd % 8 != 0 || page_size % 16 != 0 || Hkv <= 0 || H % Hkv != 0 || n_parts < 1) return -2;
-    if (Hkv > 65535 || n_qblocks > 65535) return -2;
+    if (Hkv > 65535 || n_qblocks > 65535 || n_parts > COMBINE_MAX_PARTS) return -2;
     const bf16_t* Q = (const bf16_t*)q;
     const bf16_t* K = (const bf16_t*)k_cache;
     const bf16_t* V = (const bf16_t*)v_cache;

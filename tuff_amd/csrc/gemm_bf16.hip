@@ -17,7 +17,9 @@
 // of the 16x16 result.
 #include "common.h"
 
-enum : int { OUT_BF16 = 0, OUT_F32 = 1, OUT_F32_ACCUM = 2 };
+// OUT_SWIGLU: the rows of W are gate and up rows interleaved (2f: gate f, 2f+1: up f); the
+// output is bfloat16 [M, N/2] with y[m, f] = silu(g) * u, silu(g) = g / (1 + exp(-g)).
+enum : int { OUT_BF16 = 0, OUT_F32 = 1, OUT_F32_ACCUM = 2, OUT_SWIGLU = 3 };
 
 namespace {
 
@@ -30,6 +32,19 @@ __device__ __forceinline__ void store_out(void* Y, long long idx, float v) {
     if (MODE == OUT_BF16) ((bf16_t*)Y)[idx] = (bf16_t)v;
     else if (MODE == OUT_F32) ((float*)Y)[idx] = v;
     else ((float*)Y)[idx] += v;
+}
+
+__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+
+// Stores element (row, col) of the product.  For OUT_SWIGLU `partner` is the value of column
+// col ^ 1 of the same row; even columns (the gates) write.  Every lane must call it.
+template <int MODE>
+__device__ __forceinline__ void store_elem(void* Y, long long row, long long col, int M, int N, float v, float partner) {
+    if (MODE == OUT_SWIGLU) {
+        if ((col & 1) == 0 && row < M && col < N) ((bf16_t*)Y)[row * (N / 2) + col / 2] = (bf16_t)silu_mul(v, partner);
+    } else {
+        if (row < M && col < N) store_out<MODE>(Y, row * N + col, v);
+    }
 }
 
 // 16-byte load of eight bf16 with a guard; out-of-range pieces read as zero.
@@ -113,11 +128,12 @@ __global__ __launch_bounds__(TNT) void gemm_bf16_tiled_kernel(const bf16_t* __re
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const long long col = n0 + wn + j * 16 + r16;
-            if (col >= N) continue;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const long long row = m0 + wm + i * 16 + g * 4 + e;
-                if (row < M) store_out<MODE>(Y, row * N + col, acc[i][j][e]);
+                const float v = acc[i][j][e];
+                const float partner = (MODE == OUT_SWIGLU) ? __shfl_xor(v, 1, WAVE) : 0.f;
+                store_elem<MODE>(Y, row, col, M, N, v, partner);
             }
         }
 }
@@ -127,47 +143,100 @@ constexpr int SK_CHUNK = 128;
 
 // M <= 16.  grid: tiles of 16 columns.  The NW waves of a workgroup split K: wave w takes the
 // chunks w, w + NW, w + 2 NW, ... of 128; in a chunk the wave reads 256 bytes of each of its 16 W
-// rows (and X rows) with four loads of 16 rows x 64 contiguous bytes and issues four MFMAs.  Loads run one chunk ahead.  The wave partials
-// are added in wave order through LDS.  NW is chosen from N and K only.
-template <int NW, int MODE>
-__global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
-                                                                       void* __restrict__ Y, int M, int N, int K) {
+// rows (and X rows) with four loads of 16 rows x 64 contiguous bytes and issues four MFMAs.
+// Loads run one chunk ahead.  The wave partials are added in wave order through LDS.  NW is
+// chosen from N and K only.
+//
+// NORM: X is the float32 residual stream and the product is taken of its RMSNorm,
+//   y[m, n] = (1 / sqrt(mean_k x[m,k]^2 + eps)) * sum_k bf16(x[m,k] * w[k]) W[n,k]:
+// the norm weight is applied to the operand, the row's scale to the result, and the sum of
+// squares is taken from the very values the workgroup loads anyway (in float32, lane partials
+// in a fixed butterfly, then waves in wave order).  `rows` (optional) gathers rows of X.
+template <int NW, int MODE, bool NORM>
+__global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const void* __restrict__ Xv, const bf16_t* __restrict__ W,
+                                                                       void* __restrict__ Y, int M, int N, int K,
+                                                                       const float* __restrict__ norm_w, float eps,
+                                                                       const int* __restrict__ rows) {
     __shared__ float red[NW][WAVE][4];
+    __shared__ float ssq[NW][16];
+    extern __shared__ __attribute__((aligned(16))) float nw_lds[];       // NORM: the norm weight, K floats
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
     const int r16 = lane % 16, g = lane / 16;
     const long long n0 = (long long)blockIdx.x * 16;
     const int nchunks = (K + SK_CHUNK - 1) / SK_CHUNK;
+    const bf16_t* X = (const bf16_t*)Xv;
+    const float* xrow = nullptr;
+    if (NORM && r16 < M) xrow = (const float*)Xv + (long long)(rows ? rows[r16] : r16) * K;
 
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    bf16x8 a0[4], b0[4], a1[4], b1[4];
-    auto load = [&](int c, bf16x8* a, bf16x8* b) {
+    float ss = 0.f;
+    struct Operands { bf16x8 a[4]; bf16x8 b[4]; f32x4 x[NORM ? 4 : 1][2]; };
+    Operands o0, o1;
+    auto load = [&](int c, Operands& o) {
         // instruction j of the wave reads bytes 64 j .. 64 j + 63 of the chunk of each of its 16 rows
         const int kb = c * SK_CHUNK + g * 8;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) b[j] = load8(W, n0 + r16, N, kb + j * 32, K);
+        for (int j = 0; j < 4; ++j) o.b[j] = load8(W, n0 + r16, N, kb + j * 32, K);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) a[j] = load8(X, r16, M, kb + j * 32, K);
+        for (int j = 0; j < 4; ++j) {
+            const int k = kb + j * 32;
+            if (NORM) {
+                const bool ok = xrow != nullptr && k < K;
+                o.x[j][0] = ok ? *(const f32x4*)(xrow + k) : f32x4{0.f, 0.f, 0.f, 0.f};
+                o.x[j][1] = ok ? *(const f32x4*)(xrow + k + 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+            } else {
+                o.a[j] = load8(X, r16, M, k, K);
+            }
+        }
+    };
+    auto multiply = [&](int c, Operands& o) {
+        if (NORM) {
+            const int kb = c * SK_CHUNK + g * 8;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int k = min(kb + j * 32, K - 8);               // past the end x is zero anyway
+                const f32x4 w0 = *(const f32x4*)(&nw_lds[k]), w1 = *(const f32x4*)(&nw_lds[k + 4]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float x0 = o.x[j][0][e], x1 = o.x[j][1][e];
+                    ss = fmaf(x0, x0, ss);
+                    ss = fmaf(x1, x1, ss);
+                    o.a[j][e] = (bf16_t)(x0 * w0[e]);
+                    o.a[j][4 + e] = (bf16_t)(x1 * w1[e]);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc = mfma16(o.a[j], o.b[j], acc);
     };
     // Workgroups start at different chunks (a rotation by the tile index), so that at any moment
-    // the chip reads from all columns of W and not from one: rows are a multiple of the DRAM
-    // channel interleave apart.  The order of a tile's additions still depends on N and K only.
+    // the chip reads from all columns of W and not from one.  The order of a tile's additions
+    // still depends on N and K only.
     const int rot = (int)((blockIdx.x * 5u) % (unsigned)nchunks);
     auto chunk_of = [&](int i) { int c = i + rot; return c >= nchunks ? c - nchunks : c; };
     int i = wave;
-    if (i < nchunks) load(chunk_of(i), a0, b0);
+    if (i < nchunks) load(chunk_of(i), o0);
+    if (NORM) {
+        // the norm weight goes to LDS while the first operands are on their way from HBM
+        for (int k = tid * 4; k < K; k += NW * WAVE * 4) *(f32x4*)(&nw_lds[k]) = *(const f32x4*)(norm_w + k);
+        __syncthreads();
+    }
     for (; i < nchunks; i += 2 * NW) {
         const bool more = i + NW < nchunks;
-        if (more) load(chunk_of(i + NW), a1, b1);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc = mfma16(a0[j], b0[j], acc);
+        if (more) load(chunk_of(i + NW), o1);
+        multiply(chunk_of(i), o0);
         if (more) {
-            if (i + 2 * NW < nchunks) load(chunk_of(i + 2 * NW), a0, b0);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc = mfma16(a1[j], b1[j], acc);
+            if (i + 2 * NW < nchunks) load(chunk_of(i + 2 * NW), o0);
+            multiply(chunk_of(i + NW), o1);
         }
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) red[wave][lane][e] = acc[e];
+    if (NORM) {
+        ss += __shfl_xor(ss, 16, WAVE);
+        ss += __shfl_xor(ss, 32, WAVE);
+        if (g == 0) ssq[wave][r16] = ss;
+    }
     __syncthreads();
     if (tid < 256) {
         // thread -> (lane l, element e) of the 16x16 tile; the wave partials in wave order
@@ -176,7 +245,14 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const bf1
 #pragma unroll
         for (int w = 1; w < NW; ++w) v += red[w][l][e];
         const long long row = (l / 16) * 4 + e, col = n0 + (l % 16);
-        if (row < M && col < N) store_out<MODE>(Y, row * N + col, v);
+        if (NORM) {
+            float total = ssq[0][row];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) total += ssq[w][row];
+            v *= 1.0f / sqrtf(total / (float)K + eps);
+        }
+        const float partner = (MODE == OUT_SWIGLU) ? __shfl_xor(v, 4, WAVE) : 0.f;   // thread tid ^ 4 holds column col ^ 1
+        store_elem<MODE>(Y, row, col, M, N, v, partner);
     }
 }
 
@@ -256,9 +332,9 @@ __global__ __launch_bounds__(SK_NT) void gemm_bf16_skinny64_kernel(const bf16_t*
     }
 
     const long long col = (long long)tile * 64 + wave * 16 + r16;
-    if (col >= N) return;
     if (n_slices > 1) {
         // partial tile of this slice: ws[slice][row][col]
+        if (col >= N) return;
         float* mine = ws + (long long)slice * (MT * 16) * N;
 #pragma unroll
         for (int i = 0; i < MT; ++i)
@@ -271,7 +347,9 @@ __global__ __launch_bounds__(SK_NT) void gemm_bf16_skinny64_kernel(const bf16_t*
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const long long row = i * 16 + g * 4 + e;
-            if (row < M) store_out<MODE>(Y, row * N + col, acc[i][e]);
+            const float v = acc[i][e];
+            const float partner = (MODE == OUT_SWIGLU) ? __shfl_xor(v, 1, WAVE) : 0.f;
+            store_elem<MODE>(Y, row, col, M, N, v, partner);
         }
 }
 
@@ -280,6 +358,19 @@ template <int MODE>
 __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* __restrict__ Y, int M, int N, int rows_padded,
                                      int n_slices) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (MODE == OUT_SWIGLU) {
+        const int F = N / 2;
+        if (i >= (long long)M * F) return;
+        const long long row = i / F, f = i - row * F;
+        float gt = 0.f, up = 0.f;
+        for (int s = 0; s < n_slices; ++s) {
+            const float* p = ws + ((long long)s * rows_padded + row) * N + 2 * f;
+            gt += p[0];
+            up += p[1];
+        }
+        ((bf16_t*)Y)[i] = (bf16_t)silu_mul(gt, up);
+        return;
+    }
     if (i >= (long long)M * N) return;
     float v = 0.f;
     for (int s = 0; s < n_slices; ++s) v += ws[(long long)s * rows_padded * N + i];
@@ -289,14 +380,14 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* __restr
 struct SkinnyPlan { int tiles, waves, slices, chunks_per_slice; long long ws_floats; };
 
 // How a skinny product is cut.  Depends on N and K (and on which of the two kernels M selects).
-SkinnyPlan plan_skinny(int M, int N, int K) {
+SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16) {
     const int nchunks = ceil_div(K, SK_CHUNK);
     SkinnyPlan p;
     p.slices = 1; p.chunks_per_slice = nchunks; p.ws_floats = 0; p.waves = 4;
     if (M <= 16) {
         p.tiles = ceil_div(N, 16);
         // enough waves in flight to cover the latency of HBM, at least one chunk a wave
-        while (p.waves < 16 && p.tiles * p.waves < 3072 && nchunks >= 2 * p.waves) p.waves *= 2;
+        while (p.waves < max_waves && p.tiles * p.waves < 3072 && nchunks >= 2 * p.waves) p.waves *= 2;
     } else {
         const int mt = ceil_div(M, 16);
         p.tiles = ceil_div(N, 64);
@@ -309,15 +400,22 @@ SkinnyPlan plan_skinny(int M, int N, int K) {
     return p;
 }
 
+template <int MODE, bool NORM>
+int launch_skinny16(const void* X, const bf16_t* W, void* Y, int M, int N, int K, const float* norm_w, float eps,
+                    const int* rows, hipStream_t stream) {
+    const SkinnyPlan p = plan_skinny(M, N, K, NORM ? 8 : 16);    // the fused norm needs more registers a wave
+    dim3 grid(p.tiles);
+    const size_t lds = NORM ? (size_t)K * sizeof(float) : 0;
+#define GO(NW) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<NW, MODE, NORM>), grid, dim3(NW * WAVE), lds, stream, X, W, Y, M, N, K, norm_w, eps, rows)
+    if (p.waves == 4) GO(4); else if (p.waves == 8) GO(8); else GO(16);
+#undef GO
+    return launch_status();
+}
+
 template <int MODE>
 int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, float* ws, hipStream_t stream) {
-    if (M <= 16) {
-        const SkinnyPlan p = plan_skinny(M, N, K);
-        dim3 grid(p.tiles);
-        if (p.waves == 4) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<4, MODE>), grid, dim3(256), 0, stream, X, W, Y, M, N, K);
-        else if (p.waves == 8) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<8, MODE>), grid, dim3(512), 0, stream, X, W, Y, M, N, K);
-        else hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<16, MODE>), grid, dim3(1024), 0, stream, X, W, Y, M, N, K);
-    } else if (M <= 64) {
+    if (M <= 16) return launch_skinny16<MODE, false>(X, W, Y, M, N, K, nullptr, 0.f, nullptr, stream);
+    if (M <= 64) {
         const SkinnyPlan p = plan_skinny(M, N, K);
         dim3 grid(p.tiles, p.slices), block(SK_NT);
         if (p.slices > 1 && !ws) return -4;
@@ -328,7 +426,7 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
         if (p.slices > 1) {
             int rc = launch_status();
             if (rc) return rc;
-            const long long n = (long long)M * N;
+            const long long n = (long long)M * (MODE == OUT_SWIGLU ? N / 2 : N);
             hipLaunchKernelGGL((splitk_reduce_kernel<MODE>), dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, stream,
                                (const float*)ws, Y, M, N, mt * 16, p.slices);
         }
@@ -358,5 +456,26 @@ TUFF_EXPORT int tuff_gemm_bf16(const void* X, const void* W, void* Y, int M, int
     if (mode == OUT_BF16) return launch_mode<OUT_BF16>(x, w, Y, M, N, K, ws, stream);
     if (mode == OUT_F32) return launch_mode<OUT_F32>(x, w, Y, M, N, K, ws, stream);
     if (mode == OUT_F32_ACCUM) return launch_mode<OUT_F32_ACCUM>(x, w, Y, M, N, K, ws, stream);
+    if (mode == OUT_SWIGLU) {
+        if (N % 2) return -2;
+        return launch_mode<OUT_SWIGLU>(x, w, Y, M, N, K, ws, stream);
+    }
+    return -3;
+}
+
+// Y (=|+=) RMSNorm(X[rows]) * W^T for M <= 16 rows: X float32 [*, K], norm_w float32 [K], rows
+// optional int32 [M].  K must be a multiple of 8 and at most 8192 (the norm weight sits in LDS).
+TUFF_EXPORT int tuff_gemm_bf16_normed(const float* X, const int* rows, const float* norm_w, float eps, const void* W,
+                                      void* Y, int M, int N, int K, int mode, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K % 8 != 0 || K > 8192 || M > 16) return -2;
+    const bf16_t* w = (const bf16_t*)W;
+    if (mode == OUT_BF16) return launch_skinny16<OUT_BF16, true>(X, w, Y, M, N, K, norm_w, eps, rows, stream);
+    if (mode == OUT_F32) return launch_skinny16<OUT_F32, true>(X, w, Y, M, N, K, norm_w, eps, rows, stream);
+    if (mode == OUT_F32_ACCUM) return launch_skinny16<OUT_F32_ACCUM, true>(X, w, Y, M, N, K, norm_w, eps, rows, stream);
+    if (mode == OUT_SWIGLU) {
+        if (N % 2) return -2;
+        return launch_skinny16<OUT_SWIGLU, true>(X, w, Y, M, N, K, norm_w, eps, rows, stream);
+    }
     return -3;
 }

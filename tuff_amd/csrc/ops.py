@@ -15,7 +15,7 @@ import torch
 from . import build
 
 DT_F32, DT_BF16 = 0, 1
-OUT_BF16, OUT_F32, OUT_F32_ACCUM = 0, 1, 2
+OUT_BF16, OUT_F32, OUT_F32_ACCUM, OUT_SWIGLU = 0, 1, 2, 3
 
 _c_int, _c_float, _c_void_p, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
 
@@ -38,6 +38,8 @@ _SIGNATURES = {
     "gemm_bf16": {
         "tuff_gemm_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
         "tuff_gemm_bf16_workspace": [_c_int, _c_int, _c_int, ctypes.POINTER(_c_ll)],
+        "tuff_gemm_bf16_normed": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                                  _c_int, _c_void_p],
     },
     "rope_kv": {
         "tuff_qkv_post": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
@@ -60,6 +62,8 @@ _SIGNATURES = {
     "shortconv": {
         "tuff_shortconv_fwd": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_shortconv_decode": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p,
+                                  _c_int, _c_int, _c_int, _c_void_p],
         "tuff_shortconv_state": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                  _c_int, _c_int, _c_int, _c_void_p],
     },
@@ -174,18 +178,37 @@ def fill_u32(t: torch.Tensor, value: int = 0) -> None:
 
 
 # ------------------------------------------------------------------------------ GEMM
-def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+def _bf16_mode(out: torch.Tensor, accumulate: bool, swiglu: bool, M: int, N: int) -> int:
+    if swiglu:
+        if accumulate or out.dtype != torch.bfloat16 or N % 2:
+            raise KernelError("gemm: the SwiGLU epilogue writes bfloat16 [M, N/2] and cannot accumulate")
+        _gpu("out", out, shape=(M, N // 2))
+        return OUT_SWIGLU
+    _gpu("out", out, shape=(M, N))
+    if out.dtype == torch.float32:
+        return OUT_F32_ACCUM if accumulate else OUT_F32
+    if out.dtype == torch.bfloat16:
+        if accumulate:
+            raise KernelError("gemm: accumulation needs a float32 output")
+        return OUT_BF16
+    raise KernelError(f"gemm: unsupported output type {out.dtype}")
+
+
+def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
+         swiglu: bool = False) -> None:
     """out (=|+=) x @ w.T.  x [M, K], w [N, K] of one dtype; float32 operands give the true
     float32 product, bfloat16 operands the matrix-core product with float32 accumulation.
-    `out` is float32 (stored or accumulated into) or, for bfloat16 operands, bfloat16."""
+    `out` is float32 (stored or accumulated into) or, for bfloat16 operands, bfloat16.
+    swiglu (bfloat16 only): the rows of w are gate and up rows interleaved and out [M, N/2] is
+    silu(gate) * up."""
     M, K = x.shape
     N = w.shape[0]
     _gpu("x", x)
     _gpu("w", w, x.dtype, (N, K))
-    _gpu("out", out, shape=(M, N))
     if x.dtype == torch.float32:
-        if out.dtype != torch.float32:
-            raise KernelError("gemm: float32 operands need a float32 output")
+        if out.dtype != torch.float32 or swiglu:
+            raise KernelError("gemm: float32 operands need a float32 output and have no fused epilogue")
+        _gpu("out", out, shape=(M, N))
         _check(load("gemm_f32").tuff_gemm_f32(x.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K,
                                               int(accumulate), _stream()), "gemm_f32")
         return
@@ -193,18 +216,35 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         raise KernelError(f"gemm: unsupported operand type {x.dtype}")
     if K % 8 != 0:
         raise KernelError(f"gemm: the bfloat16 kernels need an inner size that is a multiple of 8, got {K}")
-    if out.dtype == torch.float32:
-        mode = OUT_F32_ACCUM if accumulate else OUT_F32
-    elif out.dtype == torch.bfloat16:
-        if accumulate:
-            raise KernelError("gemm: accumulation needs a float32 output")
-        mode = OUT_BF16
-    else:
-        raise KernelError(f"gemm: unsupported output type {out.dtype}")
+    mode = _bf16_mode(out, accumulate, swiglu, M, N)
     ws_floats = _gemm_workspace(M, N, K)
     ws = torch.empty(ws_floats, dtype=torch.float32, device=x.device) if ws_floats else None
     _check(load("gemm_bf16").tuff_gemm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, mode,
                                             None if ws is None else ws.data_ptr(), _stream()), "gemm_bf16")
+
+
+NORMED_MAX_ROWS, NORMED_MAX_K = 16, 8192
+
+
+def gemm_normed(x: torch.Tensor, norm_w: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor, *,
+                rows: Optional[torch.Tensor] = None, accumulate: bool = False, swiglu: bool = False) -> None:
+    """out (=|+=) rmsnorm(x[rows]) @ w.T in one kernel, for at most 16 rows: x float32 [*, K],
+    norm_w float32 [K], w bfloat16 [N, K].  The row's 1/rms scales the result, the norm weight
+    the operand."""
+    K = x.shape[1]
+    M = x.shape[0] if rows is None else rows.shape[0]
+    N = w.shape[0]
+    _gpu("x", x, torch.float32)
+    _gpu("norm_w", norm_w, torch.float32, (K,))
+    _gpu("w", w, torch.bfloat16, (N, K))
+    _opt("rows", rows, torch.int32, (M,))
+    if M > NORMED_MAX_ROWS or K > NORMED_MAX_K or K % 8:
+        raise KernelError(f"gemm_normed: at most {NORMED_MAX_ROWS} rows and an inner size that is a multiple of 8 "
+                          f"up to {NORMED_MAX_K}; got {M} rows, inner size {K}")
+    mode = _bf16_mode(out, accumulate, swiglu, M, N)
+    _check(load("gemm_bf16").tuff_gemm_bf16_normed(
+        x.data_ptr(), None if rows is None else rows.data_ptr(), norm_w.data_ptr(), float(eps), w.data_ptr(),
+        out.data_ptr(), M, N, K, mode, _stream()), "gemm_bf16_normed")
 
 
 _plans: dict = {}
@@ -375,6 +415,21 @@ def shortconv_fwd(bcx, conv_w, state, out, *, req_of_token, q_start, state_slot,
     _check(load("shortconv").tuff_shortconv_fwd(
         bcx.data_ptr(), conv_w.data_ptr(), _dt(conv_w), state.data_ptr(), out.data_ptr(), _dt(out),
         req_of_token.data_ptr(), q_start.data_ptr(), state_slot.data_ptr(), T, d, K, _stream()), "shortconv_fwd")
+
+
+def shortconv_decode(bcx, conv_w, state, out, *, state_slot, K) -> None:
+    """Output and state update in one kernel for a step in which every request has one token
+    (row r of bcx is request r's token)."""
+    R, d = out.shape
+    dt = out.dtype
+    _gpu("bcx", bcx, dt, (R, 3 * d))
+    _gpu("out", out)
+    _gpu("conv_w", conv_w, shape=(d, K))
+    _gpu("state", state, torch.float32, (None, K - 1, d))
+    _gpu("state_slot", state_slot, torch.int32, (R,))
+    _check(load("shortconv").tuff_shortconv_decode(
+        bcx.data_ptr(), conv_w.data_ptr(), _dt(conv_w), state.data_ptr(), out.data_ptr(), _dt(out),
+        state_slot.data_ptr(), R, d, K, _stream()), "shortconv_decode")
 
 
 def shortconv_state(bcx, state, *, q_start, q_len, state_slot, K) -> None:

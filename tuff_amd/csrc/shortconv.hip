@@ -70,7 +70,45 @@ __global__ void shortconv_state_kernel(const T* __restrict__ bcx, float* __restr
     }
     for (int j = 0; j < K - 1; ++j) st[(long long)j * d + c] = tmp[j];
 }
+// A step of single tokens (every request of the step has exactly one): output and new state in
+// one pass.  Thread (r, c) owns column c of request r's state, so reading the old rows and
+// writing the new ones needs no second kernel.  Same chain of operations as the two above.
+template <typename T, typename TW>
+__global__ void shortconv_decode_kernel(const T* __restrict__ bcx, const TW* __restrict__ conv_w, float* __restrict__ state,
+                                        T* __restrict__ out, const int* __restrict__ state_slot, int d, int K) {
+    const int r = blockIdx.x;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= d) return;
+    float* st = state + (long long)state_slot[r] * (K - 1) * d;
+    const T* row = bcx + (long long)r * 3 * d;
+    const float u = to_f32(row[c]) * to_f32(row[2 * d + c]);
+    float y = 0.f;
+    for (int k = 0; k < K - 1; ++k) {
+        const float s = st[(long long)k * d + c];
+        const float w = to_f32(conv_w[(long long)c * K + k]);
+        y = (k == 0) ? s * w : fmaf(s, w, y);
+        if (k > 0) st[(long long)(k - 1) * d + c] = s;
+    }
+    y = fmaf(u, to_f32(conv_w[(long long)c * K + K - 1]), y);
+    st[(long long)(K - 2) * d + c] = u;
+    out[(long long)r * d + c] = from_f32<T>(to_f32(row[d + c]) * y);
+}
 }  // namespace
+
+TUFF_EXPORT int tuff_shortconv_decode(const void* bcx, const void* conv_w, int w_dt, float* state, void* out, int dt,
+                                      const int* state_slot, int n_requests, int d, int K, hipStream_t stream) {
+    if (n_requests <= 0) return 0;
+    if (K < 2 || K - 1 > MAX_TAPS) return -2;
+    dim3 block(256), grid(n_requests, ceil_div(d, 256));
+#define LAUNCH(T, TW) hipLaunchKernelGGL((shortconv_decode_kernel<T, TW>), grid, block, 0, stream, (const T*)bcx, (const TW*)conv_w, \
+        state, (T*)out, state_slot, d, K)
+    if (dt == DT_F32 && w_dt == DT_F32) LAUNCH(float, float);
+    else if (dt == DT_F32) LAUNCH(float, bf16_t);
+    else if (w_dt == DT_F32) LAUNCH(bf16_t, float);
+    else LAUNCH(bf16_t, bf16_t);
+#undef LAUNCH
+    return launch_status();
+}
 
 TUFF_EXPORT int tuff_shortconv_fwd(const void* bcx, const void* conv_w, int w_dt, const float* state, void* out, int dt,
                                    const int* req_of_token, const int* q_start, const int* state_slot,

@@ -73,7 +73,8 @@ def pack_step(entries: Sequence[StepEntry], manager, vocab_size: int,
     R = len(entries)
     T = sum(len(e.tokens) for e in entries)
     n_groups = len(manager.groups)
-    longest = max([len(manager.block_table(e.req_id, g)) for e in entries for g in range(n_groups)] + [1])
+    tables = [[manager.block_table_array(e.req_id, g) for g in range(n_groups)] for e in entries]
+    longest = max([len(t) for ts in tables for t in ts] + [1])
     if max_blocks is None:
         max_blocks = longest
     elif max_blocks < longest:
@@ -106,16 +107,22 @@ def pack_step(entries: Sequence[StepEntry], manager, vocab_size: int,
             rows[li] = t + w
             li += 1
         for g in range(n_groups):
-            table = manager.block_table(e.req_id, g)
+            table = tables[r][g]
             sm = buf[offs[8 + 2 * g]:offs[9 + 2 * g]]
             bt = buf[offs[9 + 2 * g]:offs[10 + 2 * g]].reshape(R, max_blocks)
             bt[r, :len(table)] = table
             bt[r, len(table):] = -1
-            pos = np.arange(past, total)
-            pages = np.asarray(table, dtype=np.int64)[pos // ps] if n else np.zeros(0, dtype=np.int64)
-            if n and pages.min() < 0:
-                raise RuntimeError(f"request {e.req_id!r}: a token would be written to a freed page")
-            sm[t:t + n] = pages * ps + pos % ps
+            if n == 1:
+                page = int(table[past // ps])
+                if page < 0:
+                    raise RuntimeError(f"request {e.req_id!r}: a token would be written to a freed page")
+                sm[t] = page * ps + past % ps
+            elif n:
+                pos = np.arange(past, total)
+                pages = table[pos // ps].astype(np.int64)
+                if pages.min() < 0:
+                    raise RuntimeError(f"request {e.req_id!r}: a token would be written to a freed page")
+                sm[t:t + n] = pages * ps + pos % ps
         t += n
         max_q, max_ctx = max(max_q, n), max(max_ctx, total)
     return PackedStep(buf, offs, T, R, n_logits, n_groups, max_blocks, max_q, max_ctx, q_len.copy(), ctx_len.copy())

@@ -44,6 +44,15 @@ class Request:
     def tokens(self) -> list:
         return self.prompt + self.output
 
+    def token_slice(self, start: int, n: int) -> list:
+        """tokens()[start:start + n] without building the whole list."""
+        np_ = len(self.prompt)
+        if start >= np_:
+            return self.output[start - np_:start - np_ + n]
+        if start + n <= np_:
+            return self.prompt[start:start + n]
+        return self.prompt[start:] + self.output[:start + n - np_]
+
     def remaining(self) -> int:
         return len(self.prompt) + len(self.output) - self.num_computed
 
@@ -151,7 +160,8 @@ class Scheduler:
         out: list[Scheduled] = []
 
         # running requests, decoding ones first, then prompts in admission order
-        order = sorted(self.running, key=lambda r: (r.remaining() != 1, self.running.index(r)))
+        rank = {id(r): i for i, r in enumerate(self.running)}
+        order = sorted(self.running, key=lambda r: (r.remaining() != 1, rank[id(r)]))
         for req in order:
             if req not in self.running or budget == 0:       # preempted meanwhile / nothing left
                 continue
@@ -182,7 +192,7 @@ class Scheduler:
             if n == 0:
                 continue
             self._promise(req, n, promised)
-            toks = req.tokens()[req.num_computed:req.num_computed + n]
+            toks = req.token_slice(req.num_computed, n)
             out.append(Scheduled(req, req.num_computed, toks, req.num_computed + n == len(req.prompt) + len(req.output)))
             budget -= n
 
@@ -210,7 +220,7 @@ class Scheduler:
             req.status = RUNNING
             self.running.append(req)
             self._promise(req, n, promised)
-            toks = req.tokens()[:n]
+            toks = req.token_slice(0, n)
             out.append(Scheduled(req, 0, toks, n == len(req.prompt) + len(req.output)))
             budget -= n
         return out

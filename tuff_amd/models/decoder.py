@@ -122,8 +122,14 @@ class DecoderModel:
             self.blocks[run.block].forward(x, ctx, cache_views.get(run.cache), run.writes)
         if ctx.n_logits == 0:
             return None
-        h = self.final_norm.forward(x, rows=ctx.logit_rows)
         logits = torch.empty(ctx.n_logits, self.vocab_size, dtype=torch.float32, device=rt.device)
+        if (hasattr(self.final_norm, "pending") and self.head.dtype == torch.bfloat16
+                and ctx.n_logits <= ops.NORMED_MAX_ROWS and self.hidden_size <= ops.NORMED_MAX_K
+                and self.hidden_size % 8 == 0):
+            fn = self.final_norm
+            ops.gemm_normed(x, fn.weight_f32, fn.eps, self.head, logits, rows=ctx.logit_rows)
+            return logits
+        h = self.final_norm.forward(x, rows=ctx.logit_rows)
         if h.dtype != self.head.dtype:
             h32 = torch.empty(h.shape, dtype=torch.float32, device=rt.device)
             ops.cast(h, h32)

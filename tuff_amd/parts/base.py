@@ -68,6 +68,10 @@ class Part:
     #: the host, so that a step through this part can be recorded into a graph and replayed.
     graph_safe = False
 
+    #: True if forward() may be handed a parts.norm.PendingNorm in place of the normed tensor h
+    #: (the part passes it straight to a Linear, which can run the norm inside its kernel).
+    accepts_pending_norm = False
+
 
 class Norm(Part):
     """forward(x float32 [T, d], rows=None) -> [T or len(rows), d] in the compute dtype."""

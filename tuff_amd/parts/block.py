@@ -38,8 +38,16 @@ class PreNormBlock(Block):
             p.bind(weights, rt)
 
     def forward(self, x, ctx, cache, write_cache: bool = True) -> None:
-        h = self.norm1.forward(x)
+        h = self._normed(self.norm1, x, self.mixer)
         self.mixer.forward(h, ctx, cache, x, write_cache)
         if self.ffn is not None:
-            h = self.norm2.forward(x)
+            h = self._normed(self.norm2, x, self.ffn)
             self.ffn.forward(h, ctx, x)
+
+    @staticmethod
+    def _normed(norm, x, consumer):
+        """The norm of x for `consumer`: left pending if both sides know how (the consumer's first
+        projection then runs the norm inside its kernel), else computed now."""
+        if consumer.accepts_pending_norm and hasattr(norm, "pending"):
+            return norm.pending(x)
+        return norm.forward(x)

@@ -14,7 +14,11 @@ from .base import Runtime, WeightDecl
 
 class Linear:
     def __init__(self, names: Sequence[str] | str, in_features: int,
-                 out_features: Sequence[int] | int, aliases: Sequence[Sequence[str]] | None = None):
+                 out_features: Sequence[int] | int, aliases: Sequence[Sequence[str]] | None = None,
+                 swiglu_pair: bool = False):
+        """swiglu_pair: the two stacked tensors are the gate and the up matrix of a SwiGLU; with
+        bfloat16 weights their rows are interleaved so that forward(..., swiglu=True) can apply
+        silu(gate) * up in the product's epilogue."""
         self.names = [names] if isinstance(names, str) else list(names)
         outs = [out_features] if isinstance(out_features, int) else list(out_features)
         if len(outs) != len(self.names):
@@ -23,6 +27,10 @@ class Linear:
         self.out_features = sum(self.outs)
         self.aliases = [tuple(a) for a in aliases] if aliases else [()] * len(self.names)
         self.weight: Optional[torch.Tensor] = None
+        self.swiglu_pair = bool(swiglu_pair)
+        if self.swiglu_pair and (len(self.names) != 2 or self.outs[0] != self.outs[1]):
+            raise ValueError("a SwiGLU pair is two tensors of one shape")
+        self.interleaved = False
 
     def weight_decls(self) -> list[WeightDecl]:
         return [WeightDecl(n, (o, self.in_features), "normal", aliases=a)
@@ -36,34 +44,60 @@ class Linear:
         else:
             if len({w.dtype for w in ws}) != 1:
                 ws = [w.to(torch.float32) for w in ws]
-            self.weight = torch.cat(ws, dim=0).contiguous()
+            if self.swiglu_pair and ws[0].dtype == torch.bfloat16:
+                self.weight = torch.stack(ws, dim=1).reshape(self.out_features, self.in_features).contiguous()
+                self.interleaved = True
+            else:
+                self.weight = torch.cat(ws, dim=0).contiguous()
         if self.weight.dtype == torch.bfloat16 and self.in_features % 8 != 0:
             raise ValueError(f"{self.names[0]}: the bfloat16 matrix kernels need an input size that is a "
                              f"multiple of 8, got {self.in_features}")
 
-    def forward(self, x: torch.Tensor, *, out_dtype: Optional[torch.dtype] = None,
-                accumulate_into: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-        """x [T, in] in the compute dtype.  Returns a new [T, out] tensor of `out_dtype`
-        (default: the compute dtype), or adds into `accumulate_into` (float32) and returns None."""
+    def forward(self, x, *, out_dtype: Optional[torch.dtype] = None,
+                accumulate_into: Optional[torch.Tensor] = None, swiglu: bool = False) -> Optional[torch.Tensor]:
+        """x [T, in] in the compute dtype, or a PendingNorm.  Returns a new [T, out] tensor of
+        `out_dtype` (default: the compute dtype), or adds into `accumulate_into` (float32) and
+        returns None.  swiglu (interleaved pairs only): returns silu(gate) * up, [T, out/2]."""
+        from .norm import PendingNorm
         w = self.weight
-        T = x.shape[0]
-        if x.dtype != w.dtype:
-            # a weight stored in 32-bit stays so: run this product in float32
-            if w.dtype != torch.float32:
-                raise TypeError(f"{self.names[0]}: activation {x.dtype} with weight {w.dtype}")
-            x32 = torch.empty(x.shape, dtype=torch.float32, device=x.device)
-            ops.cast(x, x32)
-            x = x32
+        if swiglu and not self.interleaved:
+            raise TypeError(f"{self.names[0]}: no fused SwiGLU for this weight")
+        pending = x if isinstance(x, PendingNorm) else None
+        if pending is not None:
+            T = pending.shape[0]
+            fused = (w.dtype == torch.bfloat16 and T <= ops.NORMED_MAX_ROWS
+                     and self.in_features <= ops.NORMED_MAX_K and self.in_features % 8 == 0)
+            if not fused:
+                x, pending = pending.tensor(), None
+        if pending is None:
+            T = x.shape[0]
+            if x.dtype != w.dtype:
+                # a weight stored in 32-bit stays so: run this product in float32
+                if w.dtype != torch.float32:
+                    raise TypeError(f"{self.names[0]}: activation {x.dtype} with weight {w.dtype}")
+                x32 = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+                ops.cast(x, x32)
+                x = x32
+
+        def product(out, accumulate=False):
+            if pending is not None:
+                ops.gemm_normed(pending.x, pending.norm.weight_f32, pending.norm.eps, w, out, rows=pending.rows,
+                                accumulate=accumulate, swiglu=swiglu)
+            else:
+                ops.gemm(x, w, out, accumulate=accumulate, swiglu=swiglu)
+
+        dev = w.device
         if accumulate_into is not None:
-            ops.gemm(x, w, accumulate_into, accumulate=True)
+            product(accumulate_into, accumulate=True)
             return None
         want = out_dtype or self.rt.dtype
+        width = self.out_features // 2 if swiglu else self.out_features
         if w.dtype == torch.float32 and want != torch.float32:
-            y32 = torch.empty(T, self.out_features, dtype=torch.float32, device=x.device)
-            ops.gemm(x, w, y32)
-            y = torch.empty(T, self.out_features, dtype=want, device=x.device)
+            y32 = torch.empty(T, width, dtype=torch.float32, device=dev)
+            product(y32)
+            y = torch.empty(T, width, dtype=want, device=dev)
             ops.cast(y32, y)
             return y
-        y = torch.empty(T, self.out_features, dtype=want, device=x.device)
-        ops.gemm(x, w, y)
+        y = torch.empty(T, width, dtype=want, device=dev)
+        product(y)
         return y

@@ -9,6 +9,30 @@ from ..csrc import ops
 from .base import NORMS, Norm, Runtime, WeightDecl
 
 
+class PendingNorm:
+    """An RMSNorm that has not run yet: the float32 rows, the weight and eps.  A projection that
+    can apply the norm inside its own kernel takes it as it is; anything else calls tensor(),
+    which runs the norm kernel once."""
+
+    def __init__(self, norm: "RMSNorm", x: torch.Tensor, rows: Optional[torch.Tensor]):
+        self.norm, self.x, self.rows = norm, x, rows
+        self._tensor: Optional[torch.Tensor] = None
+
+    @property
+    def shape(self):
+        n = self.x.shape[0] if self.rows is None else self.rows.shape[0]
+        return (n, self.norm.dim)
+
+    @property
+    def dtype(self):
+        return self.norm.rt.dtype
+
+    def tensor(self) -> torch.Tensor:
+        if self._tensor is None:
+            self._tensor = self.norm.forward(self.x, self.rows)
+        return self._tensor
+
+
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
     graph_safe = True
@@ -26,6 +50,11 @@ class RMSNorm(Norm):
     def bind(self, weights, rt: Runtime):
         self.rt = rt
         self.weight = weights[self.name]
+        self.weight_f32 = self.weight if self.weight.dtype == torch.float32 else self.weight.float()
+
+    def pending(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> PendingNorm:
+        """The norm of x as a PendingNorm, for consumers that say they accept one."""
+        return PendingNorm(self, x, rows)
 
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         n = x.shape[0] if rows is None else rows.shape[0]

@@ -19,6 +19,7 @@ MAX_KERNEL = 17      # the state kernel keeps K-1 <= 16 rows in registers
 @MIXERS.register("shortconv")
 class ShortConvMixer(Mixer):
     graph_safe = True
+    accepts_pending_norm = True
 
     def __init__(self, hidden_size: int, kernel_size: int, *, names: dict[str, str],
                  aliases: dict[str, tuple] | None = None):
@@ -54,6 +55,11 @@ class ShortConvMixer(Mixer):
         T = h.shape[0]
         bcx = self.in_proj.forward(h)
         y = self.rt.empty(T, self.d)
+        if write_cache and ctx.max_q_len == 1:
+            # single tokens only: one kernel reads the state, writes the output and the new state
+            ops.shortconv_decode(bcx, self.conv_w, cache.state, y, state_slot=ctx.state_slot, K=self.K)
+            self.out_proj.forward(y, accumulate_into=residual)
+            return
         ops.shortconv_fwd(bcx, self.conv_w, cache.state, y, req_of_token=ctx.req_of_token,
                           q_start=ctx.q_start, state_slot=ctx.state_slot, K=self.K)
         if write_cache:
