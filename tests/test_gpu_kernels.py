@@ -117,6 +117,39 @@ def test_gemm_with_the_norm_inside(gpu, M, N, K, use_rows):
         assert torch.equal(one[0], out[M - 1])
 
 
+@pytest.mark.parametrize("M,d,K1,N2", [(1, 64, 192, 512), (8, 2048, 8192, 6144), (16, 240, 328, 777 * 2), (5, 96, 96, 40)])
+def test_gemm_that_prepares_the_next_norm(gpu, M, d, K1, N2):
+    """residual += a @ w1.T leaves bf16(residual * norm weight) and per-tile row sums of squares;
+    the next product scales its rows by them: together rmsnorm(residual) @ w2.T."""
+    from tuff_amd.csrc import ops
+    a = _r(M, K1, seed=1, dtype=torch.bfloat16)
+    w1 = _r(d, K1, seed=2, scale=0.05, dtype=torch.bfloat16)
+    res0 = _r(M, d, seed=3)
+    nw = 1 + _r(d, seed=4, scale=0.1)
+    w2 = _r(N2, d, seed=5, scale=0.05, dtype=torch.bfloat16)
+    eps = 1e-5
+    res = res0.to(gpu)
+    xw = torch.empty(M, d, dtype=torch.bfloat16, device=gpu)
+    ss = torch.full((-(-d // 16), 16), float("nan"), device=gpu)
+    ops.gemm_accum_emit(a.to(gpu), w1.to(gpu), res, nw.to(gpu), xw, ss)
+    want_res = res0.double() + a.double() @ w1.double().T
+    assert (res.cpu().double() - want_res).abs().max() <= 1e-5 * float(want_res.abs().max()) + 1e-6 * K1
+    plain_acc = res0.to(gpu)
+    ops.gemm(a.to(gpu), w1.to(gpu), plain_acc, accumulate=True)
+    assert torch.equal(plain_acc, res)                       # the residual itself is what the plain product gives
+    assert (xw.cpu().double() - want_res * nw.double()).abs().max() <= 2 ** -8 * float((want_res * nw).abs().max())
+    assert (ss.cpu().double()[:, :M].sum(0) - (want_res ** 2).sum(1)).abs().max() <= 1e-4 * float((want_res ** 2).sum(1).max())
+    want = plain.rms_norm(want_res, nw.double(), eps) @ w2.double().T
+    out = torch.empty(M, N2, device=gpu)
+    ops.gemm_scaled(xw, ss, eps, w2.to(gpu), out)
+    assert (out.cpu().double() - want).abs().max() <= 2 ** -7 * float(want.abs().max())
+    sw = torch.empty(M, N2 // 2, device=gpu, dtype=torch.bfloat16)
+    ops.gemm_scaled(xw, ss, eps, w2.to(gpu), sw, swiglu=True)
+    g, u = want[:, 0::2], want[:, 1::2]
+    ref = g / (1 + torch.exp(-g)) * u
+    assert (sw.cpu().double() - ref).abs().max() <= 2 ** -6 * max(float(ref.abs().max()), 0.1 * float(want.abs().max()))
+
+
 def test_gemm_refuses_what_it_cannot_do(gpu):
     from tuff_amd.csrc import ops
     x = torch.zeros(2, 12, dtype=torch.bfloat16, device=gpu)

@@ -147,30 +147,42 @@ constexpr int SK_CHUNK = 128;
 // Loads run one chunk ahead.  The wave partials are added in wave order through LDS.  NW is
 // chosen from N and K only.
 //
-// NORM: X is the float32 residual stream and the product is taken of its RMSNorm,
+// The product may be taken of the RMSNorm of the float32 residual stream x,
 //   y[m, n] = (1 / sqrt(mean_k x[m,k]^2 + eps)) * sum_k bf16(x[m,k] * w[k]) W[n,k]:
-// the norm weight is applied to the operand, the row's scale to the result, and the sum of
-// squares is taken from the very values the workgroup loads anyway (in float32, lane partials
-// in a fixed butterfly, then waves in wave order).  `rows` (optional) gathers rows of X.
-template <int NW, int MODE, bool NORM>
+// the norm weight is applied to the operand, the row's scale to the result.
+//  * NORM_INSIDE: X is x itself; the operand is formed and the sum of squares taken from the
+//    values the workgroup loads anyway (lane partials in a fixed butterfly, waves in wave
+//    order).  `rows` (optional) gathers rows of x.
+//  * NORM_SCALED: X is bf16(x * w), made by the product that last added into x (below), and
+//    ss_in [n_ss][16] holds that product's per-tile sums of squares of each row; this kernel
+//    adds them in tile order and scales its result.  Costs no more than the plain product.
+// EMIT (with OUT_F32_ACCUM): after y += ..., the new y is also written as bf16(y * emit_nw[col])
+// to emit_xw [M, N], and the tile's sums of squares of each row to emit_ss [tile][16], for the
+// NORM_SCALED product that follows.
+enum : int { NORM_NONE = 0, NORM_INSIDE = 1, NORM_SCALED = 2 };
+
+template <int NW, int MODE, int NORM, bool EMIT>
 __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const void* __restrict__ Xv, const bf16_t* __restrict__ W,
                                                                        void* __restrict__ Y, int M, int N, int K,
                                                                        const float* __restrict__ norm_w, float eps,
-                                                                       const int* __restrict__ rows) {
+                                                                       const int* __restrict__ rows,
+                                                                       const float* __restrict__ ss_in, int n_ss,
+                                                                       const float* __restrict__ emit_nw,
+                                                                       bf16_t* __restrict__ emit_xw, float* __restrict__ emit_ss) {
     __shared__ float red[NW][WAVE][4];
-    __shared__ float ssq[NW][16];
-    extern __shared__ __attribute__((aligned(16))) float nw_lds[];       // NORM: the norm weight, K floats
+    __shared__ float ssq[16][16];                                        // [wave or part][row]
+    extern __shared__ __attribute__((aligned(16))) float nw_lds[];       // NORM_INSIDE: the norm weight, K floats
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
     const int r16 = lane % 16, g = lane / 16;
     const long long n0 = (long long)blockIdx.x * 16;
     const int nchunks = (K + SK_CHUNK - 1) / SK_CHUNK;
     const bf16_t* X = (const bf16_t*)Xv;
     const float* xrow = nullptr;
-    if (NORM && r16 < M) xrow = (const float*)Xv + (long long)(rows ? rows[r16] : r16) * K;
+    if (NORM == NORM_INSIDE && r16 < M) xrow = (const float*)Xv + (long long)(rows ? rows[r16] : r16) * K;
 
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     float ss = 0.f;
-    struct Operands { bf16x8 a[4]; bf16x8 b[4]; f32x4 x[NORM ? 4 : 1][2]; };
+    struct Operands { bf16x8 a[4]; bf16x8 b[4]; f32x4 x[NORM == NORM_INSIDE ? 4 : 1][2]; };
     Operands o0, o1;
     auto load = [&](int c, Operands& o) {
         // instruction j of the wave reads bytes 64 j .. 64 j + 63 of the chunk of each of its 16 rows
@@ -180,7 +192,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int k = kb + j * 32;
-            if (NORM) {
+            if (NORM == NORM_INSIDE) {
                 const bool ok = xrow != nullptr && k < K;
                 o.x[j][0] = ok ? *(const f32x4*)(xrow + k) : f32x4{0.f, 0.f, 0.f, 0.f};
                 o.x[j][1] = ok ? *(const f32x4*)(xrow + k + 4) : f32x4{0.f, 0.f, 0.f, 0.f};
@@ -190,7 +202,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
         }
     };
     auto multiply = [&](int c, Operands& o) {
-        if (NORM) {
+        if (NORM == NORM_INSIDE) {
             const int kb = c * SK_CHUNK + g * 8;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -216,10 +228,17 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
     auto chunk_of = [&](int i) { int c = i + rot; return c >= nchunks ? c - nchunks : c; };
     int i = wave;
     if (i < nchunks) load(chunk_of(i), o0);
-    if (NORM) {
+    if (NORM == NORM_INSIDE) {
         // the norm weight goes to LDS while the first operands are on their way from HBM
         for (int k = tid * 4; k < K; k += NW * WAVE * 4) *(f32x4*)(&nw_lds[k]) = *(const f32x4*)(norm_w + k);
         __syncthreads();
+    }
+    if (NORM == NORM_SCALED && tid < 256) {
+        // 16 parts x 16 rows: part p adds the tiles p, p + 16, ... of its row
+        const int row = tid % 16, part = tid / 16;
+        float t = 0.f;
+        for (int j = part; j < n_ss; j += 16) t += ss_in[(long long)j * 16 + row];
+        ssq[part][row] = t;
     }
     for (; i < nchunks; i += 2 * NW) {
         const bool more = i + NW < nchunks;
@@ -232,7 +251,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) red[wave][lane][e] = acc[e];
-    if (NORM) {
+    if (NORM == NORM_INSIDE) {
         ss += __shfl_xor(ss, 16, WAVE);
         ss += __shfl_xor(ss, 32, WAVE);
         if (g == 0) ssq[wave][r16] = ss;
@@ -245,14 +264,32 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
 #pragma unroll
         for (int w = 1; w < NW; ++w) v += red[w][l][e];
         const long long row = (l / 16) * 4 + e, col = n0 + (l % 16);
-        if (NORM) {
+        if (NORM != NORM_NONE) {
+            constexpr int PARTS = NORM == NORM_INSIDE ? NW : 16;
             float total = ssq[0][row];
 #pragma unroll
-            for (int w = 1; w < NW; ++w) total += ssq[w][row];
+            for (int w = 1; w < PARTS; ++w) total += ssq[w][row];
             v *= 1.0f / sqrtf(total / (float)K + eps);
         }
-        const float partner = (MODE == OUT_SWIGLU) ? __shfl_xor(v, 4, WAVE) : 0.f;   // thread tid ^ 4 holds column col ^ 1
-        store_elem<MODE>(Y, row, col, M, N, v, partner);
+        if (EMIT) {
+            // y += v; the new y also as the next norm's operand, and its square into the row's tile sum
+            float y = 0.f;
+            if (row < M && col < N) {
+                float* p = (float*)Y + row * N + col;
+                y = *p + v;
+                *p = y;
+                emit_xw[row * N + col] = (bf16_t)(y * emit_nw[col]);
+            }
+            float sq = y * y;                       // tid = (16 q + c) * 4 + e: the 16 columns c are tid bits 2..5
+            sq += __shfl_xor(sq, 4, WAVE);
+            sq += __shfl_xor(sq, 8, WAVE);
+            sq += __shfl_xor(sq, 16, WAVE);
+            sq += __shfl_xor(sq, 32, WAVE);
+            if ((l % 16) == 0) emit_ss[(long long)blockIdx.x * 16 + row] = sq;
+        } else {
+            const float partner = (MODE == OUT_SWIGLU) ? __shfl_xor(v, 4, WAVE) : 0.f;   // thread tid ^ 4 holds column col ^ 1
+            store_elem<MODE>(Y, row, col, M, N, v, partner);
+        }
     }
 }
 
@@ -400,21 +437,41 @@ SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16) {
     return p;
 }
 
-template <int MODE, bool NORM>
-int launch_skinny16(const void* X, const bf16_t* W, void* Y, int M, int N, int K, const float* norm_w, float eps,
-                    const int* rows, hipStream_t stream) {
-    const SkinnyPlan p = plan_skinny(M, N, K, NORM ? 8 : 16);    // the fused norm needs more registers a wave
+struct Skinny16Extra {
+    const float* norm_w = nullptr; float eps = 0.f; const int* rows = nullptr;       // NORM_INSIDE
+    const float* ss_in = nullptr; int n_ss = 0;                                      // NORM_SCALED (+ eps)
+    const float* emit_nw = nullptr; bf16_t* emit_xw = nullptr; float* emit_ss = nullptr;   // EMIT
+};
+
+template <int MODE, int NORM, bool EMIT>
+int launch_skinny16(const void* X, const bf16_t* W, void* Y, int M, int N, int K, const Skinny16Extra& x, hipStream_t stream) {
+    // the in-kernel norm needs more registers a wave: at most 8 waves a workgroup
+    const SkinnyPlan p = plan_skinny(M, N, K, NORM == NORM_INSIDE ? 8 : 16);
     dim3 grid(p.tiles);
-    const size_t lds = NORM ? (size_t)K * sizeof(float) : 0;
-#define GO(NW) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<NW, MODE, NORM>), grid, dim3(NW * WAVE), lds, stream, X, W, Y, M, N, K, norm_w, eps, rows)
+    const size_t lds = NORM == NORM_INSIDE ? (size_t)K * sizeof(float) : 0;
+#define GO(NW) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<NW, MODE, NORM, EMIT>), grid, dim3(NW * WAVE), lds, stream, X, W, Y, M, N, K, \
+                                  x.norm_w, x.eps, x.rows, x.ss_in, x.n_ss, x.emit_nw, x.emit_xw, x.emit_ss)
     if (p.waves == 4) GO(4); else if (p.waves == 8) GO(8); else GO(16);
 #undef GO
     return launch_status();
 }
 
+template <int NORM>
+int launch_skinny16_mode(const void* X, const bf16_t* W, void* Y, int M, int N, int K, int mode, const Skinny16Extra& x,
+                         hipStream_t stream) {
+    if (mode == OUT_BF16) return launch_skinny16<OUT_BF16, NORM, false>(X, W, Y, M, N, K, x, stream);
+    if (mode == OUT_F32) return launch_skinny16<OUT_F32, NORM, false>(X, W, Y, M, N, K, x, stream);
+    if (mode == OUT_F32_ACCUM) return launch_skinny16<OUT_F32_ACCUM, NORM, false>(X, W, Y, M, N, K, x, stream);
+    if (mode == OUT_SWIGLU) {
+        if (N % 2) return -2;
+        return launch_skinny16<OUT_SWIGLU, NORM, false>(X, W, Y, M, N, K, x, stream);
+    }
+    return -3;
+}
+
 template <int MODE>
 int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, float* ws, hipStream_t stream) {
-    if (M <= 16) return launch_skinny16<MODE, false>(X, W, Y, M, N, K, nullptr, 0.f, nullptr, stream);
+    if (M <= 16) return launch_skinny16<MODE, NORM_NONE, false>(X, W, Y, M, N, K, Skinny16Extra(), stream);
     if (M <= 64) {
         const SkinnyPlan p = plan_skinny(M, N, K);
         dim3 grid(p.tiles, p.slices), block(SK_NT);
@@ -469,13 +526,30 @@ TUFF_EXPORT int tuff_gemm_bf16_normed(const float* X, const int* rows, const flo
                                       void* Y, int M, int N, int K, int mode, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (K % 8 != 0 || K > 8192 || M > 16) return -2;
-    const bf16_t* w = (const bf16_t*)W;
-    if (mode == OUT_BF16) return launch_skinny16<OUT_BF16, true>(X, w, Y, M, N, K, norm_w, eps, rows, stream);
-    if (mode == OUT_F32) return launch_skinny16<OUT_F32, true>(X, w, Y, M, N, K, norm_w, eps, rows, stream);
-    if (mode == OUT_F32_ACCUM) return launch_skinny16<OUT_F32_ACCUM, true>(X, w, Y, M, N, K, norm_w, eps, rows, stream);
-    if (mode == OUT_SWIGLU) {
-        if (N % 2) return -2;
-        return launch_skinny16<OUT_SWIGLU, true>(X, w, Y, M, N, K, norm_w, eps, rows, stream);
-    }
-    return -3;
+    Skinny16Extra x;
+    x.norm_w = norm_w; x.eps = eps; x.rows = rows;
+    return launch_skinny16_mode<NORM_INSIDE>(X, (const bf16_t*)W, Y, M, N, K, mode, x, stream);
+}
+
+// For M <= 16 rows:  Y += X W^T, and from the new Y (the residual stream, float32 [M, N]) the
+// operand of the RMSNorm that follows: xw = bf16(Y * next_norm_w) [M, N] and ss [ceil(N/16)][16],
+// the sums of squares of each row over each tile of 16 columns.
+TUFF_EXPORT int tuff_gemm_bf16_accum_emit(const void* X, const void* W, float* Y, int M, int N, int K,
+                                          const float* next_norm_w, void* xw, float* ss, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K % 8 != 0 || M > 16) return -2;
+    Skinny16Extra x;
+    x.emit_nw = next_norm_w; x.emit_xw = (bf16_t*)xw; x.emit_ss = ss;
+    return launch_skinny16<OUT_F32_ACCUM, NORM_NONE, true>(X, (const bf16_t*)W, Y, M, N, K, x, stream);
+}
+
+// For M <= 16 rows:  Y (=|+=) (XW W^T) scaled per row by 1 / sqrt(sum_t ss[t][row] / K + eps), with
+// XW and ss as tuff_gemm_bf16_accum_emit leaves them (n_ss tiles).
+TUFF_EXPORT int tuff_gemm_bf16_scaled(const void* XW, const float* ss, int n_ss, float eps, const void* W, void* Y,
+                                      int M, int N, int K, int mode, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K % 8 != 0 || M > 16 || n_ss < 1) return -2;
+    Skinny16Extra x;
+    x.ss_in = ss; x.n_ss = n_ss; x.eps = eps;
+    return launch_skinny16_mode<NORM_SCALED>(XW, (const bf16_t*)W, Y, M, N, K, mode, x, stream);
 }

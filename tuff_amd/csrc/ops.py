@@ -38,6 +38,10 @@ _SIGNATURES = {
     "gemm_bf16": {
         "tuff_gemm_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
         "tuff_gemm_bf16_workspace": [_c_int, _c_int, _c_int, ctypes.POINTER(_c_ll)],
+        "tuff_gemm_bf16_accum_emit": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
+                                      _c_void_p, _c_void_p],
+        "tuff_gemm_bf16_scaled": [_c_void_p, _c_void_p, _c_int, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                                  _c_int, _c_void_p],
         "tuff_gemm_bf16_normed": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
                                   _c_int, _c_void_p],
     },
@@ -245,6 +249,41 @@ def gemm_normed(x: torch.Tensor, norm_w: torch.Tensor, eps: float, w: torch.Tens
     _check(load("gemm_bf16").tuff_gemm_bf16_normed(
         x.data_ptr(), None if rows is None else rows.data_ptr(), norm_w.data_ptr(), float(eps), w.data_ptr(),
         out.data_ptr(), M, N, K, mode, _stream()), "gemm_bf16_normed")
+
+
+def gemm_accum_emit(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, next_norm_w: torch.Tensor,
+                    xw: torch.Tensor, ss: torch.Tensor) -> None:
+    """residual += x @ w.T for at most 16 rows, and for the RMSNorm that follows: xw = the new
+    residual times next_norm_w as bfloat16, ss [ceil(N/16), 16] = per-tile sums of squares of each row."""
+    M, K = x.shape
+    N = w.shape[0]
+    _gpu("x", x, torch.bfloat16)
+    _gpu("w", w, torch.bfloat16, (N, K))
+    _gpu("residual", residual, torch.float32, (M, N))
+    _gpu("next_norm_w", next_norm_w, torch.float32, (N,))
+    _gpu("xw", xw, torch.bfloat16, (M, N))
+    _gpu("ss", ss, torch.float32, (-(-N // 16), 16))
+    if M > NORMED_MAX_ROWS or K % 8:
+        raise KernelError(f"gemm_accum_emit: at most {NORMED_MAX_ROWS} rows, inner size a multiple of 8")
+    _check(load("gemm_bf16").tuff_gemm_bf16_accum_emit(x.data_ptr(), w.data_ptr(), residual.data_ptr(), M, N, K,
+                                                       next_norm_w.data_ptr(), xw.data_ptr(), ss.data_ptr(),
+                                                       _stream()), "gemm_bf16_accum_emit")
+
+
+def gemm_scaled(xw: torch.Tensor, ss: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor, *,
+                accumulate: bool = False, swiglu: bool = False) -> None:
+    """out (=|+=) rmsnorm(x) @ w.T from what gemm_accum_emit left: xw = bf16(x * norm weight) and the
+    per-tile sums of squares ss; each row of the product is scaled by 1 / sqrt(sum(ss) / K + eps)."""
+    M, K = xw.shape
+    N = w.shape[0]
+    _gpu("xw", xw, torch.bfloat16)
+    _gpu("ss", ss, torch.float32, (None, 16))
+    _gpu("w", w, torch.bfloat16, (N, K))
+    if M > NORMED_MAX_ROWS or K % 8:
+        raise KernelError(f"gemm_scaled: at most {NORMED_MAX_ROWS} rows, inner size a multiple of 8")
+    mode = _bf16_mode(out, accumulate, swiglu, M, N)
+    _check(load("gemm_bf16").tuff_gemm_bf16_scaled(xw.data_ptr(), ss.data_ptr(), ss.shape[0], float(eps), w.data_ptr(),
+                                                   out.data_ptr(), M, N, K, mode, _stream()), "gemm_bf16_scaled")
 
 
 _plans: dict = {}

@@ -61,9 +61,10 @@ class PackedStep:
     max_ctx_len: int
     q_len: np.ndarray
     ctx_len: np.ndarray
+    logit_rows_identity: bool = False     # logits are wanted of every token of the step, in order
 
     def shape_key(self):
-        return (self.T, self.R, self.n_logits, self.n_groups, self.max_blocks)
+        return (self.T, self.R, self.n_logits, self.n_groups, self.max_blocks, self.logit_rows_identity)
 
 
 def pack_step(entries: Sequence[StepEntry], manager, vocab_size: int,
@@ -125,7 +126,9 @@ def pack_step(entries: Sequence[StepEntry], manager, vocab_size: int,
                 sm[t:t + n] = pages * ps + pos % ps
         t += n
         max_q, max_ctx = max(max_q, n), max(max_ctx, total)
-    return PackedStep(buf, offs, T, R, n_logits, n_groups, max_blocks, max_q, max_ctx, q_len.copy(), ctx_len.copy())
+    identity = n_logits == T and bool((rows == np.arange(T)).all())
+    return PackedStep(buf, offs, T, R, n_logits, n_groups, max_blocks, max_q, max_ctx, q_len.copy(), ctx_len.copy(),
+                      identity)
 
 
 def context_on(dev: torch.Tensor, p: PackedStep, max_ctx_len: Optional[int] = None) -> StepContext:
@@ -138,7 +141,7 @@ def context_on(dev: torch.Tensor, p: PackedStep, max_ctx_len: Optional[int] = No
                        q_start=sl(3), q_len=sl(4), ctx_len=sl(5), state_slot=sl(6), logit_rows=sl(7),
                        groups=groups, max_q_len=p.max_q_len,
                        max_ctx_len=max_ctx_len if max_ctx_len is not None else p.max_ctx_len,
-                       host={"q_len": p.q_len, "ctx_len": p.ctx_len})
+                       host={"q_len": p.q_len, "ctx_len": p.ctx_len, "logit_rows_identity": p.logit_rows_identity})
 
 
 def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int) -> StepContext:

@@ -20,6 +20,14 @@ class LayerRun:
     writes: bool = True             # False: only reads the entry, which an earlier run writes
 
 
+class _Head:
+    """Stands for the head as the consumer of the final norm."""
+    accepts_pending_norm = True
+
+
+_HEAD = _Head()
+
+
 class DecoderModel:
     def __init__(self, *, vocab_size: int, hidden_size: int, embedding: WeightDecl,
                  blocks: list[Block], final_norm: Norm, head: Optional[WeightDecl] = None,
@@ -118,16 +126,31 @@ class DecoderModel:
         rt = self.rt
         x = torch.empty(ctx.T, self.hidden_size, dtype=torch.float32, device=rt.device)
         ops.embed_rows(self.embedding, ctx.tokens, x)
-        for run in self.schedule:
-            self.blocks[run.block].forward(x, ctx, cache_views.get(run.cache), run.writes)
+        all_rows = ctx.n_logits == ctx.T and bool(ctx.host.get("logit_rows_identity", False))
+        head_fused = (hasattr(self.final_norm, "pending") and self.head.dtype == torch.bfloat16
+                      and 0 < ctx.n_logits <= ops.NORMED_MAX_ROWS and self.hidden_size <= ops.NORMED_MAX_K
+                      and self.hidden_size % 8 == 0)
+        for i, run in enumerate(self.schedule):
+            block = self.blocks[run.block]
+            if getattr(block, "takes_next_norm", False):
+                if i + 1 < len(self.schedule):
+                    nb = self.blocks[self.schedule[i + 1].block]
+                    nxt = nb.first_norm_consumer() if hasattr(nb, "first_norm_consumer") else None
+                else:
+                    nxt = (self.final_norm, _HEAD) if head_fused and all_rows else None
+                block.forward(x, ctx, cache_views.get(run.cache), run.writes, next_norm=nxt)
+            else:
+                block.forward(x, ctx, cache_views.get(run.cache), run.writes)
         if ctx.n_logits == 0:
             return None
         logits = torch.empty(ctx.n_logits, self.vocab_size, dtype=torch.float32, device=rt.device)
-        if (hasattr(self.final_norm, "pending") and self.head.dtype == torch.bfloat16
-                and ctx.n_logits <= ops.NORMED_MAX_ROWS and self.hidden_size <= ops.NORMED_MAX_K
-                and self.hidden_size % 8 == 0):
+        if head_fused:
             fn = self.final_norm
-            ops.gemm_normed(x, fn.weight_f32, fn.eps, self.head, logits, rows=ctx.logit_rows)
+            p = fn.pending(x, None if all_rows else ctx.logit_rows)
+            if p.pre is not None:
+                ops.gemm_scaled(p.pre[0], p.pre[1], fn.eps, self.head, logits)
+            else:
+                ops.gemm_normed(x, fn.weight_f32, fn.eps, self.head, logits, rows=ctx.logit_rows)
             return logits
         h = self.final_norm.forward(x, rows=ctx.logit_rows)
         if h.dtype != self.head.dtype:

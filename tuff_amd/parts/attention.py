@@ -22,6 +22,7 @@ from .linear import Linear
 @MIXERS.register("attention")
 class AttentionMixer(Mixer):
     accepts_pending_norm = True
+    adds_once_through_linear = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, *,
                  names: dict[str, str], qk_norm_eps: Optional[float] = None,

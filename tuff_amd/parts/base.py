@@ -72,6 +72,11 @@ class Part:
     #: (the part passes it straight to a Linear, which can run the norm inside its kernel).
     accepts_pending_norm = False
 
+    #: True if forward() touches the residual stream exactly once, as its last operation, through
+    #: Linear.forward(accumulate_into=residual).  The block may then let that product prepare the
+    #: operand of the norm that follows (see Linear.forward).
+    adds_once_through_linear = False
+
 
 class Norm(Part):
     """forward(x float32 [T, d], rows=None) -> [T or len(rows), d] in the compute dtype."""

@@ -37,12 +37,33 @@ class PreNormBlock(Block):
         for p in self._parts():
             p.bind(weights, rt)
 
-    def forward(self, x, ctx, cache, write_cache: bool = True) -> None:
+    takes_next_norm = True
+
+    def first_norm_consumer(self):
+        """(norm, part that consumes it) at the head of the block, for the block before this one."""
+        return self.norm1, self.mixer
+
+    def forward(self, x, ctx, cache, write_cache: bool = True, next_norm=None) -> None:
+        """next_norm: (norm, consumer) that will read x right after this block, or None."""
         h = self._normed(self.norm1, x, self.mixer)
+        self._announce(x, self.mixer, (self.norm2, self.ffn) if self.ffn is not None else next_norm)
         self.mixer.forward(h, ctx, cache, x, write_cache)
         if self.ffn is not None:
             h = self._normed(self.norm2, x, self.ffn)
+            self._announce(x, self.ffn, next_norm)
             self.ffn.forward(h, ctx, x)
+        self._announce(x, None, None)
+
+    @staticmethod
+    def _announce(x, producer, nxt) -> None:
+        """Tells the producer's last projection (through an attribute of x) which norm reads x next,
+        if producer, norm and the norm's consumer all know the protocol."""
+        ok = (producer is not None and nxt is not None and producer.adds_once_through_linear
+              and hasattr(nxt[0], "announce_operand") and nxt[1] is not None and nxt[1].accepts_pending_norm)
+        if ok:
+            x._tuff_next_norm = nxt[0]
+        elif hasattr(x, "_tuff_next_norm"):
+            del x._tuff_next_norm
 
     @staticmethod
     def _normed(norm, x, consumer):

@@ -14,6 +14,7 @@ from .linear import Linear
 class SwiGLU(FeedForward):
     graph_safe = True
     accepts_pending_norm = True
+    adds_once_through_linear = True
 
     def __init__(self, hidden_size: int, ffn_dim: int, *, names: dict[str, str],
                  aliases: dict[str, tuple] | None = None):

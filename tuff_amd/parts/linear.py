@@ -80,7 +80,10 @@ class Linear:
                 x = x32
 
         def product(out, accumulate=False):
-            if pending is not None:
+            if pending is not None and pending.pre is not None:
+                ops.gemm_scaled(pending.pre[0], pending.pre[1], pending.norm.eps, w, out,
+                                accumulate=accumulate, swiglu=swiglu)
+            elif pending is not None:
                 ops.gemm_normed(pending.x, pending.norm.weight_f32, pending.norm.eps, w, out, rows=pending.rows,
                                 accumulate=accumulate, swiglu=swiglu)
             else:
@@ -88,6 +91,15 @@ class Linear:
 
         dev = w.device
         if accumulate_into is not None:
+            nxt = getattr(accumulate_into, "_tuff_next_norm", None)
+            if (nxt is not None and pending is None and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
+                    and T <= ops.NORMED_MAX_ROWS):
+                # the norm that follows reads the sum just made: leave it its operand and row sums
+                xw = torch.empty(T, self.out_features, dtype=torch.bfloat16, device=dev)
+                ss = torch.empty(-(-self.out_features // 16), 16, dtype=torch.float32, device=dev)
+                ops.gemm_accum_emit(x, w, accumulate_into, nxt.weight_f32, xw, ss)
+                nxt.announce_operand(accumulate_into, xw, ss)
+                return None
             product(accumulate_into, accumulate=True)
             return None
         want = out_dtype or self.rt.dtype

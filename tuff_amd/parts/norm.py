@@ -14,8 +14,9 @@ class PendingNorm:
     can apply the norm inside its own kernel takes it as it is; anything else calls tensor(),
     which runs the norm kernel once."""
 
-    def __init__(self, norm: "RMSNorm", x: torch.Tensor, rows: Optional[torch.Tensor]):
+    def __init__(self, norm: "RMSNorm", x: torch.Tensor, rows: Optional[torch.Tensor], pre=None):
         self.norm, self.x, self.rows = norm, x, rows
+        self.pre = pre            # (xw, ss) left by the product that last added into x, or None
         self._tensor: Optional[torch.Tensor] = None
 
     @property
@@ -54,7 +55,17 @@ class RMSNorm(Norm):
 
     def pending(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> PendingNorm:
         """The norm of x as a PendingNorm, for consumers that say they accept one."""
-        return PendingNorm(self, x, rows)
+        pre, self._ready = None, getattr(self, "_ready", None)
+        if self._ready is not None:
+            if self._ready[0] is x and rows is None:
+                pre = self._ready[1:]
+            self._ready = None
+        return PendingNorm(self, x, rows, pre)
+
+    def announce_operand(self, x: torch.Tensor, xw: torch.Tensor, ss: torch.Tensor) -> None:
+        """Called by the product that has just added into x and, in the same kernel, written
+        xw = bf16(x * weight) and the per-tile sums of squares ss: the next pending(x) carries them."""
+        self._ready = (x, xw, ss)
 
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         n = x.shape[0] if rows is None else rows.shape[0]

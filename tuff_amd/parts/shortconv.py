@@ -20,6 +20,7 @@ MAX_KERNEL = 17      # the state kernel keeps K-1 <= 16 rows in registers
 class ShortConvMixer(Mixer):
     graph_safe = True
     accepts_pending_norm = True
+    adds_once_through_linear = True
 
     def __init__(self, hidden_size: int, kernel_size: int, *, names: dict[str, str],
                  aliases: dict[str, tuple] | None = None):
