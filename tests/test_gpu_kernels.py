@@ -359,12 +359,12 @@ def test_attention_mfma(gpu, H, Hkv, hd, ps, window):
     q = _r(T, H * hd, seed=90, dtype=dt)
     scale = 1 / math.sqrt(hd)
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
+    req_info = i32([[qs, ql, past, past + ql] for qs, ql, (past, _) in zip(q_start, q_len, reqs)])
     for nb in ([1, 2, 4] if hd <= 128 else [1, 2]):
-        blk_req, blk_col0 = ops.query_blocks(q_len, H // Hkv, nb)
+        blocks = torch.from_numpy(ops.query_blocks(q_len, H // Hkv, nb)).to(gpu)
         out = torch.full((T, H * hd), float("nan"), dtype=dt, device=gpu)
         ops.attention_mfma(q.to(gpu), kc.to(gpu), vc.to(gpu), out, block_table=table.to(gpu),
-                           blk_req=torch.from_numpy(blk_req).to(gpu), blk_col0=torch.from_numpy(blk_col0).to(gpu), nb=nb,
-                           q_start=i32(q_start), q_len=i32(q_len), positions=i32(pos), H=H, Hkv=Hkv, hd=hd,
+                           blocks=blocks, nb=nb, req_info=req_info, positions=i32(pos), H=H, Hkv=Hkv, hd=hd,
                            page_size=ps, max_ctx_len=700, window=window)
         got = out.cpu().double().reshape(T, H, hd)
         assert torch.isfinite(got).all(), nb

@@ -39,23 +39,30 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     float* __restrict__ ws_o, float* __restrict__ ws_ml,
     const int* __restrict__ block_table, int max_blocks,
-    const int* __restrict__ blk_req, const int* __restrict__ blk_col0,
-    const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ positions,
+    const int2* __restrict__ blk, const int4* __restrict__ req_info,
     int H, int Hkv, int hd, int page_size, int window, float scale, int n_parts) {
     constexpr int KC = HDP / 32;          // 32-wide chunks of the head dimension
     constexpr int DB = HDP / 16;          // 16-wide blocks of output channels
     const int part = blockIdx.x, qb = blockIdx.y, kvh = blockIdx.z;
     const int lane = threadIdx.x, n16 = lane % 16, g = lane / 16;
     const int G = H / Hkv;
-    const int r = blk_req[qb], col0 = blk_col0[qb];
-    const int t0 = q_start[r], ncols = q_len[r] * G;
+    // Every load that depends on another costs a trip to memory, so the chain is kept short:
+    // block -> request record (start, length, first position: a portion's positions are
+    // consecutive) -> the partition's page numbers, all at once -> keys and values.
+    int r = qb, col0 = 0;                  // without a block list every request is one block
+    if (blk) { const int2 b = blk[qb]; r = b.x; col0 = b.y; }
+    const int4 info = req_info[r];         // (first token of the request in the step, tokens, first position, -)
+    const int t0 = info.x, ncols = info.y * G, pos0 = info.z;
     const int* table = block_table + (long long)r * max_blocks;
+    const int key_begin = part * PART;
+    const int first_page = key_begin / page_size;
+    int my_page = -1;                      // lane i: the page of the partition's i-th block of page_size keys
+    if (lane < (PART + page_size - 1) / page_size && first_page + lane < max_blocks) my_page = table[first_page + lane];
 
     // the block's range of keys
     const int last_col = min(ncols, col0 + NB * 16) - 1;
-    const int pos_max = positions[t0 + last_col / G];
-    const int lo_min = window > 0 ? max(0, positions[t0 + col0 / G] - window + 1) : 0;
-    const int key_begin = part * PART;
+    const int pos_max = pos0 + last_col / G;
+    const int lo_min = window > 0 ? max(0, pos0 + col0 / G - window + 1) : 0;
     if (key_begin > pos_max || key_begin + PART <= lo_min) return;
     const int key_end = min(key_begin + PART, pos_max + 1);
 
@@ -69,7 +76,7 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
         const bool valid = c < ncols;
         const int tok = t0 + (valid ? c / G : 0);
         const int head = kvh * G + (valid ? c % G : 0);
-        pos_c[nb] = valid ? positions[tok] : -1;
+        pos_c[nb] = valid ? pos0 + c / G : -1;
         lo_c[nb] = (valid && window > 0) ? max(0, pos_c[nb] - window + 1) : 0;
         qrow[nb] = valid ? (long long)tok * H + head : -1;
 #pragma unroll
@@ -117,7 +124,7 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
             const int kbs = key0 + kb * 16;
             t.live[kb] = kbs <= pos_max && kbs + 15 >= lo_min;
             if (!t.live[kb]) continue;
-            const long long page = table[kbs / page_size];
+            const long long page = __shfl(my_page, kbs / page_size - first_page, WAVE);
             t.off0[kb] = kbs % page_size;
             t.base[kb] = (page * Hkv + kvh) * (long long)page_size * hd;
             if constexpr (AHEAD) {
@@ -242,14 +249,65 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
 
 // Merges the partitions of one (token, head) and writes the bfloat16 row:
 //   M = max_p m_p;  w_p = exp(m_p - M);  out = (sum_p w_p o_p) / (sum_p w_p l_p),
-// the sums over p in a fixed order (ascending p for the output, a fixed butterfly for the
-// denominator), so the result depends on the token's position only.
+// both sums over p in ascending order, so the result depends on the token's position only.
 constexpr int COMBINE_MAX_PARTS = 2048;
+
+// Up to 64 partitions: lane p keeps (m_p, l_p) in registers, weights travel by shuffle; no LDS.
+// Same arithmetic as the general kernel below.
+__global__ __launch_bounds__(WAVE) void attn_combine64_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+                                                              bf16_t* __restrict__ out, const int* __restrict__ positions,
+                                                              int H, int hd, int window, int n_parts) {
+    const long long row = blockIdx.x;                      // token * H + head
+    const int lane = threadIdx.x;
+    float m_l = -INFINITY, l_l = 0.f;
+    if (lane < n_parts) {                                  // read before the position is known: rows exist for all partitions
+        const float* ml = ws_ml + (row * n_parts + lane) * 2;
+        m_l = ml[0];
+        l_l = ml[1];
+    }
+    const int pos = positions[row / H];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int p_lo = lo / PART, p_hi = pos / PART;
+    const bool valid = lane >= p_lo && lane <= p_hi && l_l > 0.f;
+    const float M = wave_max(valid ? m_l : -INFINITY);
+    const float w_l = valid ? __expf(m_l - M) : 0.f;
+    const float wl_l = w_l * (valid ? l_l : 0.f);
+    const float* o = ws_o + row * n_parts * hd;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    float L = 0.f;                                         // both sums run over p in ascending order
+    // The loads below do not wait for the position: rows of partitions the token does not have
+    // exist too (unwritten); their weight is zero and they are skipped by a select, not a product.
+    for (int i0 = 0; i0 < n_parts; i0 += 8) {
+        float ov[8][4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int d = lane + j * WAVE;
+                ov[u][j] = (i0 + u < n_parts && d < hd) ? o[(long long)(i0 + u) * hd + d] : 0.f;
+            }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float w = __shfl(w_l, i0 + u, WAVE);
+            L += __shfl(wl_l, i0 + u, WAVE);
+            if (w > 0.f) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = fmaf(w, ov[u][j], acc[j]);
+            }
+        }
+    }
+    const float inv = 1.0f / L;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int d = lane + j * WAVE;
+        if (d < hd) out[row * hd + d] = (bf16_t)(acc[j] * inv);
+    }
+}
 
 __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                                             bf16_t* __restrict__ out, const int* __restrict__ positions,
                                                             int H, int hd, int window, int n_parts) {
-    __shared__ float wts[COMBINE_MAX_PARTS];
+    __shared__ float wts[COMBINE_MAX_PARTS], wls[COMBINE_MAX_PARTS];
     const long long row = blockIdx.x;                      // token * H + head
     const int lane = threadIdx.x;
     const int pos = positions[row / H];
@@ -259,20 +317,20 @@ __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restr
     float M = -INFINITY;
     for (int i = lane; i < np; i += WAVE) M = fmaxf(M, ml[i * 2 + 1] > 0.f ? ml[i * 2] : -INFINITY);
     M = wave_max(M);
-    float L = 0.f;
     for (int i = lane; i < np; i += WAVE) {
         const float l = ml[i * 2 + 1];
         const float w = l > 0.f ? __expf(ml[i * 2] - M) : 0.f;
         wts[i] = w;
-        L += w * l;
+        wls[i] = w * (l > 0.f ? l : 0.f);
     }
-    L = wave_sum(L);
     __syncthreads();
     const float* o = ws_o + (row * n_parts + p_lo) * hd;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    float L = 0.f;
 #pragma unroll 4
     for (int i = 0; i < np; ++i) {
         const float w = wts[i];
+        L += wls[i];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int d = lane + j * WAVE;
@@ -289,22 +347,23 @@ __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restr
 
 template <int HDP, int NB>
 void launch_partition(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, float* ws_o,
-                      float* ws_ml, const int* bt, int max_blocks, const int* blk_req, const int* blk_col0,
-                      const int* q_start, const int* q_len, const int* positions, int H, int Hkv, int hd, int ps,
-                      int window, float scale, int n_parts) {
+                      float* ws_ml, const int* bt, int max_blocks, const int2* blk, const int4* req_info,
+                      int H, int Hkv, int hd, int ps, int window, float scale, int n_parts) {
     hipLaunchKernelGGL((attn_partition_kernel<HDP, NB>), grid, dim3(WAVE), 0, stream, q, kc, vc, ws_o, ws_ml, bt, max_blocks,
-                       blk_req, blk_col0, q_start, q_len, positions, H, Hkv, hd, ps, window, scale, n_parts);
+                       blk, req_info, H, Hkv, hd, ps, window, scale, n_parts);
 }
 }  // namespace
 
-// Query blocks are listed by the host: block b holds the columns blk_col0[b] .. +16*nb-1 of request
-// blk_req[b] (a request's columns are numbered (token - q_start) * G + head within the kv group).
+// Query blocks are listed by the host: block b holds the columns blk[b].y .. +16*nb-1 of request
+// blk[b].x (a request's columns are numbered (token - its first token) * G + head within the kv
+// group); blk == null: block b is request b from column 0 (every request fits one block).
+// req_info [R]: (first token of the request in the step, its tokens, position of the first, -).
+// positions [n_tokens]: every token's position (read by the merge).
 // ws_o: float32 [n_tokens * H * n_parts * hd], ws_ml: float32 [n_tokens * H * n_parts * 2].
 // n_parts >= ceil((largest position + 1) / 256).  nb: 1, 2 or 4 column blocks a wave.
 TUFF_EXPORT int tuff_attention_mfma(const void* q, const void* k_cache, const void* v_cache, void* out,
                                     float* ws_o, float* ws_ml, const int* block_table, int max_blocks,
-                                    const int* blk_req, const int* blk_col0, int n_qblocks, int nb,
-                                    const int* q_start, const int* q_len, const int* positions,
+                                    const int* blk, int n_qblocks, int nb, const int* req_info, const int* positions,
                                     int n_tokens, int H, int Hkv, int hd, int page_size, int window, float scale,
                                     int n_parts, hipStream_t stream) {
     if (n_tokens <= 0 || n_qblocks <= 0) return 0;
@@ -314,8 +373,8 @@ TUFF_EXPORT int tuff_attention_mfma(const void* q, const void* k_cache, const vo
     const bf16_t* K = (const bf16_t*)k_cache;
     const bf16_t* V = (const bf16_t*)v_cache;
     dim3 grid(n_parts, n_qblocks, Hkv);
-#define GO(HDP, NB) launch_partition<HDP, NB>(grid, stream, Q, K, V, ws_o, ws_ml, block_table, max_blocks, blk_req, blk_col0, \
-                                              q_start, q_len, positions, H, Hkv, hd, page_size, window, scale, n_parts)
+#define GO(HDP, NB) launch_partition<HDP, NB>(grid, stream, Q, K, V, ws_o, ws_ml, block_table, max_blocks, (const int2*)blk, \
+                                              (const int4*)req_info, H, Hkv, hd, page_size, window, scale, n_parts)
 #define BY_NB(HDP) do { if (nb == 1) GO(HDP, 1); else if (nb == 2) GO(HDP, 2); else if (nb == 4) GO(HDP, 4); else return -2; } while (0)
     if (hd <= 32) BY_NB(32);
     else if (hd <= 64) BY_NB(64);
@@ -326,7 +385,11 @@ TUFF_EXPORT int tuff_attention_mfma(const void* q, const void* k_cache, const vo
 #undef GO
     int rc = launch_status();
     if (rc) return rc;
-    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)((long long)n_tokens * H)), dim3(WAVE), 0, stream,
-                       (const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, H, hd, window, n_parts);
+    if (n_parts <= WAVE)
+        hipLaunchKernelGGL(attn_combine64_kernel, dim3((unsigned)((long long)n_tokens * H)), dim3(WAVE), 0, stream,
+                           (const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, H, hd, window, n_parts);
+    else
+        hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)((long long)n_tokens * H)), dim3(WAVE), 0, stream,
+                           (const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, H, hd, window, n_parts);
     return launch_status();
 }

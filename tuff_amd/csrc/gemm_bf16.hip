@@ -180,6 +180,17 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
     const float* xrow = nullptr;
     if (NORM == NORM_INSIDE && r16 < M) xrow = (const float*)Xv + (long long)(rows ? rows[r16] : r16) * K;
 
+    // What the epilogue adds to is read now, not after the last product: a load at the end would
+    // cost one more trip to memory.
+    float y_old = 0.f, emit_w = 0.f;
+    if (MODE == OUT_F32_ACCUM && tid < 256) {
+        const long long row = (tid / 64) * 4 + tid % 4, col = n0 + (tid / 4) % 16;
+        if (row < M && col < N) {
+            y_old = ((const float*)Y)[row * N + col];
+            if (EMIT) emit_w = emit_nw[col];
+        }
+    }
+
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     float ss = 0.f;
     struct Operands { bf16x8 a[4]; bf16x8 b[4]; f32x4 x[NORM == NORM_INSIDE ? 4 : 1][2]; };
@@ -275,10 +286,9 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
             // y += v; the new y also as the next norm's operand, and its square into the row's tile sum
             float y = 0.f;
             if (row < M && col < N) {
-                float* p = (float*)Y + row * N + col;
-                y = *p + v;
-                *p = y;
-                emit_xw[row * N + col] = (bf16_t)(y * emit_nw[col]);
+                y = y_old + v;
+                ((float*)Y)[row * N + col] = y;
+                emit_xw[row * N + col] = (bf16_t)(y * emit_w);
             }
             float sq = y * y;                       // tid = (16 q + c) * 4 + e: the 16 columns c are tid bits 2..5
             sq += __shfl_xor(sq, 4, WAVE);
@@ -286,6 +296,8 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
             sq += __shfl_xor(sq, 16, WAVE);
             sq += __shfl_xor(sq, 32, WAVE);
             if ((l % 16) == 0) emit_ss[(long long)blockIdx.x * 16 + row] = sq;
+        } else if (MODE == OUT_F32_ACCUM) {
+            if (row < M && col < N) ((float*)Y)[row * N + col] = y_old + v;
         } else {
             const float partner = (MODE == OUT_SWIGLU) ? __shfl_xor(v, 4, WAVE) : 0.f;   // thread tid ^ 4 holds column col ^ 1
             store_elem<MODE>(Y, row, col, M, N, v, partner);

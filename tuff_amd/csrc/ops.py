@@ -60,7 +60,7 @@ _SIGNATURES = {
     },
     "attention_mfma": {
         "tuff_attention_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
-                                _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p,
+                                _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p],
     },
     "shortconv": {
@@ -387,10 +387,12 @@ def attention_mfma_supported(dtype, hd: int, page_size: int) -> bool:
     return dtype == torch.bfloat16 and hd % 8 == 0 and hd <= 256 and page_size % 16 == 0
 
 
-def attention_mfma(q, k_cache, v_cache, out, *, block_table, blk_req, blk_col0, nb, q_start, q_len, positions,
+def attention_mfma(q, k_cache, v_cache, out, *, block_table, blocks, nb, req_info, positions,
                    H, Hkv, hd, page_size, max_ctx_len, window=0, scale=None) -> None:
-    """Matrix-core attention over the paged bfloat16 cache.  blk_req / blk_col0 list the query
-    blocks (see query_blocks()); max_ctx_len bounds every position + 1 of the step."""
+    """Matrix-core attention over the paged bfloat16 cache.  blocks: int32 [n_blocks, 2] from
+    query_blocks(), or None when every request's columns fit one block (block b = request b).
+    req_info: int32 [R, 4] = (first token in the step, tokens, first position, -) per request.
+    max_ctx_len bounds every position + 1 of the step."""
     T = q.shape[0]
     if not attention_mfma_supported(q.dtype, hd, page_size):
         raise KernelError(f"attention_mfma: needs bfloat16, a head size that is a multiple of 8 (got {hd}) "
@@ -401,17 +403,21 @@ def attention_mfma(q, k_cache, v_cache, out, *, block_table, blk_req, blk_col0, 
     _gpu("k_cache", k_cache, torch.bfloat16, (P, Hkv, page_size, hd))
     _gpu("v_cache", v_cache, torch.bfloat16, (P, Hkv, hd, page_size))
     _gpu("block_table", block_table, torch.int32)
-    R = q_start.shape[0]
+    R = req_info.shape[0]
+    _gpu("req_info", req_info, torch.int32, (R, 4))
     if block_table.dim() != 2 or block_table.shape[0] != R:
         raise KernelError("attention_mfma: block_table must be [requests, blocks]")
     n_parts = max(1, -(-int(max_ctx_len) // ATTN_PARTITION))
     if block_table.shape[1] * page_size < int(max_ctx_len):
         raise KernelError("attention_mfma: block_table is narrower than the longest context")
-    nblk = blk_req.shape[0]
-    _gpu("blk_req", blk_req, torch.int32, (nblk,))
-    _gpu("blk_col0", blk_col0, torch.int32, (nblk,))
-    _gpu("q_start", q_start, torch.int32, (R,))
-    _gpu("q_len", q_len, torch.int32, (R,))
+    G = H // Hkv
+    if blocks is None:
+        if G > 16 * nb:
+            raise KernelError("attention_mfma: without a block list a request's columns must fit one block")
+        nblk = R
+    else:
+        nblk = blocks.shape[0]
+        _gpu("blocks", blocks, torch.int32, (nblk, 2))
     _gpu("positions", positions, torch.int32, (T,))
     if nb not in (1, 2, 4) or (hd > 128 and nb == 4) or H % Hkv:
         raise KernelError(f"attention_mfma: unsupported column blocking nb={nb} for head size {hd}")
@@ -421,22 +427,22 @@ def attention_mfma(q, k_cache, v_cache, out, *, block_table, blk_req, blk_col0, 
     ws_ml = torch.empty(T * H * n_parts * 2, dtype=torch.float32, device=q.device)
     _check(load("attention_mfma").tuff_attention_mfma(
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), ws_o.data_ptr(), ws_ml.data_ptr(),
-        block_table.data_ptr(), block_table.shape[1], blk_req.data_ptr(), blk_col0.data_ptr(), nblk, nb,
-        q_start.data_ptr(), q_len.data_ptr(), positions.data_ptr(), T, H, Hkv, hd, page_size,
+        block_table.data_ptr(), block_table.shape[1], None if blocks is None else blocks.data_ptr(), nblk, nb,
+        req_info.data_ptr(), positions.data_ptr(), T, H, Hkv, hd, page_size,
         int(window or 0), float(scale), n_parts, _stream()), "attention_mfma")
 
 
 def query_blocks(q_len, G: int, nb: int):
-    """Host lists of query blocks for attention_mfma: for request r with q_len[r] tokens the
-    columns (token, head in group) are cut into blocks of 16 * nb.  Returns (blk_req, blk_col0)
-    as int32 numpy arrays."""
+    """Host list of query blocks for attention_mfma: for request r with q_len[r] tokens the
+    columns (token, head in group) are cut into blocks of 16 * nb.  Returns int32 [n_blocks, 2]
+    = (request, first column)."""
     import numpy as np
     q_len = np.asarray(q_len, dtype=np.int64)
     per = -(-(q_len * G) // (16 * nb))
-    blk_req = np.repeat(np.arange(len(q_len)), per).astype(np.int32)
+    blk_req = np.repeat(np.arange(len(q_len)), per)
     starts = np.concatenate([[0], np.cumsum(per)])[:-1]
-    blk_col0 = ((np.arange(int(per.sum())) - np.repeat(starts, per)) * 16 * nb).astype(np.int32)
-    return blk_req, blk_col0
+    blk_col0 = (np.arange(int(per.sum())) - np.repeat(starts, per)) * 16 * nb
+    return np.stack([blk_req, blk_col0], axis=1).astype(np.int32)
 
 
 # ------------------------------------------------------------------------- short conv

@@ -40,6 +40,7 @@ class StepContext:
     ctx_len: torch.Tensor          # int32 [R] length of the request after this step
     state_slot: torch.Tensor       # int32 [R]
     logit_rows: torch.Tensor       # int32 [n_logits] indices into the step's tokens
+    req_info: torch.Tensor         # int32 [R, 4]: (q_start, q_len, position of the first token, ctx_len)
     groups: list[GroupContext]
     # host-side facts kernels may be chosen by
     max_q_len: int = 1
@@ -84,11 +85,12 @@ def pack_step(entries: Sequence[StepEntry], manager, vocab_size: int,
     ps = manager.page_size
     # [tokens | positions | req_of_token | q_start | q_len | ctx_len | slot | logit_rows |
     #  per group: slot_mapping, block_table]
-    sizes = [T, T, T, R, R, R, R, n_logits] + [T, R * max_blocks] * n_groups
+    sizes = [T, T, T, R, R, R, R, n_logits] + [T, R * max_blocks] * n_groups + [4 * R]
     offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
     buf = np.zeros(int(offs[-1]), dtype=np.int32)
     tokens, positions, req_of = (buf[offs[i]:offs[i + 1]] for i in range(3))
     q_start, q_len, ctx_len, slot, rows = (buf[offs[i]:offs[i + 1]] for i in range(3, 8))
+    info = buf[offs[8 + 2 * n_groups]:offs[9 + 2 * n_groups]].reshape(R, 4)
     t = li = 0
     max_q = max_ctx = 1
     for r, e in enumerate(entries):
@@ -102,6 +104,7 @@ def pack_step(entries: Sequence[StepEntry], manager, vocab_size: int,
         positions[t:t + n] = np.arange(past, total)
         req_of[t:t + n] = r
         q_start[r], q_len[r], ctx_len[r], slot[r] = t, n, total, manager.slot(e.req_id)
+        info[r] = (t, n, past, total)
         for w in e.want:
             if not 0 <= w < n:
                 raise ValueError(f"request {e.req_id!r}: wanted place {w} is outside its {n} tokens")
@@ -139,7 +142,7 @@ def context_on(dev: torch.Tensor, p: PackedStep, max_ctx_len: Optional[int] = No
               for g in range(p.n_groups)]
     return StepContext(T=p.T, R=p.R, n_logits=p.n_logits, tokens=sl(0), positions=sl(1), req_of_token=sl(2),
                        q_start=sl(3), q_len=sl(4), ctx_len=sl(5), state_slot=sl(6), logit_rows=sl(7),
-                       groups=groups, max_q_len=p.max_q_len,
+                       req_info=sl(8 + 2 * p.n_groups).view(p.R, 4), groups=groups, max_q_len=p.max_q_len,
                        max_ctx_len=max_ctx_len if max_ctx_len is not None else p.max_ctx_len,
                        host={"q_len": p.q_len, "ctx_len": p.ctx_len, "logit_rows_identity": p.logit_rows_identity})
 

@@ -115,15 +115,15 @@ class AttentionMixer(Mixer):
                 nb = 1 if G <= 16 else (2 if G <= 32 else 4)
             else:
                 nb = 4 if self.hd <= 128 else 2
-            key = ("query_blocks", G, nb)
-            blocks = ctx.host.get(key)
-            if blocks is None:
-                blk_req, blk_col0 = ops.query_blocks(ctx.host["q_len"], G, nb)
-                blocks = (torch.from_numpy(blk_req).to(q.device), torch.from_numpy(blk_col0).to(q.device))
-                ctx.host[key] = blocks
-            ops.attention_mfma(q, cache.k, cache.v, o, block_table=g.block_table, blk_req=blocks[0],
-                               blk_col0=blocks[1], nb=nb, q_start=ctx.q_start, q_len=ctx.q_len,
-                               positions=ctx.positions, H=self.H, Hkv=self.Hkv, hd=self.hd,
+            blocks = None
+            if ctx.max_q_len > 1 or G > 16 * nb:
+                key = ("query_blocks", G, nb)
+                blocks = ctx.host.get(key)
+                if blocks is None:
+                    blocks = torch.from_numpy(ops.query_blocks(ctx.host["q_len"], G, nb)).to(q.device)
+                    ctx.host[key] = blocks
+            ops.attention_mfma(q, cache.k, cache.v, o, block_table=g.block_table, blocks=blocks, nb=nb,
+                               req_info=ctx.req_info, positions=ctx.positions, H=self.H, Hkv=self.Hkv, hd=self.hd,
                                page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len,
                                window=self.window or 0, scale=self.scale)
             return
