@@ -11,13 +11,13 @@
 // else was in the batch.
 //
 // Inside a wave (S^T = K Q^T, O^T = V^T P^T, all with v_mfma_f32_16x16x32_bf16):
-//  * 32 keys a step, as two blocks of 16.  A operand of S^T: K rows [key][hd], 16 bytes a lane.
-//    B operand: Q [column][hd], loaded once.
-//  * The result tile gives lane (column = l % 16, group g = l / 16) the scores of keys
-//    4g..4g+3 of each block.  After masking, running max and exp these eight values are,
-//    as they lie, the lane's part of the B operand P^T of the second product if the product's
-//    summed index is numbered k = 8g + i  <->  key (i < 4 ? 4g + i : 16 + 4g + i - 4).  The
-//    A operand V^T follows the same numbering: two 8-byte loads from the transposed V page.
+//  * 32 keys a step, in two products of 16.  A operand of S^T: K rows [key][hd], 16 bytes a lane;
+//    B operand: Q [column][hd], loaded once.  Row m of product kb is key 8 (m/4) + 4 kb + m % 4.
+//  * A result tile gives lane (column = l % 16, group g = l / 16) rows 4g..4g+3, so over both
+//    products the lane holds the scores of keys 8g..8g+7 in order.  After masking, running max
+//    and exp these eight values are, as they lie, the lane's part of the B operand P^T of the
+//    second product (k = 8g + i), and the A operand V^T is one 16-byte load of eight consecutive
+//    positions of a channel from the transposed V page.
 //  * No LDS, no transposes, no barriers; K rows and V columns of the next step are loaded
 //    while the current step computes.
 //
@@ -97,62 +97,76 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
         for (int db = 0; db < DB; ++db) o[db][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // One step covers 32 keys as two blocks of 16.  A step's K rows and V columns are loaded
-    // into registers a step ahead of their use (where the head size leaves room for it).
-    // Large tiles (head size x columns) leave no registers for that: they load as they go.
+    // One step covers 32 keys, two halves of 16 that each lie in one page.  The two S^T products
+    // of a step do not take the keys in order: row m of product kb is key 8 (m / 4) + 4 kb + m % 4
+    // of the step, so that lane group g ends up with the scores of keys 8g .. 8g+7, which is what
+    // the second product's operands hold for k = 8g + i.  A step's K rows and V columns are loaded
+    // into registers a step ahead of their use (where the head size leaves room for it); large
+    // tiles (head size x columns) load as they go.
     constexpr bool AHEAD = HDP * NB <= 256;
     struct Tile {
         bf16x8 kf[2][AHEAD ? KC : 1];
-        bf16x4 vx[2][AHEAD ? DB : 1];
-        long long base[2];                 // (page, kv head) start in both caches
-        int off0[2];
-        bool live[2];
+        bf16x8 vx[AHEAD ? DB : 1];
+        long long base[2];                 // per half: (page, kv head) start in both caches
+        int off0[2];                       // per half: offset of its first key in the page
+        bool live[2];                      // per half: holds keys some column may see
     };
-    auto k_frag = [&](long long base, int off0, int kc) {
+    const int k_half = n16 / 8;                                    // half of this lane's K rows
+    const int k_off = 8 * ((n16 / 4) % 2) + n16 % 4;               // + 4 kb: offset of the row's key in its half
+    auto k_frag = [&](const Tile& t, int kb, int kc) {
         const int k = kc * 32 + g * 8;
         bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-        return (k < hd) ? *(const bf16x8*)(k_cache + base + (long long)(off0 + n16) * hd + k) : z;
+        // selects, not indexing by a lane-dependent value (that would put the arrays in scratch memory)
+        const bool live = k_half ? t.live[1] : t.live[0];
+        const long long base = k_half ? t.base[1] : t.base[0];
+        const int off0 = k_half ? t.off0[1] : t.off0[0];
+        if (!live || k >= hd) return z;
+        return *(const bf16x8*)(k_cache + base + (long long)(off0 + k_off + 4 * kb) * hd + k);
     };
-    auto v_frag = [&](long long base, int off0, int db) {
+    auto v_frag = [&](const Tile& t, int db) {
         const int dim = db * 16 + n16;
-        bf16x4 z = {0, 0, 0, 0};
-        return (dim < hd) ? *(const bf16x4*)(v_cache + base + off0 + 4 * g + (long long)dim * page_size) : z;
+        bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+        const bool live = (g / 2) ? t.live[1] : t.live[0];
+        const long long base = (g / 2) ? t.base[1] : t.base[0];
+        const int off0 = (g / 2) ? t.off0[1] : t.off0[0];
+        if (!live || dim >= hd) return z;
+        return *(const bf16x8*)(v_cache + base + (long long)dim * page_size + off0 + (g % 2) * 8);
     };
     auto load_tile = [&](int key0, Tile& t) {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-            const int kbs = key0 + kb * 16;
-            t.live[kb] = kbs <= pos_max && kbs + 15 >= lo_min;
-            if (!t.live[kb]) continue;
-            const long long page = __shfl(my_page, kbs / page_size - first_page, WAVE);
-            t.off0[kb] = kbs % page_size;
-            t.base[kb] = (page * Hkv + kvh) * (long long)page_size * hd;
-            if constexpr (AHEAD) {
+        for (int h = 0; h < 2; ++h) {
+            const int hs = key0 + h * 16;
+            t.live[h] = hs <= pos_max && hs + 15 >= lo_min;
+            const long long page = t.live[h] ? __shfl(my_page, hs / page_size - first_page, WAVE) : 0;
+            t.off0[h] = hs % page_size;
+            t.base[h] = (page * Hkv + kvh) * (long long)page_size * hd;
+        }
+        if constexpr (AHEAD) {
 #pragma unroll
-                for (int kc = 0; kc < KC; ++kc) t.kf[kb][kc] = k_frag(t.base[kb], t.off0[kb], kc);
+            for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int db = 0; db < DB; ++db) t.vx[kb][db] = v_frag(t.base[kb], t.off0[kb], db);
-            }
+                for (int kc = 0; kc < KC; ++kc) t.kf[kb][kc] = k_frag(t, kb, kc);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) t.vx[db] = v_frag(t, db);
         }
     };
     auto compute = [&](int key0, const Tile& t) {
-        // ---- S^T = K Q^T for two blocks of 16 keys
+        // ---- S^T = K Q^T, twice 16 keys
         f32x4 s[2][NB];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) s[kb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (t.live[kb]) {
 #pragma unroll
-                for (int kc = 0; kc < KC; ++kc) {
-                    bf16x8 kf;
-                    if constexpr (AHEAD) kf = t.kf[kb][kc]; else kf = k_frag(t.base[kb], t.off0[kb], kc);
+            for (int kc = 0; kc < KC; ++kc) {
+                bf16x8 kf;
+                if constexpr (AHEAD) kf = t.kf[kb][kc]; else kf = k_frag(t, kb, kc);
 #pragma unroll
-                    for (int nb = 0; nb < NB; ++nb) s[kb][nb] = mfma32(kf, qf[nb][kc], s[kb][nb]);
-                }
+                for (int nb = 0; nb < NB; ++nb) s[kb][nb] = mfma32(kf, qf[nb][kc], s[kb][nb]);
             }
         }
         // ---- mask, running maximum, exp; P^T stays in registers as the next B operand
+        const bool my_live = (g / 2) ? t.live[1] : t.live[0];   // this lane's eight keys lie in half g / 2
         bf16x8 pf[NB];
         float corr[NB];
 #pragma unroll
@@ -163,8 +177,8 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const int key = key0 + kb * 16 + 4 * g + e;
-                    const bool ok = t.live[kb] && key <= pos_c[nb] && key >= lo_c[nb];
+                    const int key = key0 + 8 * g + 4 * kb + e;
+                    const bool ok = my_live && key <= pos_c[nb] && key >= lo_c[nb];
                     const float x = ok ? s[kb][nb][e] * scale : -INFINITY;
                     v[kb * 4 + e] = x;
                     mx = fmaxf(mx, x);
@@ -188,17 +202,12 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
         const bool tail = key0 + 31 > pos_max;             // keys beyond pos_max were never written
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-            bf16x8 vf = {0, 0, 0, 0, 0, 0, 0, 0};
+            bf16x8 vf;
+            if constexpr (AHEAD) vf = t.vx[db]; else vf = v_frag(t, db);
+            if (tail) {
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                if (!t.live[kb]) continue;
-                bf16x4 x;
-                if constexpr (AHEAD) x = t.vx[kb][db]; else x = v_frag(t.base[kb], t.off0[kb], db);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const bool written = !tail || (key0 + kb * 16 + 4 * g + e <= pos_max);
-                    vf[kb * 4 + e] = written ? x[e] : (bf16_t)0.f;
-                }
+                for (int i = 0; i < 8; ++i)
+                    if (key0 + 8 * g + i > pos_max) vf[i] = (bf16_t)0.f;
             }
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
