@@ -137,6 +137,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--point-steps", type=int, default=32)
+    ap.add_argument("--only-prefill", action="store_true",
+                    help="measure the 2,048-token prefill alone (for profiling) and print its record")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -157,6 +159,13 @@ def main() -> int:
     llm = LLM(engine=eng, max_num_seqs=max_b, max_batched_tokens=2048, ctx_size=args.context, ignore_eos=True)
     model = eng.model
 
+    if args.only_prefill:
+        dt = run_prefill(llm, cfg, PREFILL_TOKENS)
+        flops = prefill_flops(cfg, model, PREFILL_TOKENS)
+        print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / dt, 1), "tokens": PREFILL_TOKENS,
+                                      "ms": round(dt * 1e3, 3),
+                                      "frac": round(flops / dt / (PEAK_TFLOPS[args.dtype] * 1e12), 4)}}))
+        return 0
     secs, ctx_mean = run_decode(llm, cfg, args.batch, args.context, args.steps, args.warmup, SEED)
     tok_s = args.batch * args.steps / secs
     ms_step = 1e3 * secs / args.steps
