@@ -2,7 +2,7 @@
 // X and W bfloat16 with K contiguous, products accumulated in float32.
 //
 // Three kernels, chosen by M on the host:
-//  * tiled     M > 64: 128x128 block tiles staged through LDS (compute bound);
+//  * tiled     M > 64: 128x128 or 256x256 block tiles staged through LDS (compute bound);
 //  * skinny64  16 < M <= 64: a workgroup owns 64 rows of W, one MFMA column tile a wave; the
 //    activations of a K chunk are staged once in LDS for all four waves (bandwidth bound);
 //  * skinny16  M <= 16: a workgroup owns 16 rows of W; its four waves split K (bandwidth bound).
@@ -16,6 +16,7 @@
 // and eight consecutive k at 8 * (l / 16); it receives rows 4 * (l / 16) + 0..3, column (l % 16)
 // of the 16x16 result.
 #include "common.h"
+#include <type_traits>
 
 // OUT_SWIGLU: the rows of W are gate and up rows interleaved (2f: gate f, 2f+1: up f); the
 // output is bfloat16 [M, N/2] with y[m, f] = silu(g) * u, silu(g) = g / (1 + exp(-g)).
@@ -25,6 +26,14 @@ namespace {
 
 __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+template <int N, typename F, int I = 0>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>());
+        static_for<N, F, I + 1>(static_cast<F&&>(f));
+    }
 }
 
 template <int MODE>
@@ -55,7 +64,21 @@ __device__ __forceinline__ bf16x8 load8(const bf16_t* base, long long row, int n
 }
 
 // ------------------------------------------------------------------ tiled kernel
-constexpr int TBM = 128, TBN = 128, TBK = 64, TNT = 256;
+// A workgroup of WAVES_M x WAVES_N waves computes a block of Y; each wave a (16 TM) x (16 TN) part
+// of it as TM x TN MFMA tiles.  K is walked in steps of 64 through two LDS buffers: while a step
+// is multiplied out of one buffer, the next step's operands travel from memory to registers and,
+// piece by piece between the MFMAs, into the other buffer; one barrier a step.
+//
+// What the shapes answer to, measured on this part: one wave per SIMD issues MFMAs at little more
+// than half the rate two waves reach, the LDS takes about 170 bytes/ns per CU and gives 350 to
+// 430, against 8600 flop/ns per CU of the matrix cores.  So
+//   large:  256 x 256 blocks of eight waves (2 x 4, 128 x 64 each), 128 KB of LDS: two waves per
+//           SIMD, and per flop the least LDS traffic two buffers of 160 KB allow;
+//   small:  128 x 128 blocks of eight waves (2 x 4, 64 x 32 each), 64 KB of LDS, where the product
+//           has too few large blocks to give every CU one.
+// The MFMA takes W as its first operand, so a lane ends up with four neighbouring columns of one
+// row of Y and stores them as one piece.
+constexpr int TBK = 64;
 constexpr int CHUNKS = TBK / 8;                     // 16-byte chunks in one row of a tile
 
 // Chunk c of row r lives at chunk position c ^ (r % CHUNKS): the sixteen lanes that
@@ -63,79 +86,154 @@ constexpr int CHUNKS = TBK / 8;                     // 16-byte chunks in one row
 __device__ __forceinline__ int swz(int r, int c) { return r * TBK + ((c ^ (r % CHUNKS)) * 8); }
 
 template <int MODE>
-__global__ __launch_bounds__(TNT) void gemm_bf16_tiled_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
-                                                              void* __restrict__ Y, int M, int N, int K) {
-    __shared__ __attribute__((aligned(16))) bf16_t As[2][TBM * TBK];
-    __shared__ __attribute__((aligned(16))) bf16_t Bs[2][TBN * TBK];
+__device__ __forceinline__ void store_quad(void* Y, long long row, long long col, int M, int N, f32x4 v) {
+    if (row >= M) return;
+    if (MODE == OUT_SWIGLU) {
+        bf16_t* out = (bf16_t*)Y + row * (N / 2) + col / 2;
+        if (col + 3 < N && N % 4 == 0) {
+            bf16x2 o = {(bf16_t)silu_mul(v[0], v[1]), (bf16_t)silu_mul(v[2], v[3])};
+            *(bf16x2*)out = o;
+        } else {
+            if (col + 1 < N) out[0] = (bf16_t)silu_mul(v[0], v[1]);
+            if (col + 3 < N) out[1] = (bf16_t)silu_mul(v[2], v[3]);
+        }
+    } else if (col + 3 < N && N % 4 == 0) {
+        if (MODE == OUT_BF16) {
+            bf16x4 o = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+            *(bf16x4*)((bf16_t*)Y + row * N + col) = o;
+        } else {
+            f32x4* out = (f32x4*)((float*)Y + row * N + col);
+            if (MODE == OUT_F32_ACCUM) { const f32x4 old = *out; v[0] += old[0]; v[1] += old[1]; v[2] += old[2]; v[3] += old[3]; }
+            *out = v;
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (col + e < N) store_out<MODE>(Y, row * N + col + e, v[e]);
+    }
+}
+
+template <int TM, int TN, int WAVES_M, int WAVES_N, int AHEAD, int MODE>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_tiled_kernel(
+        const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, int M, int N, int K) {
+    constexpr int NT = 64 * WAVES_M * WAVES_N;
+    constexpr int BM = 16 * TM * WAVES_M, BN = 16 * TN * WAVES_N;
+    constexpr int PA = BM * CHUNKS / NT, PB = BN * CHUNKS / NT;     // 16-byte pieces of X and of W a thread moves a step
+    constexpr int ROWS_PER_PIECE = NT / CHUNKS;
+    static_assert(BM * CHUNKS % NT == 0 && BN * CHUNKS % NT == 0, "whole pieces");
+    static_assert(TN <= TM, "the fragments of W are fetched over TM inner steps");
+    extern __shared__ __attribute__((aligned(16))) bf16_t tiles[];       // [2][BM * TBK] of X then [2][BN * TBK] of W
+    bf16_t* As = tiles;
+    bf16_t* Bs = tiles + 2 * BM * TBK;
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
-    const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;
+    const int wm = (wave / WAVES_N) * 16 * TM, wn = (wave % WAVES_N) * 16 * TN;
     const int r16 = lane % 16, g = lane / 16;
-    const long long m0 = (long long)blockIdx.y * TBM, n0 = (long long)blockIdx.x * TBN;
+    const long long m0 = (long long)blockIdx.y * BM, n0 = (long long)blockIdx.x * BN;
 
-    f32x4 acc[4][4];
+    f32x4 acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    constexpr int PER_THREAD = (TBM * CHUNKS) / TNT;     // 4 chunks of A and 4 of B per thread
-    bf16x8 ra[PER_THREAD], rb[PER_THREAD];
-
-    auto load_global = [&](int k0) {
+    // Rows beyond the matrix read its last row instead (their results are never stored), so the
+    // loads of a full step need no guard.  Offsets are relative to the block's first row.
+    const bf16_t* Xb = X + m0 * K;
+    const bf16_t* Wb = W + n0 * K;
+    const int row0 = tid / CHUNKS, c0 = tid % CHUNKS;
+    const int last_a = (int)min((long long)BM - 1, (long long)M - 1 - m0);
+    const int last_b = (int)min((long long)BN - 1, (long long)N - 1 - n0);
+    unsigned offa[PA], offb[PB];
 #pragma unroll
-        for (int i = 0; i < PER_THREAD; ++i) {
-            const int id = tid + i * TNT;
-            const int row = id / CHUNKS, c = id % CHUNKS;
-            ra[i] = load8(X, m0 + row, M, k0 + c * 8, K);
-            rb[i] = load8(W, n0 + row, N, k0 + c * 8, K);
-        }
-    };
-    auto store_lds = [&](int buf) {
+    for (int i = 0; i < PA; ++i) offa[i] = (unsigned)min(row0 + i * ROWS_PER_PIECE, last_a) * (unsigned)K + c0 * 8;
 #pragma unroll
-        for (int i = 0; i < PER_THREAD; ++i) {
-            const int id = tid + i * TNT;
-            const int row = id / CHUNKS, c = id % CHUNKS;
-            *(bf16x8*)(&As[buf][swz(row, c)]) = ra[i];
-            *(bf16x8*)(&Bs[buf][swz(row, c)]) = rb[i];
-        }
-    };
-
+    for (int i = 0; i < PB; ++i) offb[i] = (unsigned)min(row0 + i * ROWS_PER_PIECE, last_b) * (unsigned)K + c0 * 8;
+    const int lds_st = swz(row0, c0);                    // piece i goes ROWS_PER_PIECE * TBK * i further
+    // Memory answers later than a step lasts, so the operands of AHEAD steps are on their way at
+    // any time, each in a register set of its own; a set is free again once it went into LDS.
+    bf16x8 ra[AHEAD][PA], rb[AHEAD][PB];
     const int nk = (K + TBK - 1) / TBK;
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) load_global((kt + 1) * TBK);
+
+    auto load_global = [&](auto set_tag, int kt) {
+        constexpr int set = decltype(set_tag)::value;
+        const int k0 = min(kt, nk - 1) * TBK;            // steps past the end read the last one again; nobody uses them
+        if (k0 + TBK <= K) {
 #pragma unroll
-        for (int ks = 0; ks < TBK / 32; ++ks) {
-            bf16x8 a[4], b[4];
+            for (int i = 0; i < PA; ++i) ra[set][i] = *(const bf16x8*)(Xb + k0 + offa[i]);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) a[i] = *(const bf16x8*)(&As[buf][swz(wm + i * 16 + r16, ks * 4 + g)]);
+            for (int i = 0; i < PB; ++i) rb[set][i] = *(const bf16x8*)(Wb + k0 + offb[i]);
+        } else {                                         // the last, partial step: zeros beyond K
+            const bool in = k0 + c0 * 8 < K;
+            const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) b[j] = *(const bf16x8*)(&Bs[buf][swz(wn + j * 16 + r16, ks * 4 + g)]);
+            for (int i = 0; i < PA; ++i) ra[set][i] = in ? *(const bf16x8*)(Xb + k0 + offa[i]) : z;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = mfma16(a[i], b[j], acc[i][j]);
+            for (int i = 0; i < PB; ++i) rb[set][i] = in ? *(const bf16x8*)(Wb + k0 + offb[i]) : z;
         }
-        if (kt + 1 < nk) store_lds(buf ^ 1);
-        __syncthreads();
+    };
+    auto store_piece = [&](auto set_tag, int buf, int p) {             // p counts the pieces of X, then those of W
+        constexpr int set = decltype(set_tag)::value;
+        if (p < PA) *(bf16x8*)(&As[buf * BM * TBK + lds_st + p * ROWS_PER_PIECE * TBK]) = ra[set][p < PA ? p : 0];
+        else *(bf16x8*)(&Bs[buf * BN * TBK + lds_st + (p - PA) * ROWS_PER_PIECE * TBK]) = rb[set][p < PA ? 0 : p - PA];
+    };
+    // fragment offsets inside a buffer: row r16 of MFMA tile 0 of this wave, k-chunk g (+4 for the second half)
+    const int fa0 = swz(wm + r16, g), fa1 = swz(wm + r16, 4 + g);
+    const int fb0 = swz(wn + r16, g), fb1 = swz(wn + r16, 4 + g);
+
+    // One step out of buffer `buf`: two halves (k 0..31, 32..63) of TM inner steps.  An inner step
+    // multiplies one fragment of X with the TN fragments of W; meanwhile the next fragment of X
+    // and, in the first half, the fragments of W for the second half are on their way from LDS,
+    // and in the second half the pieces of register set `fill` go into the other buffer.
+    auto multiply = [&](int buf, auto fill) {
+        const bf16_t* Ab = As + buf * BM * TBK;
+        const bf16_t* Bb = Bs + buf * BN * TBK;
+        bf16x8 b[TN], bn[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[j] = *(const bf16x8*)(Bb + fb0 + j * 16 * TBK);
+        bf16x8 a = *(const bf16x8*)(Ab + fa0);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const bf16x8 an = *(const bf16x8*)(Ab + (i + 1 < TM ? fa0 + (i + 1) * 16 * TBK : fa1));
+            if (i < TN) bn[i] = *(const bf16x8*)(Bb + fb1 + i * 16 * TBK);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = mfma16(b[j], a, acc[i][j]);
+            a = an;
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            bf16x8 an = a;
+            if (i + 1 < TM) an = *(const bf16x8*)(Ab + fa1 + (i + 1) * 16 * TBK);
+#pragma unroll
+            for (int p = 0; p < PA + PB; ++p)
+                if (p * TM / (PA + PB) == i) store_piece(fill, buf ^ 1, p);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = mfma16(bn[j], a, acc[i][j]);
+            a = an;
+        }
+    };
+
+    // set s holds step s, later step s + AHEAD, ...; step kt + 1 is filled in while step kt is multiplied
+    static_for<AHEAD>([&](auto s) { load_global(s, decltype(s)::value); });
+#pragma unroll
+    for (int p = 0; p < PA + PB; ++p) store_piece(std::integral_constant<int, 0>(), 0, p);
+    __syncthreads();
+    for (int kt0 = 0; kt0 < nk; kt0 += AHEAD) {
+        static_for<AHEAD>([&](auto u) {
+            constexpr int set = decltype(u)::value;
+            const int kt = kt0 + set;
+            if (kt < nk) {
+                load_global(u, kt + AHEAD);
+                multiply(kt & 1, std::integral_constant<int, (set + 1) % AHEAD>());
+                __syncthreads();
+            }
+        });
     }
 
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const long long col = n0 + wn + j * 16 + r16;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const long long row = m0 + wm + i * 16 + g * 4 + e;
-                const float v = acc[i][j][e];
-                const float partner = (MODE == OUT_SWIGLU) ? __shfl_xor(v, 1, WAVE) : 0.f;
-                store_elem<MODE>(Y, row, col, M, N, v, partner);
-            }
-        }
+        for (int j = 0; j < TN; ++j)
+            store_quad<MODE>(Y, m0 + wm + i * 16 + r16, n0 + wn + j * 16 + g * 4, M, N, acc[i][j]);
 }
 
 // ----------------------------------------------------------------- skinny kernels
@@ -500,8 +598,25 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
                                (const float*)ws, Y, M, N, mt * 16, p.slices);
         }
     } else {
-        dim3 grid(ceil_div(N, TBN), ceil_div(M, TBM)), block(TNT);
-        hipLaunchKernelGGL((gemm_bf16_tiled_kernel<MODE>), grid, block, 0, stream, X, W, Y, M, N, K);
+        // Large blocks where they give most CUs one.  Of the small ones a CU holds two if there are
+        // enough; if not, a block is alone on its CU and hides the memory's latency by itself, with
+        // the operands of four steps under way.
+        const long long large = (long long)ceil_div(N, 256) * ceil_div(M, 256);
+        const long long small = (long long)ceil_div(N, 128) * ceil_div(M, 128);
+#define TILED(TM, TN, WM, WN, AHEAD) do { \
+            auto kern = gemm_bf16_tiled_kernel<TM, TN, WM, WN, AHEAD, MODE>; \
+            constexpr int bm = 16 * TM * WM, bn = 16 * TN * WN, lds = 2 * (bm + bn) * TBK * 2; \
+            static bool set = false; \
+            if (!set) { \
+                if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -1; \
+                set = true; \
+            } \
+            hipLaunchKernelGGL(kern, dim3(ceil_div(N, bn), ceil_div(M, bm)), dim3(64 * WM * WN), lds, stream, X, W, Y, M, N, K); \
+        } while (0)
+        if (large >= 160) TILED(8, 4, 2, 4, 1);
+        else if (small > 256) TILED(4, 2, 2, 4, 1);
+        else TILED(4, 2, 2, 4, 4);
+#undef TILED
     }
     return launch_status();
 }
