@@ -327,6 +327,49 @@ def test_attention_general(gpu, H, Hkv, hd, ps, dt, window):
         assert (got - want).abs().max() <= tol * max(1.0, float(want.abs().max())), (t, int(req[t]), int(pos[t]))
 
 
+def _mixed_step_case(gpu, reqs, H, Hkv, hd, ps):
+    """A step over requests given as (tokens already in the cache, tokens of this step), pages
+    shuffled, stale pages full of NaN."""
+    dt = torch.bfloat16
+    n_blocks = [-(-(past + n) // ps) for past, n in reqs]
+    n_pages = sum(n_blocks) + 2
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(7)).tolist()
+    kc = torch.full((n_pages, Hkv, ps, hd), float("nan"), dtype=dt)
+    vc = torch.full((n_pages, Hkv, hd, ps), float("nan"), dtype=dt)
+    table = torch.full((len(reqs), max(n_blocks)), -1, dtype=torch.int32)
+    Ks, Vs, q_start, q_len, pos = [], [], [], [], []
+    for r, ((past, n), nb_) in enumerate(zip(reqs, n_blocks)):
+        pages = torch.tensor([perm.pop() for _ in range(nb_)])
+        table[r, :nb_] = pages.to(torch.int32)
+        K = _r(past + n, Hkv, hd, seed=50 + r, dtype=dt)
+        V = _r(past + n, Hkv, hd, seed=70 + r, dtype=dt)
+        t = torch.arange(past + n)
+        kc[pages[t // ps], :, t % ps, :] = K
+        vc[pages[t // ps], :, :, t % ps] = V
+        Ks.append(K.double())
+        Vs.append(V.double())
+        q_start.append(len(pos))
+        q_len.append(n)
+        pos += list(range(past, past + n))
+    q = _r(len(pos), H * hd, seed=90, dtype=dt)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
+    req_info = i32([[qs, ql, past, past + ql] for qs, ql, (past, _) in zip(q_start, q_len, reqs)])
+    return dict(kc=kc.to(gpu), vc=vc.to(gpu), table=table.to(gpu), q=q, Ks=Ks, Vs=Vs, q_len=q_len,
+                positions=i32(pos), req_info=req_info, max_ctx_len=max(p + n for p, n in reqs))
+
+
+def _check_step(case, reqs, got, H, hd, window, tag):
+    scale = 1 / math.sqrt(hd)
+    assert torch.isfinite(got).all(), tag
+    t = 0
+    for r, (past, n) in enumerate(reqs):
+        for j in range(n):
+            want = _attention_reference(case["q"][t].double().reshape(H, hd), case["Ks"][r], case["Vs"][r], past + j,
+                                        window, scale)
+            assert (got[t] - want).abs().max() <= 2 ** -6 * max(1.0, float(want.abs().max())), (tag, r, j)
+            t += 1
+
+
 @pytest.mark.parametrize("H,Hkv,hd,ps", [(4, 2, 16, 16), (4, 1, 24, 16), (3, 3, 80, 16), (2, 1, 256, 32),
                                           (32, 8, 64, 16), (8, 2, 128, 64), (32, 1, 64, 16), (5, 5, 40, 48)])
 @pytest.mark.parametrize("window", [0, 37, 300])
@@ -334,53 +377,119 @@ def test_attention_mfma(gpu, H, Hkv, hd, ps, window):
     """A mixed step: a decoded token deep in a long request, a prompt portion in the middle of
     another, a whole short prompt, a first token.  Stale pages hold NaN."""
     from tuff_amd.csrc import ops
-    dt = torch.bfloat16
-    # (tokens already in the cache, tokens of this step)
     reqs = [(699, 1), (230, 50), (0, 33), (0, 1), (255, 3), (511, 2)]
-    n_blocks = [-(-(past + n) // ps) for past, n in reqs]
-    n_pages = sum(n_blocks) + 2
-    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(7)).tolist()
-    kc = torch.full((n_pages, Hkv, ps, hd), float("nan"), dtype=dt)
-    vc = torch.full((n_pages, Hkv, hd, ps), float("nan"), dtype=dt)
-    maxb = max(n_blocks)
-    table = torch.full((len(reqs), maxb), -1, dtype=torch.int32)
-    Ks, Vs, q_start, q_len, pos = [], [], [], [], []
-    for r, ((past, n), nb_) in enumerate(zip(reqs, n_blocks)):
-        pages = [perm.pop() for _ in range(nb_)]
-        table[r, :nb_] = torch.tensor(pages, dtype=torch.int32)
-        K = _r(past + n, Hkv, hd, seed=50 + r, dtype=dt)
-        V = _r(past + n, Hkv, hd, seed=70 + r, dtype=dt)
-        for t in range(past + n):
-            kc[pages[t // ps], :, t % ps, :] = K[t]
-            vc[pages[t // ps], :, :, t % ps] = V[t]
-        Ks.append(K.double())
-        Vs.append(V.double())
-        q_start.append(len(pos))
-        q_len.append(n)
-        pos += list(range(past, past + n))
-    T = len(pos)
-    q = _r(T, H * hd, seed=90, dtype=dt)
-    scale = 1 / math.sqrt(hd)
-    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
-    req_info = i32([[qs, ql, past, past + ql] for qs, ql, (past, _) in zip(q_start, q_len, reqs)])
+    case = _mixed_step_case(gpu, reqs, H, Hkv, hd, ps)
+    T = case["q"].shape[0]
     for nb in ([1, 2, 4] if hd <= 128 else [1, 2]):
-        blocks = torch.from_numpy(ops.query_blocks(q_len, H // Hkv, nb)).to(gpu)
-        out = torch.full((T, H * hd), float("nan"), dtype=dt, device=gpu)
-        ops.attention_mfma(q.to(gpu), kc.to(gpu), vc.to(gpu), out, block_table=table.to(gpu),
-                           blocks=blocks, nb=nb, req_info=req_info, positions=i32(pos), H=H, Hkv=Hkv, hd=hd,
-                           page_size=ps, max_ctx_len=700, window=window)
+        blocks = torch.from_numpy(ops.query_blocks(case["q_len"], H // Hkv, nb)).to(gpu)
+        out = torch.full((T, H * hd), float("nan"), dtype=torch.bfloat16, device=gpu)
+        ops.attention_mfma(case["q"].to(gpu), case["kc"], case["vc"], out, block_table=case["table"],
+                           blocks=blocks, nb=nb, req_info=case["req_info"], positions=case["positions"], H=H, Hkv=Hkv,
+                           hd=hd, page_size=ps, max_ctx_len=700, window=window)
         got = out.cpu().double().reshape(T, H, hd)
-        assert torch.isfinite(got).all(), nb
         if nb == 1:
             first = got
         else:
             assert torch.equal(got, first), "the result depends on the column blocking"
-        t = 0
-        for r, (past, n) in enumerate(reqs):
-            for j in range(n):
-                want = _attention_reference(q[t].double().reshape(H, hd), Ks[r], Vs[r], past + j, window, scale)
-                assert (got[t] - want).abs().max() <= 2 ** -6 * max(1.0, float(want.abs().max())), (nb, r, j)
-                t += 1
+        _check_step(case, reqs, got, H, hd, window, nb)
+
+
+@pytest.mark.parametrize("H,Hkv,hd,ps", [(4, 2, 16, 16), (4, 1, 24, 16), (3, 3, 80, 16), (2, 1, 256, 32),
+                                          (32, 8, 64, 16), (8, 2, 128, 64), (32, 1, 64, 16), (5, 5, 40, 48),
+                                          (6, 2, 96, 80)])
+@pytest.mark.parametrize("window", [0, 37, 300])
+def test_attention_prefill(gpu, H, Hkv, hd, ps, window):
+    """Prompt portions of several blocks of columns, starting anywhere, beside single tokens; a
+    token's result must not depend on where its portion started."""
+    from tuff_amd.csrc import ops
+    cols = ops.attention_prefill_block_columns(hd)
+
+    def run(reqs):
+        case = _mixed_step_case(gpu, reqs, H, Hkv, hd, ps)
+        T = case["q"].shape[0]
+        blocks = torch.from_numpy(ops.query_blocks(case["q_len"], H // Hkv, cols // 16)).to(gpu)
+        out = torch.full((T, H * hd), float("nan"), dtype=torch.bfloat16, device=gpu)
+        ops.attention_prefill(case["q"].to(gpu), case["kc"], case["vc"], out, block_table=case["table"],
+                              blocks=blocks, req_info=case["req_info"], H=H, Hkv=Hkv, hd=hd, page_size=ps,
+                              max_ctx_len=case["max_ctx_len"], window=window)
+        got = out.cpu().double().reshape(T, H, hd)
+        _check_step(case, reqs, got, H, hd, window, "prefill")
+        return case, got
+
+    reqs = [(699, 1), (230, 150), (0, 333), (0, 1), (255, 3), (1100, 70)]
+    case, got = run(reqs)
+    # tokens 70..149 of request 1 (positions 300..379) again, as a step of their own that starts
+    # at position 300: bit for bit the same
+    first = sum(n for _, n in reqs[:1]) + 70
+    sel = torch.arange(first, first + 80)
+    q3 = case["q"][sel]
+    # give the single request the keys and values of request 1 of the first step
+    K, V = case["Ks"][1].to(torch.bfloat16), case["Vs"][1].to(torch.bfloat16)
+    n_blk = -(-380 // ps)
+    kc = torch.full((n_blk + 1, Hkv, ps, hd), float("nan"), dtype=torch.bfloat16)
+    vc = torch.full((n_blk + 1, Hkv, hd, ps), float("nan"), dtype=torch.bfloat16)
+    t = torch.arange(380)
+    kc[t // ps, :, t % ps, :] = K
+    vc[t // ps, :, :, t % ps] = V
+    table = torch.arange(n_blk, dtype=torch.int32)[None].to(gpu)
+    out = torch.full((80, H * hd), float("nan"), dtype=torch.bfloat16, device=gpu)
+    blocks = torch.from_numpy(ops.query_blocks([80], H // Hkv, cols // 16)).to(gpu)
+    ops.attention_prefill(q3.to(gpu), kc.to(gpu), vc.to(gpu), out, block_table=table, blocks=blocks,
+                          req_info=torch.tensor([[0, 80, 300, 380]], dtype=torch.int32, device=gpu), H=H, Hkv=Hkv, hd=hd,
+                          page_size=ps, max_ctx_len=380, window=window)
+    assert torch.equal(out.cpu().double().reshape(80, H, hd), got[sel]), "the result depends on where the portion starts"
+
+
+@pytest.mark.parametrize("kernel", ["mfma", "prefill"])
+def test_attention_matrix_kernels_find_a_far_key_and_the_window_edge(gpu, kernel):
+    """One key among a thousand matches the query: the output is that key's value row, wherever
+    the key sits (first position, edges of pages, of steps and of partitions, the last position).
+    With a window W the key at pos - W + 1 is seen and the one at pos - W is not."""
+    from tuff_amd.csrc import ops
+    hd, ps, n = 32, 16, 1000
+    dt = torch.bfloat16
+    n_pages = n // ps + 1
+    table = torch.arange(n_pages, dtype=torch.int32)[None].to(gpu)
+
+    def run(q, kc, vc, n_q, window):
+        out = torch.empty(n_q, hd, dtype=dt, device=gpu)
+        pos0 = n - n_q
+        info = torch.tensor([[0, n_q, pos0, n]], dtype=torch.int32, device=gpu)
+        common = dict(block_table=table, req_info=info, H=1, Hkv=1, hd=hd, page_size=ps, max_ctx_len=n, window=window)
+        if kernel == "mfma":
+            blocks = torch.from_numpy(ops.query_blocks([n_q], 1, 1)).to(gpu)
+            ops.attention_mfma(q.to(gpu), kc.to(gpu), vc.to(gpu), out, blocks=blocks, nb=1,
+                               positions=torch.arange(pos0, n, dtype=torch.int32, device=gpu), **common)
+        else:
+            blocks = torch.from_numpy(ops.query_blocks([n_q], 1, ops.attention_prefill_block_columns(hd) // 16)).to(gpu)
+            ops.attention_prefill(q.to(gpu), kc.to(gpu), vc.to(gpu), out, blocks=blocks, **common)
+        return out.cpu()
+
+    for hot in (0, 15, 16, 31, 32, 63, 64, 255, 256, 447, 448, 959, 960, 998, 999):
+        kc = _r(n_pages, 1, ps, hd, seed=3, scale=0.05, dtype=dt)
+        vc = _r(n_pages, 1, hd, ps, seed=4, dtype=dt)
+        q = torch.zeros(3, hd, dtype=dt)
+        q[:, 5] = 30.0
+        kc[hot // ps, 0, hot % ps, 5] = 30.0                     # score 900/sqrt(32) = 159 above the rest
+        out = run(q, kc, vc, 3, 0)
+        for j in range(3):                                        # queries at positions n-3, n-2, n-1
+            if hot <= n - 3 + j:
+                assert torch.equal(out[j], vc[hot // ps, 0, :, hot % ps]), (hot, j)
+    W = 300
+    for n_q in (1, 5):
+        pos = n - n_q                                             # the first query of the step
+        for edge, seen in ((pos - W + 1, True), (pos - W, False)):
+            kc = torch.zeros(n_pages, 1, ps, hd, dtype=dt)
+            vc = torch.zeros(n_pages, 1, hd, ps, dtype=dt)
+            q = torch.zeros(n_q, hd, dtype=dt)
+            q[:, 0] = 20.0
+            kc[edge // ps, 0, edge % ps, 0] = 20.0
+            vc[edge // ps, 0, :, edge % ps] = 1.0
+            out = run(q, kc, vc, n_q, W)
+            if seen:
+                assert float(out[0].min()) > 0.99, (n_q, edge)
+            else:
+                assert float(out[0].abs().max()) == 0.0, (n_q, edge)
 
 
 def test_attention_finds_a_far_key(gpu):

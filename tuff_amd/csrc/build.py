@@ -30,6 +30,7 @@ MODULES = {
     "rope_kv": "rope_kv.hip",
     "attention": "attention.hip",
     "attention_mfma": "attention_mfma.hip",
+    "attention_prefill": "attention_prefill.hip",
     "shortconv": "shortconv.hip",
     "sampling": "sampling.hip",
 }

@@ -63,6 +63,11 @@ _SIGNATURES = {
                                 _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p],
     },
+    "attention_prefill": {
+        "tuff_attention_prefill": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
+                                   _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p],
+        "tuff_attention_prefill_block_columns": [_c_int],
+    },
     "shortconv": {
         "tuff_shortconv_fwd": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
@@ -430,6 +435,51 @@ def attention_mfma(q, k_cache, v_cache, out, *, block_table, blocks, nb, req_inf
         block_table.data_ptr(), block_table.shape[1], None if blocks is None else blocks.data_ptr(), nblk, nb,
         req_info.data_ptr(), positions.data_ptr(), T, H, Hkv, hd, page_size,
         int(window or 0), float(scale), n_parts, _stream()), "attention_mfma")
+
+
+def attention_prefill_block_columns(hd: int) -> int:
+    """Columns (token, head in the kv group) a query block of attention_prefill holds."""
+    return 128 if hd <= 128 else 64
+
+
+def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info,
+                      H, Hkv, hd, page_size, max_ctx_len, window=0, scale=None) -> None:
+    """Matrix-core attention for steps with prompt portions: a workgroup walks over all keys of a
+    block of query columns, keys and values staged through LDS; writes `out` directly.
+    blocks: int32 [n_blocks, 2] from query_blocks(q_len, G, attention_prefill_block_columns(hd) // 16),
+    or None when every request's columns fit one block (block b = request b)."""
+    T = q.shape[0]
+    if not attention_mfma_supported(q.dtype, hd, page_size):
+        raise KernelError(f"attention_prefill: needs bfloat16, a head size that is a multiple of 8 (got {hd}) "
+                          f"and a page size that is a multiple of 16 (got {page_size})")
+    _gpu("q", q, torch.bfloat16, (T, H * hd))
+    _gpu("out", out, torch.bfloat16, (T, H * hd))
+    P = k_cache.shape[0]
+    _gpu("k_cache", k_cache, torch.bfloat16, (P, Hkv, page_size, hd))
+    _gpu("v_cache", v_cache, torch.bfloat16, (P, Hkv, hd, page_size))
+    _gpu("block_table", block_table, torch.int32)
+    R = req_info.shape[0]
+    _gpu("req_info", req_info, torch.int32, (R, 4))
+    if block_table.dim() != 2 or block_table.shape[0] != R:
+        raise KernelError("attention_prefill: block_table must be [requests, blocks]")
+    if block_table.shape[1] * page_size < int(max_ctx_len):
+        raise KernelError("attention_prefill: block_table is narrower than the longest context")
+    if H % Hkv:
+        raise KernelError("attention_prefill: the query heads must be a multiple of the kv heads")
+    G = H // Hkv
+    if blocks is None:
+        if G > attention_prefill_block_columns(hd):
+            raise KernelError("attention_prefill: without a block list a request's columns must fit one block")
+        nblk = R
+    else:
+        nblk = blocks.shape[0]
+        _gpu("blocks", blocks, torch.int32, (nblk, 2))
+    if scale is None:
+        scale = 1.0 / math.sqrt(hd)
+    _check(load("attention_prefill").tuff_attention_prefill(
+        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
+        block_table.data_ptr(), block_table.shape[1], None if blocks is None else blocks.data_ptr(), nblk,
+        req_info.data_ptr(), H, Hkv, hd, page_size, int(window or 0), float(scale), _stream()), "attention_prefill")
 
 
 def query_blocks(q_len, G: int, nb: int):

@@ -60,7 +60,7 @@ class AttentionMixer(Mixer):
         return decls
 
     def kernel_modules(self):
-        mods = ["rope_kv", "attention", "attention_mfma"]
+        mods = ["rope_kv", "attention", "attention_mfma", "attention_prefill"]
         if self.position is not None:
             mods += self.position.kernel_modules()
         return mods
@@ -108,24 +108,30 @@ class AttentionMixer(Mixer):
         self.attend(q, o, ctx, cache, g)
         self.out.forward(o, accumulate_into=residual)
 
+    @staticmethod
+    def _blocks(ctx, G, nb, device):
+        key = ("query_blocks", G, nb)
+        blocks = ctx.host.get(key)
+        if blocks is None:
+            blocks = torch.from_numpy(ops.query_blocks(ctx.host["q_len"], G, nb)).to(device)
+            ctx.host[key] = blocks
+        return blocks
+
     def attend(self, q, o, ctx, cache, g) -> None:
         G = self.H // self.Hkv
         if ops.attention_mfma_supported(q.dtype, self.hd, cache.page_size):
-            if ctx.max_q_len == 1:
-                nb = 1 if G <= 16 else (2 if G <= 32 else 4)
-            else:
-                nb = 4 if self.hd <= 128 else 2
-            blocks = None
-            if ctx.max_q_len > 1 or G > 16 * nb:
-                key = ("query_blocks", G, nb)
-                blocks = ctx.host.get(key)
-                if blocks is None:
-                    blocks = torch.from_numpy(ops.query_blocks(ctx.host["q_len"], G, nb)).to(q.device)
-                    ctx.host[key] = blocks
-            ops.attention_mfma(q, cache.k, cache.v, o, block_table=g.block_table, blocks=blocks, nb=nb,
-                               req_info=ctx.req_info, positions=ctx.positions, H=self.H, Hkv=self.Hkv, hd=self.hd,
-                               page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len,
-                               window=self.window or 0, scale=self.scale)
+            common = dict(block_table=g.block_table, req_info=ctx.req_info, H=self.H, Hkv=self.Hkv, hd=self.hd,
+                          page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len, window=self.window or 0,
+                          scale=self.scale)
+            if ctx.max_q_len > 1:
+                # prompt portions in the step: blocks of columns walk over their keys through LDS
+                nb = ops.attention_prefill_block_columns(self.hd) // 16
+                ops.attention_prefill(q, cache.k, cache.v, o, blocks=self._blocks(ctx, G, nb, q.device), **common)
+                return
+            # single tokens: the keys of a request are split over many waves, then merged
+            nb = 1 if G <= 16 else (2 if G <= 32 else 4)
+            blocks = self._blocks(ctx, G, nb, q.device) if G > 16 * nb else None
+            ops.attention_mfma(q, cache.k, cache.v, o, blocks=blocks, nb=nb, positions=ctx.positions, **common)
             return
         ops.attention_general(q, cache.k, cache.v, o, block_table=g.block_table,
                               req_of_token=ctx.req_of_token, positions=ctx.positions,
