@@ -5,7 +5,7 @@
 // request (a column = one query head of one token; NBW * 16 columns a wave) and walks over all
 // keys these columns may see, 64 at a time, from key 0 (or the first 64 the window still
 // reaches).  The K rows and V columns of a step are copied from the pages into LDS once, by all
-// threads, one step ahead of their use; every wave reads its MFMA operands from there.  Each
+// threads, a few steps ahead of their use; every wave reads its MFMA operands from there.  Each
 // column carries a running maximum, sum and output (online softmax) and is written normalised at
 // the end: no work space and no second kernel.
 //
@@ -26,6 +26,7 @@
 namespace {
 constexpr int STEP = 64;            // keys a step
 constexpr int NT = 256;             // threads a workgroup
+constexpr float SLACK = 8.f;        // see half_step
 constexpr int VROW = STEP + 8;      // bf16 a row of V^T in LDS: 64 keys and 16 bytes that keep rows off each other's banks
 
 __device__ __forceinline__ f32x4 mfma32(bf16x8 a, bf16x8 b, f32x4 c) {
@@ -39,7 +40,7 @@ __device__ __forceinline__ int k_row_of_key(int key) {
     return sub * 32 + kb * 16 + h * 8 + q * 4 + m;
 }
 
-template <int HDP, int NBW>
+template <int HDP, int NBW, int AHEAD>
 __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ block_table, int max_blocks,
@@ -119,54 +120,97 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         const long long idx = ((long long)(gran0 + batch * 64 + lane) * 16) / page_size;
         return idx < max_blocks ? table[idx] : -1;
     };
-    int pages_cur = pages_of(0), pages_next = -1;
+    int pages_cur = pages_of(0), pages_next = pages_of(1);
 
-    // ---- copies: what this thread moves each step
-    bf16x8 kreg[KPT], vreg[VPT];
-    auto load_step = [&](int s) {                       // step s of the block -> registers
+    // ---- copies: what this thread moves each step.  Memory answers later than a step lasts, so
+    // the keys and values of AHEAD steps are on their way at any time, each in a register set.
+    // Per piece the thread keeps what does not change from step to step: the granule (16 keys, one
+    // page) it lies in, its offset inside the granule's rows, and where it goes in LDS.
+    bf16x8 kreg[AHEAD][KPT], vreg[AHEAD][VPT];
+    int k_gran[KPT], k_key[KPT], k_off[KPT], k_lds[KPT], v_gran[VPT], v_key[VPT], v_off[VPT], v_lds[VPT];
+    bool k_ok[KPT], v_ok[VPT];
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+        const int id = tid + i * NT, key = id / HC, c = id % HC;
+        k_gran[i] = key / 16;
+        k_key[i] = key;
+        k_off[i] = (key % 16) * hd + c * 8;
+        k_ok[i] = c * 8 < hd;
+        k_lds[i] = k_row_of_key(key) * KROW + c * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int id = tid + i * NT, dim = id / 8, c8 = id % 8;
+        v_gran[i] = c8 / 2;
+        v_key[i] = c8 * 8;
+        v_off[i] = dim * page_size + (c8 % 2) * 8;
+        v_ok[i] = dim < hd;
+        v_lds[i] = dim * VROW + c8 * 8;
+    }
+    const bool whole_rows = hd == HDP;
+    int ld_off = key_start % page_size;                 // offset in its page of the first key of the next step to load
+    auto pick = [](int gsel, long long b0, long long b1, long long b2, long long b3) {
+        return gsel == 0 ? b0 : gsel == 1 ? b1 : gsel == 2 ? b2 : b3;
+    };
+    auto load_step = [&](int set, int s, int pages) {   // step s of the block -> register set; zeros beyond pos_max
         const int key0 = key_start + s * STEP;
-        const int gslot0 = (s % 16) * 4;                // granule of the step's first key within pages_cur
+        const int gslot0 = (s % 16) * 4;                // granule of the step's first key within `pages`
+        // per granule, the same for all threads: where its rows start in both caches
+        long long bk[4], bv[4];
+        bool all_live = key0 + STEP - 1 <= pos_max;
+        int go = ld_off;
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            const int page = __builtin_amdgcn_readlane(pages, gslot0 + g4);
+            all_live = all_live && page >= 0;
+            const long long head = (long long)max(page, 0) * Hkv + kvh;
+            bk[g4] = page >= 0 ? (head * page_size + go) * hd : -1;
+            bv[g4] = head * hd * page_size + go;
+            go += 16;
+            if (go >= page_size) go -= page_size;
+        }
+        ld_off = go;
+        if (all_live && whole_rows) {
+#pragma unroll
+            for (int i = 0; i < KPT; ++i)
+                kreg[set][i] = *(const bf16x8*)(k_cache + pick(k_gran[i], bk[0], bk[1], bk[2], bk[3]) + k_off[i]);
+#pragma unroll
+            for (int i = 0; i < VPT; ++i)
+                vreg[set][i] = *(const bf16x8*)(v_cache + pick(v_gran[i], bv[0], bv[1], bv[2], bv[3]) + v_off[i]);
+            return;
+        }
+        // first steps under a window, the last step, narrow heads: pieces that do not exist read as zero
         const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int i = 0; i < KPT; ++i) {
-            const int id = tid + i * NT;
-            const int key = id / HC, c = id % HC;
-            const int page = __shfl(pages_cur, gslot0 + key / 16, WAVE);
-            const int kabs = key0 + key;
-            const bool live = page >= 0 && kabs <= pos_max && c * 8 < hd;
-            kreg[i] = live ? *(const bf16x8*)(k_cache + (((long long)page * Hkv + kvh) * page_size + kabs % page_size) * hd + c * 8) : z;
+            const long long base = pick(k_gran[i], bk[0], bk[1], bk[2], bk[3]);
+            const bool live = base >= 0 && key0 + k_key[i] <= pos_max && k_ok[i];
+            const bf16x8 v = *(const bf16x8*)(k_cache + (live ? base + k_off[i] : 0));
+            kreg[set][i] = live ? v : z;
         }
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
-            const int id = tid + i * NT;
-            const int dim = id / 8, c8 = id % 8;
-            const int page = __shfl(pages_cur, gslot0 + c8 / 2, WAVE);
-            const int kabs = key0 + c8 * 8;
-            const bool live = page >= 0 && kabs <= pos_max && dim < hd;
-            bf16x8 v = live ? *(const bf16x8*)(v_cache + (((long long)page * Hkv + kvh) * hd + dim) * page_size + kabs % page_size) : z;
-            if (kabs + 7 > pos_max) {                   // positions beyond the last were never written
+            const long long base = pick(v_gran[i], bv[0], bv[1], bv[2], bv[3]);
+            const int kabs = key0 + v_key[i];
+            const bool live = pick(v_gran[i], bk[0], bk[1], bk[2], bk[3]) >= 0 && kabs <= pos_max && v_ok[i];
+            bf16x8 v = *(const bf16x8*)(v_cache + (live ? base + v_off[i] : 0));
+            v = live ? v : z;
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (kabs + e > pos_max) v[e] = (bf16_t)0.f;
-            }
-            vreg[i] = v;
+            for (int e = 0; e < 8; ++e)                  // positions beyond the last were never written
+                if (kabs + e > pos_max) v[e] = (bf16_t)0.f;
+            vreg[set][i] = v;
         }
     };
-    auto store_step = [&](int buf) {
+    auto store_step = [&](int set, int buf) {
 #pragma unroll
-        for (int i = 0; i < KPT; ++i) {
-            const int id = tid + i * NT;
-            *(bf16x8*)(Ks + buf * KBUF + k_row_of_key(id / HC) * KROW + (id % HC) * 8) = kreg[i];
-        }
+        for (int i = 0; i < KPT; ++i) *(bf16x8*)(Ks + buf * KBUF + k_lds[i]) = kreg[set][i];
 #pragma unroll
-        for (int i = 0; i < VPT; ++i) {
-            const int id = tid + i * NT;
-            *(bf16x8*)(Vs + buf * VBUF + (id / 8) * VROW + (id % 8) * 8) = vreg[i];
-        }
+        for (int i = 0; i < VPT; ++i) *(bf16x8*)(Vs + buf * VBUF + v_lds[i]) = vreg[set][i];
     };
 
     // ---- one half step (32 keys) of this wave out of LDS
-    auto half_step = [&](int buf, int sub, int key0) {
+    auto half_step = [&](int buf, int sub, int key0, auto open_tag) {
+        constexpr bool open = decltype(open_tag)::value;
         const bf16_t* Kb = Ks + buf * KBUF + (sub * 32 + n16) * KROW + g * 8;
         const bf16_t* Vb = Vs + buf * VBUF + n16 * VROW + sub * 32 + g * 8;
         f32x4 s[2][NBW];
@@ -181,76 +225,90 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
                 for (int nb = 0; nb < NBW; ++nb) s[kb][nb] = mfma32(kf, qf[nb][kc], s[kb][nb]);
             }
         }
-        // every key of the half is visible to every column of the wave: no mask
-        const bool open = key0 + 31 <= wave_pos_min && key0 >= wave_lo_max;
+        // open: every key of the half is visible to every column of the wave, no mask
         bf16x8 pf[NBW];
         float corr[NBW];
         bool same = true;
 #pragma unroll
         for (int nb = 0; nb < NBW; ++nb) {
-            float v[8];
+            // The maximum is taken over the raw scores and scaled afterwards (scale > 0, rounding is
+            // monotonic), so that score * scale - maximum is one fused operation: written as fmaf,
+            // it is the same instruction with and without the mask.
             float mx = -INFINITY;
+            bool ok[8];
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int key = key0 + 8 * g + 4 * kb + e;
-                    const bool ok = open || (key <= pos_c[nb] && key >= lo_c[nb]);
-                    const float x = ok ? s[kb][nb][e] * scale_log2e : -INFINITY;
-                    v[kb * 4 + e] = x;
-                    mx = fmaxf(mx, x);
+                    ok[kb * 4 + e] = open || (key <= pos_c[nb] && key >= lo_c[nb]);
+                    mx = fmaxf(mx, ok[kb * 4 + e] ? s[kb][nb][e] : -INFINITY);
                 }
             mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
             mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-            const float m_new = fmaxf(m_run[nb], mx);
+            // The reference point of the exponents moves only when a score exceeds it by more than
+            // 2^SLACK: until then the weights may reach 2^SLACK instead of 1, which float32 sums and
+            // bfloat16 weights hold as well, and the output so far need not be rescaled.
+            const float m_cand = mx * scale_log2e;
+            const float m_new = (m_cand > m_run[nb] + SLACK) ? m_cand : m_run[nb];
             const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
             corr[nb] = __builtin_amdgcn_exp2f(m_run[nb] - m_safe);           // 0 while nothing was seen yet
             same = same && (m_new == m_run[nb]);
             float sum = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float p = __builtin_amdgcn_exp2f(v[i] - m_safe);
+                const float p = ok[i] ? __builtin_amdgcn_exp2f(fmaf(s[i / 4][nb][i % 4], scale_log2e, -m_safe)) : 0.f;
                 sum += p;
                 pf[nb][i] = (bf16_t)p;
             }
-            l_run[nb] = l_run[nb] * corr[nb] + sum;
+            l_run[nb] = fmaf(l_run[nb], corr[nb], sum);
             m_run[nb] = m_new;
         }
-        const bool rescale = !__all(same);                   // corr is exactly 1 where the maximum stayed
+        if (!__all(same)) {                                  // rare; corr is exactly 1 where the reference stayed
+            asm volatile("" ::: "memory");                   // a branch, not a select over every accumulator
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int nb = 0; nb < NBW; ++nb)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[db][nb][e] *= corr[nb];
+        }
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
             const bf16x8 vf = *(const bf16x8*)(Vb + db * 16 * VROW);
 #pragma unroll
-            for (int nb = 0; nb < NBW; ++nb) {
-                f32x4 acc = o[db][nb];
-                if (rescale) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[e] *= corr[nb];
-                }
-                o[db][nb] = mfma32(vf, pf[nb], acc);
-            }
+            for (int nb = 0; nb < NBW; ++nb) o[db][nb] = mfma32(vf, pf[nb], o[db][nb]);
         }
     };
 
-    load_step(0);
-    store_step(0);
-    __syncthreads();
-    for (int s = 0; s < nsteps; ++s) {
-        const int buf = s & 1;
-        const int key0 = key_start + s * STEP;
-        const bool more = s + 1 < nsteps;
-        if (s % 16 == 0) pages_next = pages_of(s / 16 + 1);
-        if (more) {
-            if ((s + 1) % 16 == 0) pages_cur = pages_next;
-            load_step(s + 1);
-        }
+    // set u holds step u, later step u + AHEAD, ...; step s + 1 goes into LDS while step s is computed.
+    // (Loops over sets are unrolled, so a set's registers are named at compile time.)
 #pragma unroll
-        for (int sub = 0; sub < 2; ++sub) {
-            const int k0 = key0 + sub * 32;
-            if (k0 <= wave_pos_max && k0 + 31 >= (window > 0 ? max(0, wave_pos_min - window + 1) : 0)) half_step(buf, sub, k0);
+    for (int u = 0; u < AHEAD; ++u) load_step(u, u, pages_cur);
+    store_step(0, 0);
+    __syncthreads();
+    for (int s0 = 0; s0 < nsteps; s0 += AHEAD) {
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u) {
+            const int s = s0 + u;
+            if (s >= nsteps) break;
+            const int buf = s & 1;
+            const int key0 = key_start + s * STEP;
+            const int ls = s + AHEAD;                   // the step whose loads start now
+            if (ls % 16 == 0) pages_cur = pages_next;
+            if (ls % 16 == 1) pages_next = pages_of(ls / 16 + 1);
+            load_step(u, ls, pages_cur);
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub) {
+                const int k0 = key0 + sub * 32;
+                if (k0 <= wave_pos_max && k0 + 31 >= (window > 0 ? max(0, wave_pos_min - window + 1) : 0)) {
+                    if (k0 + 31 <= wave_pos_min && k0 >= wave_lo_max) half_step(buf, sub, k0, std::true_type());
+                    else half_step(buf, sub, k0, std::false_type());
+                }
+            }
+            store_step((u + 1) % AHEAD, buf ^ 1);
+            __syncthreads();
         }
-        if (more) store_step(buf ^ 1);
-        __syncthreads();
     }
 
     // ---- normalise and write
@@ -273,11 +331,11 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     }
 }
 
-template <int HDP, int NBW>
+template <int HDP, int NBW, int AHEAD>
 int launch(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, bf16_t* out,
            const int* bt, int max_blocks, const int2* blk, const int4* req_info,
            int H, int Hkv, int hd, int ps, int window, float scale_log2e) {
-    auto kern = attn_prefill_kernel<HDP, NBW>;
+    auto kern = attn_prefill_kernel<HDP, NBW, AHEAD>;
     constexpr int lds = 2 * (STEP * (HDP + 8) + HDP * VROW) * 2;
     static bool set = false;
     if (!set) {
@@ -303,18 +361,18 @@ TUFF_EXPORT int tuff_attention_prefill(const void* q, const void* k_cache, const
                                        float scale, hipStream_t stream) {
     if (n_qblocks <= 0) return 0;
     if (hd > 256 || hd % 8 != 0 || page_size % 16 != 0 || Hkv <= 0 || H % Hkv != 0) return -2;
-    if (Hkv > 65535) return -2;
+    if (Hkv > 65535 || !(scale > 0.f)) return -2;
     const bf16_t* Q = (const bf16_t*)q;
     const bf16_t* K = (const bf16_t*)k_cache;
     const bf16_t* V = (const bf16_t*)v_cache;
     dim3 grid(n_qblocks, Hkv);
     const float sl = scale * 1.4426950408889634f;
-#define GO(HDP, NBW) return launch<HDP, NBW>(grid, stream, Q, K, V, (bf16_t*)out, block_table, max_blocks, (const int2*)blk, \
+#define GO(HDP, NBW, AHEAD) return launch<HDP, NBW, AHEAD>(grid, stream, Q, K, V, (bf16_t*)out, block_table, max_blocks, (const int2*)blk, \
                                              (const int4*)req_info, H, Hkv, hd, page_size, window, sl)
-    if (hd <= 32) GO(32, 2);
-    else if (hd <= 64) GO(64, 2);
-    else if (hd <= 96) GO(96, 2);
-    else if (hd <= 128) GO(128, 2);
-    else GO(256, 1);
+    if (hd <= 32) GO(32, 2, 3);
+    else if (hd <= 64) GO(64, 2, 3);
+    else if (hd <= 96) GO(96, 2, 2);
+    else if (hd <= 128) GO(128, 2, 2);
+    else GO(256, 1, 1);
 #undef GO
 }

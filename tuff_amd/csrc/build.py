@@ -20,7 +20,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ARCH = "gfx950"
 # -packed-fp32-ops off: the compiler must not form packed float32 instructions.
 FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC", "-shared", "-fvisibility=hidden",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
+         # MFMA results in ordinary vector registers: without this the compiler parks accumulators in
+         # the accumulation registers and copies them back and forth around every non-matrix use
+         "-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 HEADERS = ["common.h"]
 
 MODULES = {

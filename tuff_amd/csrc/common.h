@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 #define TUFF_EXPORT extern "C" __attribute__((visibility("default")))
 
@@ -49,6 +50,16 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 #pragma unroll
     for (int i = 0; i < NWAVES; ++i) t += scratch[i];
     return t;
+}
+
+// f(std::integral_constant<int, 0>()), ..., f(std::integral_constant<int, N - 1>()): a loop whose
+// index is a compile-time constant inside the body (register arrays stay registers).
+template <int N, typename F, int I = 0>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>());
+        static_for<N, F, I + 1>(static_cast<F&&>(f));
+    }
 }
 
 static inline int launch_status() { return (int)hipGetLastError(); }

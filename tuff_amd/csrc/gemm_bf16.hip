@@ -16,7 +16,6 @@
 // and eight consecutive k at 8 * (l / 16); it receives rows 4 * (l / 16) + 0..3, column (l % 16)
 // of the 16x16 result.
 #include "common.h"
-#include <type_traits>
 
 // OUT_SWIGLU: the rows of W are gate and up rows interleaved (2f: gate f, 2f+1: up f); the
 // output is bfloat16 [M, N/2] with y[m, f] = silu(g) * u, silu(g) = g / (1 + exp(-g)).
@@ -26,14 +25,6 @@ namespace {
 
 __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-}
-
-template <int N, typename F, int I = 0>
-__device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>());
-        static_for<N, F, I + 1>(static_cast<F&&>(f));
-    }
 }
 
 template <int MODE>
