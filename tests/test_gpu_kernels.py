@@ -268,6 +268,32 @@ def test_qkv_post(gpu, H, Hkv, hd, ps, dt):
     assert (k2.cpu().double().reshape(T, Hkv, hd) - wantk).abs().max() <= tol * float(wantk.abs().max())
 
 
+def test_qkv_post_many_tokens_equal_few(gpu):
+    """With many tokens a wave takes several heads of a token in turn; the result is, bit for
+    bit, that of the same tokens in small steps."""
+    from tuff_amd.csrc import ops
+    T, H, Hkv, hd, ps, dt = 3000, 7, 3, 48, 16, torch.bfloat16
+    qkv = _r(T, (H + 2 * Hkv) * hd, seed=11, dtype=dt).to(gpu)
+    qw, kw = (1 + _r(hd, seed=12, scale=0.1)).to(gpu), (1 + _r(hd, seed=13, scale=0.1)).to(gpu)
+    pos = torch.arange(T, dtype=torch.int32, device=gpu) + 5
+    slots = torch.randperm(T + 32, generator=torch.Generator().manual_seed(1))[:T].to(torch.int32).to(gpu)
+    inv_freq = (10000.0 ** (-2 * torch.arange(hd // 2, dtype=torch.float64) / hd)).float().to(gpu)
+    n_pages = (T + 32) // ps + 1
+
+    def run(step):
+        kc = torch.zeros(n_pages, Hkv, ps, hd, dtype=dt, device=gpu)
+        vc = torch.zeros(n_pages, Hkv, hd, ps, dtype=dt, device=gpu)
+        q = torch.empty(T, H * hd, dtype=dt, device=gpu)
+        for a in range(0, T, step):
+            b = min(T, a + step)
+            ops.qkv_post(qkv[a:b], q[a:b], H=H, Hkv=Hkv, hd=hd, positions=pos[a:b], eps=1e-5, q_norm_w=qw, k_norm_w=kw,
+                         inv_freq=inv_freq, rotary_dim=hd, k_cache=kc, v_cache=vc, slot_mapping=slots[a:b], page_size=ps)
+        return q, kc, vc
+    q1, k1, v1 = run(T)
+    q2, k2, v2 = run(100)
+    assert torch.equal(q1, q2) and torch.equal(k1, k2) and torch.equal(v1, v2)
+
+
 # -------------------------------------------------------------------------- attention
 def _attention_reference(q, K, V, pos, window, scale):
     """q [H, hd]; K, V [n, Hkv, hd] of one request; keys lo..pos."""
@@ -607,6 +633,46 @@ def test_shortconv_single_token_kernel_equals_the_general_pair(gpu, d, K, dt):
         ops.shortconv_state(bcx, s1, q_start=ar, q_len=ones, state_slot=slots, K=K)
         ops.shortconv_decode(bcx, w, s2, o2, state_slot=slots, K=K)
         assert torch.equal(o1, o2) and torch.equal(s1, s2), step
+
+
+@pytest.mark.parametrize("d,K", [(64, 3), (96, 4), (240, 2), (2048, 3), (300, 7)])
+def test_shortconv_long_portions_equal_single_tokens(gpu, d, K):
+    """Portions of more than 16 tokens (eight channels a thread in bfloat16) give, bit for bit,
+    what the same tokens give one at a time."""
+    from tuff_amd.csrc import ops
+    dt = torch.bfloat16
+    lens, cuts = [70, 33], [[40, 30], [33]]
+    w = _r(d, K, seed=20, dtype=dt).to(gpu)
+    bcx_all = [_r(n, 3 * d, seed=21 + i, dtype=dt).to(gpu) for i, n in enumerate(lens)]
+    slots = [2, 0]
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
+    # one token at a time
+    s1 = torch.zeros(4, K - 1, d, device=gpu)
+    single = [[], []]
+    for r in range(2):
+        for t in range(lens[r]):
+            o = torch.empty(1, d, dtype=dt, device=gpu)
+            ops.shortconv_decode(bcx_all[r][t:t + 1], w, s1, o, state_slot=i32([slots[r]]), K=K)
+            single[r].append(o)
+    # in portions, both requests in one step where both have one
+    s2 = torch.zeros(4, K - 1, d, device=gpu)
+    got = [[], []]
+    done = [0, 0]
+    for step in range(2):
+        who = [r for r in range(2) if step < len(cuts[r])]
+        q_len = [cuts[r][step] for r in who]
+        q_start = [sum(q_len[:i]) for i in range(len(who))]
+        bcx = torch.cat([bcx_all[r][done[r]:done[r] + n] for r, n in zip(who, q_len)])
+        out = torch.empty(bcx.shape[0], d, dtype=dt, device=gpu)
+        meta = dict(q_start=i32(q_start), state_slot=i32([slots[r] for r in who]))
+        ops.shortconv_fwd(bcx, w, s2, out, req_of_token=i32([i for i, n in enumerate(q_len) for _ in range(n)]), K=K, **meta)
+        ops.shortconv_state(bcx, s2, q_len=i32(q_len), K=K, **meta)
+        for i, r in enumerate(who):
+            got[r].append(out[q_start[i]:q_start[i] + q_len[i]])
+            done[r] += q_len[i]
+    for r in range(2):
+        assert torch.equal(torch.cat(got[r]), torch.cat(single[r])), r
+    assert torch.equal(s1, s2)
 
 
 def test_shortconv_last_tap_is_the_current_token(gpu):
