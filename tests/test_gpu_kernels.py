@@ -133,7 +133,7 @@ def test_gemm_that_prepares_the_next_norm(gpu, M, d, K1, N2):
     eps = 1e-5
     res = res0.to(gpu)
     xw = torch.empty(M, d, dtype=torch.bfloat16, device=gpu)
-    ss = torch.full((-(-d // 16), 16), float("nan"), device=gpu)
+    ss = torch.full((ops.gemm_emit_tiles(d, K1), 16), float("nan"), device=gpu)
     ops.gemm_accum_emit(a.to(gpu), w1.to(gpu), res, nw.to(gpu), xw, ss)
     want_res = res0.double() + a.double() @ w1.double().T
     assert (res.cpu().double() - want_res).abs().max() <= 1e-5 * float(want_res.abs().max()) + 1e-6 * K1

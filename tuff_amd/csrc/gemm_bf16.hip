@@ -250,7 +250,7 @@ constexpr int SK_CHUNK = 128;
 // NORM_SCALED product that follows.
 enum : int { NORM_NONE = 0, NORM_INSIDE = 1, NORM_SCALED = 2 };
 
-template <int NW, int MODE, int NORM, bool EMIT>
+template <int NW, int MODE, int NORM, bool EMIT, int COLS>
 __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const void* __restrict__ Xv, const bf16_t* __restrict__ W,
                                                                        void* __restrict__ Y, int M, int N, int K,
                                                                        const float* __restrict__ norm_w, float eps,
@@ -263,9 +263,10 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
     extern __shared__ __attribute__((aligned(16))) float nw_lds[];       // NORM_INSIDE: the norm weight, K floats
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
     const int r16 = lane % 16, g = lane / 16;
-    const long long n0 = (long long)blockIdx.x * 16;
+    const long long n0 = (long long)blockIdx.x * COLS;
     const int nchunks = (K + SK_CHUNK - 1) / SK_CHUNK;
     const bf16_t* X = (const bf16_t*)Xv;
+    const long long w_rows = min((long long)N, n0 + COLS);               // this tile's rows of W end here
     const float* xrow = nullptr;
     if (NORM == NORM_INSIDE && r16 < M) xrow = (const float*)Xv + (long long)(rows ? rows[r16] : r16) * K;
 
@@ -274,7 +275,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
     float y_old = 0.f, emit_w = 0.f;
     if (MODE == OUT_F32_ACCUM && tid < 256) {
         const long long row = (tid / 64) * 4 + tid % 4, col = n0 + (tid / 4) % 16;
-        if (row < M && col < N) {
+        if (row < M && col < w_rows) {
             y_old = ((const float*)Y)[row * N + col];
             if (EMIT) emit_w = emit_nw[col];
         }
@@ -288,7 +289,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
         // instruction j of the wave reads bytes 64 j .. 64 j + 63 of the chunk of each of its 16 rows
         const int kb = c * SK_CHUNK + g * 8;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) o.b[j] = load8(W, n0 + r16, N, kb + j * 32, K);
+        for (int j = 0; j < 4; ++j) o.b[j] = load8(W, n0 + r16, w_rows, kb + j * 32, K);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int k = kb + j * 32;
@@ -333,12 +334,15 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
         for (int k = tid * 4; k < K; k += NW * WAVE * 4) *(f32x4*)(&nw_lds[k]) = *(const f32x4*)(norm_w + k);
         __syncthreads();
     }
+    // NORM_SCALED: 16 parts x 16 rows; part p adds the tiles p, p + 16, ... of its row.  The first
+    // sixteen of them are only asked for here and added after the products, when they have long
+    // arrived; a wider matrix adds the rest right away.
+    float ss_part[16], ss_rest = 0.f;
     if (NORM == NORM_SCALED && tid < 256) {
-        // 16 parts x 16 rows: part p adds the tiles p, p + 16, ... of its row
         const int row = tid % 16, part = tid / 16;
-        float t = 0.f;
-        for (int j = part; j < n_ss; j += 16) t += ss_in[(long long)j * 16 + row];
-        ssq[part][row] = t;
+#pragma unroll
+        for (int u = 0; u < 16; ++u) ss_part[u] = (part + 16 * u < n_ss) ? ss_in[(long long)(part + 16 * u) * 16 + row] : 0.f;
+        for (int j = part + 256; j < n_ss; j += 16) ss_rest += ss_in[(long long)j * 16 + row];
     }
     for (; i < nchunks; i += 2 * NW) {
         const bool more = i + NW < nchunks;
@@ -351,6 +355,12 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) red[wave][lane][e] = acc[e];
+    if (NORM == NORM_SCALED && tid < 256) {
+        float t = ss_rest;
+#pragma unroll
+        for (int u = 0; u < 16; ++u) t += ss_part[u];
+        ssq[tid / 16][tid % 16] = t;
+    }
     if (NORM == NORM_INSIDE) {
         ss += __shfl_xor(ss, 16, WAVE);
         ss += __shfl_xor(ss, 32, WAVE);
@@ -363,8 +373,9 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
         float v = red[0][l][e];
 #pragma unroll
         for (int w = 1; w < NW; ++w) v += red[w][l][e];
-        const long long row = (l / 16) * 4 + e, col = n0 + (l % 16);
-        if (NORM != NORM_NONE) {
+        const long long col = n0 + (l % 16);
+        const long long row = col < w_rows ? (l / 16) * 4 + e : 16;     // columns beyond the tile: no row
+        if (NORM != NORM_NONE && row < 16) {
             constexpr int PARTS = NORM == NORM_INSIDE ? NW : 16;
             float total = ssq[0][row];
 #pragma unroll
@@ -389,7 +400,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
             if (row < M && col < N) ((float*)Y)[row * N + col] = y_old + v;
         } else {
             const float partner = (MODE == OUT_SWIGLU) ? __shfl_xor(v, 4, WAVE) : 0.f;   // thread tid ^ 4 holds column col ^ 1
-            store_elem<MODE>(Y, row, col, M, N, v, partner);
+            store_elem<MODE>(Y, row, col, min(M, 16), N, v, partner);
         }
     }
 }
@@ -515,15 +526,19 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* __restr
     store_out<MODE>(Y, i, v);
 }
 
-struct SkinnyPlan { int tiles, waves, slices, chunks_per_slice; long long ws_floats; };
+struct SkinnyPlan { int tiles, waves, slices, chunks_per_slice, cols; long long ws_floats; };
 
 // How a skinny product is cut.  Depends on N and K (and on which of the two kernels M selects).
 SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16) {
     const int nchunks = ceil_div(K, SK_CHUNK);
     SkinnyPlan p;
     p.slices = 1; p.chunks_per_slice = nchunks; p.ws_floats = 0; p.waves = 4;
+    p.cols = 16;
     if (M <= 16) {
-        p.tiles = ceil_div(N, 16);
+        // tiles of 8 columns where 16 would leave CUs without a workgroup (half of each MFMA idles,
+        // which costs nothing here: these products wait for memory)
+        if (ceil_div(N, 16) <= 128) p.cols = 8;
+        p.tiles = ceil_div(N, p.cols);
         // enough waves in flight to cover the latency of HBM, at least one chunk a wave
         while (p.waves < max_waves && p.tiles * p.waves < 3072 && nchunks >= 2 * p.waves) p.waves *= 2;
     } else {
@@ -550,9 +565,10 @@ int launch_skinny16(const void* X, const bf16_t* W, void* Y, int M, int N, int K
     const SkinnyPlan p = plan_skinny(M, N, K, NORM == NORM_INSIDE ? 8 : 16);
     dim3 grid(p.tiles);
     const size_t lds = NORM == NORM_INSIDE ? (size_t)K * sizeof(float) : 0;
-#define GO(NW) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<NW, MODE, NORM, EMIT>), grid, dim3(NW * WAVE), lds, stream, X, W, Y, M, N, K, \
-                                  x.norm_w, x.eps, x.rows, x.ss_in, x.n_ss, x.emit_nw, x.emit_xw, x.emit_ss)
-    if (p.waves == 4) GO(4); else if (p.waves == 8) GO(8); else GO(16);
+#define GO(NW, COLS) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<NW, MODE, NORM, EMIT, COLS>), grid, dim3(NW * WAVE), lds, stream, \
+                                        X, W, Y, M, N, K, x.norm_w, x.eps, x.rows, x.ss_in, x.n_ss, x.emit_nw, x.emit_xw, x.emit_ss)
+    if (p.cols == 16) { if (p.waves == 4) GO(4, 16); else if (p.waves == 8) GO(8, 16); else GO(16, 16); }
+    else { if (p.waves == 4) GO(4, 8); else if (p.waves == 8) GO(8, 8); else GO(16, 8); }
 #undef GO
     return launch_status();
 }
@@ -612,6 +628,10 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
     return launch_status();
 }
 }  // namespace
+
+// Tiles of columns a product of at most 16 rows is cut into: the first dimension of the sums of
+// squares tuff_gemm_bf16_accum_emit leaves.
+TUFF_EXPORT int tuff_gemm_bf16_emit_tiles(int N, int K) { return plan_skinny(1, N, K).tiles; }
 
 // Work space a product of this shape needs: *ws_floats float32 for partial tiles (0: none).
 TUFF_EXPORT int tuff_gemm_bf16_workspace(int M, int N, int K, long long* ws_floats) {

@@ -38,6 +38,7 @@ _SIGNATURES = {
     "gemm_bf16": {
         "tuff_gemm_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
         "tuff_gemm_bf16_workspace": [_c_int, _c_int, _c_int, ctypes.POINTER(_c_ll)],
+        "tuff_gemm_bf16_emit_tiles": [_c_int, _c_int],
         "tuff_gemm_bf16_accum_emit": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                                       _c_void_p, _c_void_p],
         "tuff_gemm_bf16_scaled": [_c_void_p, _c_void_p, _c_int, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
@@ -256,10 +257,22 @@ def gemm_normed(x: torch.Tensor, norm_w: torch.Tensor, eps: float, w: torch.Tens
         out.data_ptr(), M, N, K, mode, _stream()), "gemm_bf16_normed")
 
 
+_emit_tiles: dict = {}
+
+
+def gemm_emit_tiles(N: int, K: int) -> int:
+    """Tiles of columns gemm_accum_emit cuts a product with N outputs and inner size K into."""
+    key = (N, K)
+    if key not in _emit_tiles:
+        _emit_tiles[key] = int(load("gemm_bf16").tuff_gemm_bf16_emit_tiles(N, K))
+    return _emit_tiles[key]
+
+
 def gemm_accum_emit(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, next_norm_w: torch.Tensor,
                     xw: torch.Tensor, ss: torch.Tensor) -> None:
     """residual += x @ w.T for at most 16 rows, and for the RMSNorm that follows: xw = the new
-    residual times next_norm_w as bfloat16, ss [ceil(N/16), 16] = per-tile sums of squares of each row."""
+    residual times next_norm_w as bfloat16, ss [gemm_emit_tiles(N, K), 16] = per-tile sums of squares
+    of each row."""
     M, K = x.shape
     N = w.shape[0]
     _gpu("x", x, torch.bfloat16)
@@ -267,7 +280,7 @@ def gemm_accum_emit(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, ne
     _gpu("residual", residual, torch.float32, (M, N))
     _gpu("next_norm_w", next_norm_w, torch.float32, (N,))
     _gpu("xw", xw, torch.bfloat16, (M, N))
-    _gpu("ss", ss, torch.float32, (-(-N // 16), 16))
+    _gpu("ss", ss, torch.float32, (gemm_emit_tiles(N, K), 16))
     if M > NORMED_MAX_ROWS or K % 8:
         raise KernelError(f"gemm_accum_emit: at most {NORMED_MAX_ROWS} rows, inner size a multiple of 8")
     _check(load("gemm_bf16").tuff_gemm_bf16_accum_emit(x.data_ptr(), w.data_ptr(), residual.data_ptr(), M, N, K,

@@ -96,7 +96,7 @@ class Linear:
                     and T <= ops.NORMED_MAX_ROWS):
                 # the norm that follows reads the sum just made: leave it its operand and row sums
                 xw = torch.empty(T, self.out_features, dtype=torch.bfloat16, device=dev)
-                ss = torch.empty(-(-self.out_features // 16), 16, dtype=torch.float32, device=dev)
+                ss = torch.empty(ops.gemm_emit_tiles(self.out_features, self.in_features), 16, dtype=torch.float32, device=dev)
                 ops.gemm_accum_emit(x, w, accumulate_into, nxt.weight_f32, xw, ss)
                 nxt.announce_operand(accumulate_into, xw, ss)
                 return None
