@@ -74,7 +74,10 @@ def run_decode(llm, cfg, batch: int, ctx_end: int, steps: int, warmup: int, seed
     from tuff_amd.sampling.params import SamplingParams
     g = torch.Generator().manual_seed(seed)
     eng = llm.engine
-    n_new = steps + warmup
+    # two tokens more than are timed: the loop starts a step before it has accounted for the one
+    # before, so both time marks wait for a step that is already under way, and the window between
+    # them holds exactly `steps` steps only if the run goes on past it
+    n_new = steps + warmup + 2
     n_prompt = ctx_end - n_new
     sched = llm.new_scheduler()
     for b in range(batch):

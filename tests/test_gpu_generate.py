@@ -141,6 +141,32 @@ def test_eos_stops_a_request(gpu):
     assert out.token_ids == free and out.finish_reason == "length"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_starting_the_next_step_early_changes_nothing(gpu, dtype):
+    """Requests that finish at different steps, by length and by the end token, greedy beside
+    seeded temperature: the same tokens whether or not decode steps are started before the tokens
+    of the step before have reached the host."""
+    from tuff_amd.engine.llm import LLM
+    from tuff_amd.sampling.params import SamplingParams
+    V = util.TINY_B["vocab_size"]
+    prompts = [util.rand_tokens(n, V, 70 + n) for n in (3, 17, 40, 9)]
+    params = [SamplingParams(max_new_tokens=25), SamplingParams(temp=0.7, seed=3, max_new_tokens=40),
+              SamplingParams(max_new_tokens=33), SamplingParams(temp=1.1, top_k=20, seed=4, max_new_tokens=12)]
+    got = {}
+    for ahead in (False, True):
+        llm = LLM(util.model_folder("B", dtype), dtype=dtype, max_num_seqs=4, max_batched_tokens=32, ctx_size=128,
+                  run_ahead=ahead)
+        free = llm.generate(prompts, params)
+        assert (llm.last_stats["steps_started_ahead"] > 20) == ahead
+        llm.engine.model.eos_token_id = free[2].token_ids[10]         # request 2 stops early, the others go on
+        stopped = llm.generate(prompts, params)
+        assert stopped[2].finish_reason == "stop" and len(stopped[2].token_ids) <= 11
+        got[ahead] = [o.token_ids for o in free] + [o.token_ids for o in stopped]
+        llm.engine.manager.check()
+        assert not llm.engine.manager.live()
+    assert got[False] == got[True]
+
+
 def _tuff(*args):
     return subprocess.run([sys.executable, os.path.join(util.ROOT, "bin", "tuff"), *args],
                           capture_output=True, text=True, timeout=300)

@@ -236,7 +236,6 @@ def test_seeded_sampling_state_survives_preemption():
     sched = make(ex)
     sched.add(r)
     first = [r.sampler.rng.uniform() for _ in range(2)]
-    sched._preempt_for_test = None
     fresh = SamplerState(p)
     assert first == [fresh.rng.uniform() for _ in range(2)]
     nxt = fresh.rng.uniform()
@@ -244,3 +243,125 @@ def test_seeded_sampling_state_survives_preemption():
     ex.begin("x")
     sched._preempt(r)
     assert r.sampler.rng.uniform() == nxt and r.num_computed == 0 and sched.waiting[0] is r
+
+
+# ---------------------------------------------------------------- deciding a step ahead
+def run_ahead(sched, ex, eos=None):
+    """The loop of LLM.run over the fake executor: where schedule_ahead() allows, the next step
+    is 'started' (the executor extends the cache and records a stand-in token) before the
+    current step's tokens are handed to update()."""
+    steps, ahead = [], 0
+    under_way = None
+    while under_way is not None or sched.has_unfinished():
+        if under_way is None:
+            batch = sched.schedule()
+            assert batch, "the scheduler stalled"
+            sampled = ex.step(batch)
+        else:
+            batch, sampled = under_way
+            under_way = None
+        nxt = sched.schedule_ahead(batch)
+        if nxt is not None:
+            # the executor sees the real token of every request, as the GPU does
+            for s in nxt:
+                s.tokens = [sampled[s.request.id]]
+            under_way = (nxt, ex.step_stale_ok(nxt, sched))
+            ahead += 1
+        sched.update(batch, sampled)
+        steps.append(batch)
+    return steps, ahead
+
+
+class AheadExecutor(FakeExecutor):
+    def step_stale_ok(self, batch, sched):
+        """Like step(); a request may end (and be released) while this step is under way."""
+        return self.step(batch)
+
+    def end(self, rid):
+        self.manager.release(rid)
+        self.fed.pop(rid, None)
+
+
+def test_a_step_decided_ahead_feeds_the_same_tokens():
+    prompts = {"a": list(range(9)), "b": list(range(40, 47)), "c": list(range(100, 103))}
+    new = {"a": 12, "b": 7, "c": 20}
+    outs = {}
+    for mode in ("plain", "ahead"):
+        ex = AheadExecutor()
+        sched = make(ex, max_batched_tokens=8)
+        reqs = {k: Request(k, prompts[k], SamplingParams(max_new_tokens=new[k])) for k in prompts}
+        for r in reqs.values():
+            sched.add(r)
+        if mode == "plain":
+            run(sched, ex)
+        else:
+            _, ahead = run_ahead(sched, ex)
+            assert ahead >= 10
+        outs[mode] = {k: r.output for k, r in reqs.items()}
+        assert all(r.finish_reason == "length" for r in reqs.values())
+        assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == 64
+    assert outs["plain"] == outs["ahead"]
+    assert outs["plain"]["a"] == expected_output(prompts["a"], 12)
+
+
+def test_no_step_is_decided_ahead_when_the_next_one_is_not_plain():
+    ex = AheadExecutor()
+    sched = make(ex, max_batched_tokens=8)
+    a = Request("a", list(range(7)), SamplingParams(max_new_tokens=3))
+    b = Request("b", list(range(20, 26)), SamplingParams(max_new_tokens=30))
+    sched.add(a)
+    batch = sched.schedule()                      # a's prompt: 7 tokens, samples
+    sched.add(b)
+    assert sched.schedule_ahead(batch) is None    # someone waits for admission
+    sched.update(batch, ex.step(batch))
+    batch = sched.schedule()                      # a decodes, b's prompt
+    assert [len(s.tokens) for s in batch] == [1, 6]
+    sampled = ex.step(batch)
+    nxt = sched.schedule_ahead(batch)             # a has 1 of 3, gets its second now: the third is still open
+    assert nxt is not None and [(s.request.id, s.start, s.samples) for s in nxt] == [("a", 8, True), ("b", 6, True)]
+    for s in nxt:
+        s.tokens = [sampled[s.request.id]]
+    sampled2 = ex.step(nxt)
+    sched.update(batch, sampled)
+    assert sched.schedule_ahead(nxt) is None      # a gets its last token in nxt
+    sched.update(nxt, sampled2)
+    assert a.finish_reason == "length" and len(a.output) == 3
+
+
+def test_deciding_ahead_stops_where_pages_run_out():
+    """Three pages of four tokens for two requests that need two each: when both want their second
+    page no step is decided ahead, schedule() preempts, and the output is what it would have been."""
+    outs = {}
+    for mode in ("plain", "ahead"):
+        ex = AheadExecutor(num_pages=3)
+        sched = make(ex)
+        reqs = [Request(k, list(range(i, i + 3)), SamplingParams(max_new_tokens=4)) for i, k in enumerate("ab")]
+        for r in reqs:
+            sched.add(r)
+        if mode == "plain":
+            run(sched, ex)
+        else:
+            run_ahead(sched, ex)
+        assert sched.num_preemptions >= 1
+        outs[mode] = [r.output for r in reqs]
+        assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == 3
+    assert outs["plain"] == outs["ahead"] == [expected_output(range(i, i + 3), 4) for i in range(2)]
+
+
+def test_a_request_that_ends_while_the_next_step_is_under_way():
+    ex = AheadExecutor()
+    sched = make(ex, eos_token_id=None)
+    a = Request("a", list(range(5)), SamplingParams(max_new_tokens=30))
+    b = Request("b", list(range(50, 58)), SamplingParams(max_new_tokens=30))
+    sched.add(a)
+    sched.add(b)
+    free_run_a = expected_output(range(5), 30)
+    sched.eos_token_id = free_run_a[6]            # a stops after its 7th token
+    steps, ahead = run_ahead(sched, ex)
+    cut = free_run_a.index(free_run_a[6]) + 1
+    assert a.output == free_run_a[:cut] and a.finish_reason == "stop"
+    assert len(b.output) <= 30 and b.finish_reason in ("length", "stop")
+    want_b = expected_output(range(50, 58), 30)
+    assert b.output == want_b[:len(b.output)]
+    assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == 64
+    ex.manager.check()

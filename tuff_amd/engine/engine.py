@@ -105,10 +105,13 @@ class Engine:
         return self.manager.length(req_id)
 
     # ------------------------------------------------------------------------ step
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Runs one batch.  Returns float32 logits [wanted, vocab] on the device, in the order
         of the entries and of their `want` lists, or None if nothing is wanted.
-        Raises OutOfPages (and leaves every request as it was) if the pool is too small."""
+        Raises OutOfPages (and leaves every request as it was) if the pool is too small.
+        device_tokens (int32 on the device, one per token of the step): the token ids are taken
+        from there, by a copy on the stream, instead of from the entries (whose ids then only
+        stand in); for a caller that starts a step before it has seen the last one's tokens."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         entries = [e for e in entries if len(e.tokens) > 0]
         if not entries:
@@ -136,17 +139,25 @@ class Engine:
             for e in done:
                 self.manager.truncate(e.req_id, self.manager.length(e.req_id) - len(e.tokens))
             raise
+        if device_tokens is not None:
+            n = sum(len(e.tokens) for e in entries)
+            if device_tokens.dtype != torch.int32 or device_tokens.shape != (n,) or device_tokens.device != self.device:
+                for e in done:
+                    self.manager.truncate(e.req_id, self.manager.length(e.req_id) - len(e.tokens))
+                raise ValueError(f"device_tokens must be int32 [{n}] on {self.device}")
         self.steps += 1
         if self.use_graphs and all(len(e.tokens) == 1 for e in entries):
-            return self._decode_step(entries)
+            return self._decode_step(entries, device_tokens)
         ctx = build_context(entries, self.manager, self.device, self.model.vocab_size)
+        if device_tokens is not None:
+            ctx.tokens.copy_(device_tokens)
         return self.model.forward(ctx, self.storage.views)
 
     # --------------------------------------------------------------- recorded decode
     GRAPH_TABLE_BUCKET = 64          # block tables of recorded steps are padded to multiples of this
     MAX_GRAPHS = 12
 
-    def _decode_step(self, entries) -> Optional[torch.Tensor]:
+    def _decode_step(self, entries, device_tokens=None) -> Optional[torch.Tensor]:
         """A step of single tokens.  The first step of a shape runs eagerly on persistent
         buffers and is then recorded; later steps of that shape refresh the buffer and replay.
         Everything a kernel's launch depends on (batch size, table width, number of key
@@ -162,7 +173,7 @@ class Engine:
                 self._graphs.pop(next(iter(self._graphs)))
             g = _RecordedStep(p, self.device, width * self.page_size)
             self._graphs[key] = g
-            g.refresh(p)
+            g.refresh(p, device_tokens)
             logits = self.model.forward(g.ctx, self.storage.views)
             try:
                 g.record(lambda: self.model.forward(g.ctx, self.storage.views))
@@ -174,7 +185,7 @@ class Engine:
                 self._graphs.clear()
             return logits
         self._graphs[key] = self._graphs.pop(key)           # most recently used last
-        g.refresh(p)
+        g.refresh(p, device_tokens)
         g.graph.replay()
         self.graph_replays += 1
         return g.logits
@@ -191,11 +202,13 @@ class _RecordedStep:
         self.graph = None
         self.logits = None
 
-    def refresh(self, p) -> None:
+    def refresh(self, p, device_tokens=None) -> None:
         self.copied.synchronize()                           # the last copy out of `pinned` is done
         self.pinned.numpy()[:] = p.buf
         self.dev.copy_(self.pinned, non_blocking=True)
         self.copied.record()
+        if device_tokens is not None:
+            self.ctx.tokens.copy_(device_tokens)
 
     def record(self, forward) -> None:
         torch.cuda.synchronize()

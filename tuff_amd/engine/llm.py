@@ -33,7 +33,8 @@ class Generation:
 class LLM:
     def __init__(self, model=None, *, engine: Optional[Engine] = None, dtype="bfloat16", device="cuda:0",
                  max_num_seqs: int = 8, max_batched_tokens: int = 2048, ctx_size: Optional[int] = None,
-                 page_size: int = 16, num_pages: Optional[int] = None, ignore_eos: bool = False):
+                 page_size: int = 16, num_pages: Optional[int] = None, ignore_eos: bool = False,
+                 run_ahead: bool = True):
         """model: a folder with config.json and model.safetensors.  ctx_size (-c): the longest
         prompt + generation of one request.  num_pages: size of the page pool; default: room for
         max_num_seqs requests of ctx_size."""
@@ -54,6 +55,7 @@ class LLM:
         self.max_num_seqs = min(max_num_seqs, engine.manager.num_slots)
         self.max_batched_tokens = max_batched_tokens
         self.ignore_eos = ignore_eos
+        self.run_ahead = run_ahead
         self.sampler = Sampler(engine.device)
         self._ids = itertools.count()
         self.last_stats: dict = {}
@@ -65,28 +67,50 @@ class LLM:
                          max_model_len=self.ctx_size, eos_token_id=eos)
 
     def run(self, sched: Scheduler, on_step=None) -> None:
-        """Steps until every request of the scheduler has finished."""
-        steps = tokens = 0
-        while sched.has_unfinished():
-            batch = sched.schedule()
-            if not batch:
-                if sched.has_unfinished():
-                    raise RuntimeError("the scheduler made no progress: no request fits the cache")
-                break
+        """Steps until every request of the scheduler has finished.
+
+        While the requests only decode, the next step is started before the tokens of the
+        current one have reached the host: it takes them from the sampler's output on the device
+        (`run_ahead`).  The host then accounts for a step while the GPU runs the next one."""
+        steps = tokens = ahead_steps = 0
+
+        def start(batch, device_tokens=None):
             entries = [StepEntry(s.request.id, s.tokens, [len(s.tokens) - 1] if s.samples else [])
                        for s in batch]
-            logits = self.engine.step(entries)
+            logits = self.engine.step(entries, device_tokens)
             sampling = [s.request for s in batch if s.samples]
+            pending = self.sampler.launch(logits, [r.sampler for r in sampling]) if sampling else None
+            return sampling, pending
+
+        under_way = None                                  # a step started ahead: (batch, sampling, pending)
+        while under_way is not None or sched.has_unfinished():
+            if under_way is None:
+                batch = sched.schedule()
+                if not batch:
+                    if sched.has_unfinished():
+                        raise RuntimeError("the scheduler made no progress: no request fits the cache")
+                    break
+                sampling, pending = start(batch)
+            else:
+                batch, sampling, pending = under_way
+                under_way = None
+            if self.run_ahead and pending is not None and len(sampling) == len(batch) \
+                    and not any(self.sampler.needs_history(r.sampler) for r in sampling):
+                nxt = sched.schedule_ahead(batch)
+                if nxt is not None:
+                    under_way = (nxt,) + start(nxt, pending.out)
+                    ahead_steps += 1
             sampled = {}
-            if sampling:
-                toks = self.sampler.sample(logits, [r.sampler for r in sampling])
-                sampled = {r.id: t for r, t in zip(sampling, toks)}
+            if pending is not None:
+                sampled = {r.id: t for r, t in zip(sampling, pending.tokens())}
+            live = [s for s in batch if s.request.status != "finished"]
             sched.update(batch, sampled)
             steps += 1
-            tokens += sum(len(s.tokens) for s in batch)
+            tokens += sum(len(s.tokens) for s in live)
             if on_step is not None:
-                on_step(batch, sampled)
-        self.last_stats = {"steps": steps, "tokens_run": tokens, "preemptions": sched.num_preemptions}
+                on_step(live, {s.request.id: sampled[s.request.id] for s in live if s.samples})
+        self.last_stats = {"steps": steps, "tokens_run": tokens, "preemptions": sched.num_preemptions,
+                           "steps_started_ahead": ahead_steps}
 
     def generate(self, prompts: Sequence[Sequence[int]], params=None) -> list[Generation]:
         """prompts: token id lists.  params: one SamplingParams for all, or one per prompt."""

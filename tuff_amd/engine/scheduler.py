@@ -225,12 +225,41 @@ class Scheduler:
             budget -= n
         return out
 
+    def schedule_ahead(self, prev: list[Scheduled]) -> Optional[list[Scheduled]]:
+        """The step after `prev`, decided before prev's tokens are known: every request of prev
+        feeds the token it is about to get (Scheduled.tokens holds a stand-in).  Only in the
+        plain case: prev draws a token for every running request, none of them can finish by
+        length with it, nobody waits for admission, and the pages for one more token each are
+        free.  Otherwise None: decide with schedule() once prev has been accounted.
+        A request that does finish with prev's token (end of sequence) still runs in the step
+        returned here; update() ignores it."""
+        if self.waiting or not prev or len(prev) != len(self.running):
+            return None
+        promised = [0] * len(self.manager.groups)
+        out = []
+        for s in prev:
+            req = s.request
+            if not s.samples or req.status != RUNNING:
+                return None
+            n_out = len(req.output) + 1                      # with the token prev is drawing
+            if n_out >= req.params.max_new_tokens:
+                return None
+            if self.max_model_len is not None and len(req.prompt) + n_out >= self.max_model_len:
+                return None
+            if not self._fits(req, 1, promised):
+                return None
+            self._promise(req, 1, promised)
+            out.append(Scheduled(req, s.start + len(s.tokens), [0], True))
+        return out
+
     def update(self, scheduled: list[Scheduled], sampled: dict) -> list[Request]:
         """sampled: {request id: token} for every Scheduled with samples=True.
         Returns the requests that finished in this step."""
         done = []
         for s in scheduled:
             req = s.request
+            if req.status == FINISHED:                       # finished while this step was under way
+                continue
             req.num_computed += len(s.tokens)
             if not s.samples:
                 continue

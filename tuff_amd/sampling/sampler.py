@@ -16,6 +16,27 @@ from ..csrc import ops
 from .params import SamplerState
 
 
+class PendingSample:
+    """Tokens that are being drawn: `out` (int32 [R], device) is valid for kernels launched after
+    this one on the same stream; tokens() waits for the copy to the host."""
+
+    def __init__(self, out: torch.Tensor, states: Sequence[SamplerState]):
+        self.out, self.states = out, list(states)
+        self.host = torch.empty(out.shape, dtype=torch.int32, pin_memory=True)
+        self.host.copy_(out, non_blocking=True)
+        self.done = torch.cuda.Event()
+        self.done.record()
+        self._tokens = None
+
+    def tokens(self) -> list[int]:
+        if self._tokens is None:
+            self.done.synchronize()
+            self._tokens = self.host.tolist()
+            for s, t in zip(self.states, self._tokens):
+                s.accept(t)
+        return self._tokens
+
+
 class Sampler:
     def __init__(self, device):
         self.device = device
@@ -24,11 +45,24 @@ class Sampler:
         """logits: float32 [R, vocab] on the device (changed in place where a penalty applies);
         states: the R requests' sampler states, in row order.  Returns R token ids and records
         them in the states' rings."""
+        if logits.shape[0] == 0 and not states:
+            return []
+        return self.launch(logits, states).tokens()
+
+    @staticmethod
+    def needs_history(state: SamplerState) -> bool:
+        """The draw depends on the request's earlier tokens (repetition penalty)."""
+        return state.params.temp > 0.0 and state.params.repeat_penalty > 1.0
+
+    def _upload(self, array: np.ndarray) -> torch.Tensor:
+        """To the device through pinned memory, without making the host wait for the stream."""
+        return torch.from_numpy(array).pin_memory().to(self.device, non_blocking=True)
+
+    def launch(self, logits: torch.Tensor, states: Sequence[SamplerState]) -> PendingSample:
+        """Starts the draw and returns without waiting for it."""
         R = logits.shape[0]
         if R != len(states):
             raise ValueError(f"{R} logits rows for {len(states)} requests")
-        if R == 0:
-            return []
         out = torch.empty(R, dtype=torch.int32, device=self.device)
         stochastic = [s.params.temp > 0.0 for s in states]
         if not any(stochastic):
@@ -43,7 +77,7 @@ class Sampler:
                 if stochastic[r]:
                     f32[3, r] = s.rng.uniform()
                     f32[4, r] = p.repeat_penalty
-            dev = torch.from_numpy(f32).to(self.device)
+            dev = self._upload(f32)
             penalised = [r for r, s in enumerate(states)
                          if stochastic[r] and s.params.repeat_penalty > 1.0 and s.count > 0]
             if penalised:
@@ -53,11 +87,7 @@ class Sampler:
                 for r in penalised:
                     recent[r, :states[r].count] = states[r].recent[:states[r].count]
                     counts[r] = states[r].count
-                ops.repeat_penalty(logits, torch.from_numpy(recent).to(self.device),
-                                   torch.from_numpy(counts).to(self.device), dev[4].contiguous())
-            ops.sample(logits, out, temps=dev[0].contiguous(), top_ks=torch.from_numpy(top_k).to(self.device),
+                ops.repeat_penalty(logits, self._upload(recent), self._upload(counts), dev[4].contiguous())
+            ops.sample(logits, out, temps=dev[0].contiguous(), top_ks=self._upload(top_k),
                        top_ps=dev[1].contiguous(), min_ps=dev[2].contiguous(), uniforms=dev[3].contiguous())
-        tokens = out.cpu().tolist()
-        for s, t in zip(states, tokens):
-            s.accept(t)
-        return tokens
+        return PendingSample(out, states)
