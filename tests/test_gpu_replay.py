@@ -183,3 +183,42 @@ def test_recorded_decode_steps_equal_eager_steps(gpu, dtype):
     full = util.plain_logits(name, reqs["y"][:fed["y"]], stored_for(dtype))
     mask = ~torch.isnan(got["y"][:, 0])
     util.assert_close(dtype, got["y"][mask], full[mask], "y")
+
+
+def test_layers_of_full_size_bfloat16_against_float32(gpu):
+    """Layers with the sizes of a 1.2B model (hidden 2048, 32 query and 8 kv heads of 64, feed-forward
+    8192, vocabulary 65536; two conv layers and an attention layer): the bfloat16 kernels chosen at
+    these sizes (large matrix tiles, portions of several query blocks, single tokens over several
+    key partitions) against the float32 path, which the tiny configurations pin to the plain
+    implementation.  Both engines hold the same weights (made in bfloat16)."""
+    from tuff_amd.engine.batch import StepEntry
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.models.registry import config_from_dict
+    cfg = config_from_dict(dict(
+        architectures=["Lfm2ForCausalLM"], num_hidden_layers=3, layer_types=["conv", "conv", "full_attention"],
+        hidden_size=2048, num_attention_heads=32, num_key_value_heads=8, block_ff_dim=12288,
+        block_auto_adjust_ff_dim=True, block_multiple_of=256, block_ffn_dim_multiplier=1.0, vocab_size=65536,
+        rope_theta=1000000.0, conv_L_cache=3, norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=8192))
+    assert cfg.ffn_dim == 8192
+    tokens = util.rand_tokens(700, cfg.vocab_size, 5)
+    other = util.rand_tokens(90, cfg.vocab_size, 6)
+    outs = {}
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine.from_config(cfg, 3, dtype=dtype, page_size=16, num_pages=64, max_requests=2)
+        got = []
+        eng.begin("a")
+        eng.begin("b")
+        got.append(eng.step([StepEntry("a", tokens[:600], [0, 299, 599])]))          # one large portion
+        got.append(eng.step([StepEntry("a", tokens[600:690], [89]), StepEntry("b", other[:80], [79])]))
+        for i in range(690, 700):                                                     # single tokens, two requests
+            got.append(eng.step([StepEntry("a", [tokens[i]], [0]), StepEntry("b", [other[i - 610]], [0])]))
+        outs[dtype] = torch.cat([g.float().cpu() for g in got])
+        eng.end("a")
+        eng.end("b")
+        del eng
+        torch.cuda.empty_cache()
+    util.assert_close_bf16(outs["bfloat16"], outs["float32"], "full-size layers")
+    # and the first choice agrees wherever float32 is not close to a tie
+    top = torch.topk(outs["float32"], 2, dim=-1).values
+    clear = (top[:, 0] - top[:, 1]) > 0.05 * float(outs["float32"].std())
+    assert (outs["bfloat16"].argmax(-1) == outs["float32"].argmax(-1))[clear].all()
