@@ -130,6 +130,27 @@ __device__ Cut descend(const RowView& row, Cut cut, u64 target, Shared& sh, u64*
     return e;
 }
 
+// A thread's part of the search for the largest value of a row and its first index: pieces of four
+// values, several loads under way.  The thread sees its indices in ascending order, so a strict
+// comparison keeps the first of equal values.
+template <int NT>
+__device__ __forceinline__ void scan_max(const float* __restrict__ l, int V, int tid, float& best, int& best_i) {
+    const bool vec = (V % 4 == 0) && ((reinterpret_cast<uintptr_t>(l) & 15) == 0);
+    if (vec) {
+        const f32x4* l4 = (const f32x4*)l;
+        const int n4 = V / 4;
+#pragma unroll 4
+        for (int i = tid; i < n4; i += NT) {
+            const f32x4 v = l4[i];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (v[e] > best) { best = v[e]; best_i = i * 4 + e; }
+        }
+    } else {
+        for (int i = tid; i < V; i += NT) { const float v = l[i]; if (v > best) { best = v; best_i = i; } }
+    }
+}
+
 __global__ __launch_bounds__(SNT) void sample_kernel(const float* __restrict__ logits, const float* __restrict__ temps,
                                                      const int* __restrict__ top_ks, const float* __restrict__ top_ps,
                                                      const float* __restrict__ min_ps, const float* __restrict__ uniforms,
@@ -140,7 +161,7 @@ __global__ __launch_bounds__(SNT) void sample_kernel(const float* __restrict__ l
 
     // maximum and its first index
     float best = -INFINITY; int best_i = 0x7fffffff;
-    for (int i = tid; i < V; i += SNT) { const float v = l[i]; if (v > best) { best = v; best_i = i; } }
+    scan_max<SNT>(l, V, tid, best, best_i);
 #pragma unroll
     for (int m = WAVE / 2; m > 0; m >>= 1) {
         const float ov = __shfl_xor(best, m, WAVE); const int oi = __shfl_xor(best_i, m, WAVE);
@@ -228,7 +249,7 @@ __global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ l
     const int r = blockIdx.x, tid = threadIdx.x;
     const float* l = logits + (long long)r * V;
     float best = -INFINITY; int best_i = 0x7fffffff;
-    for (int i = tid; i < V; i += 256) { const float v = l[i]; if (v > best) { best = v; best_i = i; } }
+    scan_max<256>(l, V, tid, best, best_i);
 #pragma unroll
     for (int m = WAVE / 2; m > 0; m >>= 1) {
         const float ov = __shfl_xor(best, m, WAVE); const int oi = __shfl_xor(best_i, m, WAVE);
