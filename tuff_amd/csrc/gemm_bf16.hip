@@ -258,7 +258,9 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
                                                                        const float* __restrict__ ss_in, int n_ss,
                                                                        const float* __restrict__ emit_nw,
                                                                        bf16_t* __restrict__ emit_xw, float* __restrict__ emit_ss) {
-    __shared__ float red[NW][WAVE][4];
+    constexpr int TN = COLS > 16 ? COLS / 16 : 1;                        // MFMA tiles side by side: they share the rows of X
+    static_assert(!EMIT || TN == 1, "the emitting epilogue works on one tile");
+    __shared__ float red[TN][NW][WAVE][4];
     __shared__ float ssq[16][16];                                        // [wave or part][row]
     extern __shared__ __attribute__((aligned(16))) float nw_lds[];       // NORM_INSIDE: the norm weight, K floats
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
@@ -272,24 +274,32 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
 
     // What the epilogue adds to is read now, not after the last product: a load at the end would
     // cost one more trip to memory.
-    float y_old = 0.f, emit_w = 0.f;
-    if (MODE == OUT_F32_ACCUM && tid < 256) {
-        const long long row = (tid / 64) * 4 + tid % 4, col = n0 + (tid / 4) % 16;
-        if (row < M && col < w_rows) {
-            y_old = ((const float*)Y)[row * N + col];
-            if (EMIT) emit_w = emit_nw[col];
+    float y_old[TN], emit_w = 0.f;
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+        y_old[tn] = 0.f;
+        if (MODE == OUT_F32_ACCUM && tid < 256) {
+            const long long row = (tid / 64) * 4 + tid % 4, col = n0 + tn * 16 + (tid / 4) % 16;
+            if (row < M && col < w_rows) {
+                y_old[tn] = ((const float*)Y)[row * N + col];
+                if (EMIT) emit_w = emit_nw[col];
+            }
         }
     }
 
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    f32x4 acc[TN];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) acc[tn] = f32x4{0.f, 0.f, 0.f, 0.f};
     float ss = 0.f;
-    struct Operands { bf16x8 a[4]; bf16x8 b[4]; f32x4 x[NORM == NORM_INSIDE ? 4 : 1][2]; };
+    struct Operands { bf16x8 a[4]; bf16x8 b[TN][4]; f32x4 x[NORM == NORM_INSIDE ? 4 : 1][2]; };
     Operands o0, o1;
     auto load = [&](int c, Operands& o) {
         // instruction j of the wave reads bytes 64 j .. 64 j + 63 of the chunk of each of its 16 rows
         const int kb = c * SK_CHUNK + g * 8;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) o.b[j] = load8(W, n0 + r16, w_rows, kb + j * 32, K);
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o.b[tn][j] = load8(W, n0 + tn * 16 + r16, w_rows, kb + j * 32, K);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int k = kb + j * 32;
@@ -320,7 +330,9 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
             }
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc = mfma16(o.a[j], o.b[j], acc);
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[tn] = mfma16(o.a[j], o.b[tn][j], acc[tn]);
     };
     // Workgroups start at different chunks (a rotation by the tile index), so that at any moment
     // the chip reads from all columns of W and not from one.  The order of a tile's additions
@@ -354,7 +366,9 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
         }
     }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) red[wave][lane][e] = acc[e];
+    for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) red[tn][wave][lane][e] = acc[tn][e];
     if (NORM == NORM_SCALED && tid < 256) {
         float t = ss_rest;
 #pragma unroll
@@ -368,39 +382,45 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
     }
     __syncthreads();
     if (tid < 256) {
-        // thread -> (lane l, element e) of the 16x16 tile; the wave partials in wave order
+        // thread -> (lane l, element e) of each 16x16 tile; the wave partials in wave order
         const int e = tid % 4, l = tid / 4;
-        float v = red[0][l][e];
-#pragma unroll
-        for (int w = 1; w < NW; ++w) v += red[w][l][e];
-        const long long col = n0 + (l % 16);
-        const long long row = col < w_rows ? (l / 16) * 4 + e : 16;     // columns beyond the tile: no row
-        if (NORM != NORM_NONE && row < 16) {
+        float scale = 1.f;
+        if (NORM != NORM_NONE) {
             constexpr int PARTS = NORM == NORM_INSIDE ? NW : 16;
+            const int row = (l / 16) * 4 + e;
             float total = ssq[0][row];
 #pragma unroll
             for (int w = 1; w < PARTS; ++w) total += ssq[w][row];
-            v *= 1.0f / sqrtf(total / (float)K + eps);
+            scale = 1.0f / sqrtf(total / (float)K + eps);
         }
-        if (EMIT) {
-            // y += v; the new y also as the next norm's operand, and its square into the row's tile sum
-            float y = 0.f;
-            if (row < M && col < N) {
-                y = y_old + v;
-                ((float*)Y)[row * N + col] = y;
-                emit_xw[row * N + col] = (bf16_t)(y * emit_w);
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+            float v = red[tn][0][l][e];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) v += red[tn][w][l][e];
+            const long long col = n0 + tn * 16 + (l % 16);
+            const long long row = col < w_rows ? (l / 16) * 4 + e : 16;     // columns beyond the tile: no row
+            if (NORM != NORM_NONE) v *= scale;
+            if (EMIT) {
+                // y += v; the new y also as the next norm's operand, and its square into the row's tile sum
+                float y = 0.f;
+                if (row < M && col < N) {
+                    y = y_old[tn] + v;
+                    ((float*)Y)[row * N + col] = y;
+                    emit_xw[row * N + col] = (bf16_t)(y * emit_w);
+                }
+                float sq = y * y;                       // tid = (16 q + c) * 4 + e: the 16 columns c are tid bits 2..5
+                sq += __shfl_xor(sq, 4, WAVE);
+                sq += __shfl_xor(sq, 8, WAVE);
+                sq += __shfl_xor(sq, 16, WAVE);
+                sq += __shfl_xor(sq, 32, WAVE);
+                if ((l % 16) == 0 && row < 16) emit_ss[(long long)blockIdx.x * 16 + row] = sq;
+            } else if (MODE == OUT_F32_ACCUM) {
+                if (row < M && col < N) ((float*)Y)[row * N + col] = y_old[tn] + v;
+            } else {
+                const float partner = (MODE == OUT_SWIGLU) ? __shfl_xor(v, 4, WAVE) : 0.f;   // thread tid ^ 4 holds column col ^ 1
+                store_elem<MODE>(Y, row, col, min(M, 16), N, v, partner);
             }
-            float sq = y * y;                       // tid = (16 q + c) * 4 + e: the 16 columns c are tid bits 2..5
-            sq += __shfl_xor(sq, 4, WAVE);
-            sq += __shfl_xor(sq, 8, WAVE);
-            sq += __shfl_xor(sq, 16, WAVE);
-            sq += __shfl_xor(sq, 32, WAVE);
-            if ((l % 16) == 0) emit_ss[(long long)blockIdx.x * 16 + row] = sq;
-        } else if (MODE == OUT_F32_ACCUM) {
-            if (row < M && col < N) ((float*)Y)[row * N + col] = y_old + v;
-        } else {
-            const float partner = (MODE == OUT_SWIGLU) ? __shfl_xor(v, 4, WAVE) : 0.f;   // thread tid ^ 4 holds column col ^ 1
-            store_elem<MODE>(Y, row, col, min(M, 16), N, v, partner);
         }
     }
 }
@@ -535,9 +555,15 @@ SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16) {
     p.slices = 1; p.chunks_per_slice = nchunks; p.ws_floats = 0; p.waves = 4;
     p.cols = 16;
     if (M <= 16) {
-        // tiles of 8 columns where 16 would leave CUs without a workgroup (half of each MFMA idles,
-        // which costs nothing here: these products wait for memory)
-        if (ceil_div(N, 16) <= 128) p.cols = 8;
+        // Narrow outputs: tiles of 8 columns, where 16 would leave CUs without a workgroup (half of
+        // each MFMA idles, which costs nothing here: these products wait for memory).  Wide outputs:
+        // 32 or 64 columns, whose MFMA tiles share the rows of X: with 16 columns the rows of X
+        // (from the L2, again for every workgroup) are up to as many bytes again as the weights.
+        const int tiles16 = ceil_div(N, 16);
+        if (tiles16 <= 128) p.cols = 8;
+        else if (tiles16 >= 4096) p.cols = 64;
+        else if (tiles16 >= 384) p.cols = 32;
+        if (max_waves < 16 && p.cols > 16) p.cols = 16;                 // the norm inside keeps float32 rows in registers
         p.tiles = ceil_div(N, p.cols);
         // enough waves in flight to cover the latency of HBM, at least one chunk a wave
         while (p.waves < max_waves && p.tiles * p.waves < 3072 && nchunks >= 2 * p.waves) p.waves *= 2;
@@ -568,7 +594,12 @@ int launch_skinny16(const void* X, const bf16_t* W, void* Y, int M, int N, int K
 #define GO(NW, COLS) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<NW, MODE, NORM, EMIT, COLS>), grid, dim3(NW * WAVE), lds, stream, \
                                         X, W, Y, M, N, K, x.norm_w, x.eps, x.rows, x.ss_in, x.n_ss, x.emit_nw, x.emit_xw, x.emit_ss)
     if (p.cols == 16) { if (p.waves == 4) GO(4, 16); else if (p.waves == 8) GO(8, 16); else GO(16, 16); }
-    else { if (p.waves == 4) GO(4, 8); else if (p.waves == 8) GO(8, 8); else GO(16, 8); }
+    else if (p.cols == 8) { if (p.waves == 4) GO(4, 8); else if (p.waves == 8) GO(8, 8); else GO(16, 8); }
+    else if constexpr (!EMIT && NORM != NORM_INSIDE) {
+        if (p.cols == 32) { if (p.waves == 4) GO(4, 32); else if (p.waves == 8) GO(8, 32); else GO(16, 32); }
+        else if (p.cols == 64) { if (p.waves == 4) GO(4, 64); else if (p.waves == 8) GO(8, 64); else GO(16, 64); }
+        else return -3;
+    } else return -3;
 #undef GO
     return launch_status();
 }
