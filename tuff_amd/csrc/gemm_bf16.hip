@@ -562,7 +562,7 @@ SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16) {
         const int tiles16 = ceil_div(N, 16);
         if (tiles16 <= 128) p.cols = 8;
         else if (tiles16 >= 4096) p.cols = 64;
-        else if (tiles16 >= 384) p.cols = 32;
+        else if (tiles16 >= 512) p.cols = 32;
         if (max_waves < 16 && p.cols > 16) p.cols = 16;                 // the norm inside keeps float32 rows in registers
         p.tiles = ceil_div(N, p.cols);
         // enough waves in flight to cover the latency of HBM, at least one chunk a wave
