@@ -466,6 +466,29 @@ def test_attention_prefill(gpu, H, Hkv, hd, ps, window):
     assert torch.equal(out.cpu().double().reshape(80, H, hd), got[sel]), "the result depends on where the portion starts"
 
 
+def test_attention_long_context(gpu):
+    """Past 64 partitions of 256 keys (the general merge) and past many batches of page numbers:
+    single tokens and a portion deep in requests of about 20,000 tokens, one with a window."""
+    from tuff_amd.csrc import ops
+    H, Hkv, hd, ps = 4, 2, 64, 16
+    for window in (0, 5000):
+        reqs = [(19999, 1), (17000, 200), (16390, 1)]
+        case = _mixed_step_case(gpu, reqs, H, Hkv, hd, ps)
+        T = case["q"].shape[0]
+        common = dict(block_table=case["table"], req_info=case["req_info"], H=H, Hkv=Hkv, hd=hd, page_size=ps,
+                      max_ctx_len=case["max_ctx_len"], window=window)
+        out = torch.full((T, H * hd), float("nan"), dtype=torch.bfloat16, device=gpu)
+        blocks = torch.from_numpy(ops.query_blocks(case["q_len"], H // Hkv, 1)).to(gpu)
+        ops.attention_mfma(case["q"].to(gpu), case["kc"], case["vc"], out, blocks=blocks, nb=1,
+                           positions=case["positions"], **common)
+        _check_step(case, reqs, out.cpu().double().reshape(T, H, hd), H, hd, window, ("mfma", window))
+        out2 = torch.full((T, H * hd), float("nan"), dtype=torch.bfloat16, device=gpu)
+        cols = ops.attention_prefill_block_columns(hd)
+        blocks = torch.from_numpy(ops.query_blocks(case["q_len"], H // Hkv, cols // 16)).to(gpu)
+        ops.attention_prefill(case["q"].to(gpu), case["kc"], case["vc"], out2, blocks=blocks, **common)
+        _check_step(case, reqs, out2.cpu().double().reshape(T, H, hd), H, hd, window, ("prefill", window))
+
+
 @pytest.mark.parametrize("kernel", ["mfma", "prefill"])
 def test_attention_matrix_kernels_find_a_far_key_and_the_window_edge(gpu, kernel):
     """One key among a thousand matches the query: the output is that key's value row, wherever
