@@ -301,3 +301,106 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(gpu):
     finally:
         MIXERS.unregister("leaky_sum")
         registry.unregister_architecture("ToyLeakyForCausalLM")
+
+
+# ------------------------------------------------------- run order and cache groups as data
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_layer_run_twice_a_shared_cache_and_a_window_group(gpu, dtype):
+    """A toy architecture whose run order names block 0 twice (two cache entries of its own) and
+    lets block 2 read the keys and values block 1 writes; block 0 has a window of 24, so its
+    entries form a page group of their own whose pages are given back as the window moves on.
+    Whole, in portions and mixed with few pages, against a plain loop."""
+    from tuff_amd.config.base import ModelConfig
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.models import registry
+    from tuff_amd.models.decoder import DecoderModel, LayerRun
+    from tuff_amd.parts.attention import AttentionMixer
+    from tuff_amd.parts.base import WeightDecl
+    from tuff_amd.parts.block import PreNormBlock
+    from tuff_amd.parts.ffn import SwiGLU
+    from tuff_amd.parts.norm import RMSNorm
+    from tuff_amd.parts.rope import Rotary
+    from tuff_amd.weights.random_init import random_weights
+    d, H, Hkv, hd, ffn, V, W, theta, eps = 64, 4, 2, 16, 96, 211, 24, 1e4, 1e-5
+
+    @dataclasses.dataclass
+    class OrderConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyOrderForCausalLM"
+        vocab_size: int
+
+    def names(i):
+        return {k: f"l{i}.{k}" for k in ("q", "k", "v", "o", "q_norm", "k_norm")}
+
+    def build(cfg):
+        def block(i, window):
+            return PreNormBlock(RMSNorm(d, eps, f"l{i}.n1"),
+                                AttentionMixer(d, H, Hkv, hd, names=names(i), qk_norm_eps=eps, position=Rotary(hd, theta),
+                                               window=window),
+                                RMSNorm(d, eps, f"l{i}.n2"),
+                                SwiGLU(d, ffn, names={"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"}))
+        return DecoderModel(vocab_size=cfg.vocab_size, hidden_size=d, embedding=WeightDecl("emb", (cfg.vocab_size, d)),
+                            blocks=[block(0, W), block(1, None), block(2, None)], final_norm=RMSNorm(d, eps, "fn"),
+                            schedule=[LayerRun(0), LayerRun(1, cache=7), LayerRun(0), LayerRun(2, cache=7, writes=False)])
+
+    registry.register_architecture("ToyOrderForCausalLM", OrderConfig, build)
+    try:
+        cfg = registry.config_from_dict({"architectures": ["ToyOrderForCausalLM"], "vocab_size": V})
+        model = registry.build_model(cfg)
+        stored = torch.float32 if dtype == "float32" else torch.bfloat16
+        weights = random_weights(model.weight_decls(), 4, stored, "cpu", stored_dtype=stored)
+        reqs = {f"r{i}": util.rand_tokens(n, V, 30 + i) for i, n in enumerate([90, 61, 75, 40, 52])}
+        plan = util.plan_mixed(reqs, seed=3, decode_tail=20)
+        eng = Engine(model, {k: v.to(gpu) for k, v in weights.items()}, dtype=dtype, page_size=16,
+                     max_tokens=util.live_tokens_peak(plan))
+        assert sorted(w is None for w in eng.layout.group_windows) == [False, True]      # two page groups
+        whole = util.run_plan(eng, util.plan_whole(reqs))
+        allocated = [g.pool.allocations for g in eng.manager.groups]
+        mixed = util.run_plan(eng, plan)
+        chunks = util.run_plan(eng, util.plan_chunks(reqs))
+        eng.manager.check()
+        assert not eng.manager.live()
+        # the window group handed its pages out again and again
+        win = [i for i, g in enumerate(eng.manager.groups) if g.window is not None][0]
+        assert eng.manager.groups[win].pool.allocations - allocated[win] > eng.manager.groups[win].pool.num_pages
+
+        # ---- the plain loop
+        w = {k: v.double() for k, v in weights.items()}
+
+        def keys_values(i, h):
+            T = h.shape[0]
+            pos = torch.arange(T)
+            k = plain.rope_neox(plain.rms_norm((h @ w[f"l{i}.k"].T).reshape(T, Hkv, hd), w[f"l{i}.k_norm"], eps), pos, theta)
+            return k, (h @ w[f"l{i}.v"].T).reshape(T, Hkv, hd)
+
+        def attend(i, h, k, v, window):
+            T = h.shape[0]
+            pos = torch.arange(T)
+            q = plain.rope_neox(plain.rms_norm((h @ w[f"l{i}.q"].T).reshape(T, H, hd), w[f"l{i}.q_norm"], eps), pos, theta)
+            k, v = k.repeat_interleave(H // Hkv, 1), v.repeat_interleave(H // Hkv, 1)
+            s = torch.einsum("thd,shd->hts", q, k) / math.sqrt(hd)
+            a, b = torch.arange(T)[:, None], torch.arange(T)[None, :]
+            seen = (b <= a) if window is None else ((b <= a) & (b > a - window))
+            s = s.masked_fill(~seen, float("-inf"))
+            return torch.einsum("hts,shd->thd", torch.softmax(s, -1), v).reshape(T, H * hd) @ w[f"l{i}.o"].T
+
+        def ffn_of(i, x):
+            return plain.swiglu(plain.rms_norm(x, w[f"l{i}.n2"], eps), w[f"l{i}.g"], w[f"l{i}.u"], w[f"l{i}.d"])
+
+        for rid, toks in reqs.items():
+            x = w["emb"][toks]
+            shared = None
+            for i, reads in ((0, False), (1, False), (0, False), (2, True)):
+                h = plain.rms_norm(x, w[f"l{i}.n1"], eps)
+                if reads:
+                    k, v = shared                                # block 1's keys and values, block 2's queries
+                else:
+                    k, v = keys_values(i, h)
+                    if i == 1:
+                        shared = (k, v)
+                x = x + attend(i, h, k, v, W if i == 0 else None)
+                x = x + ffn_of(i, x)
+            want = plain.rms_norm(x, w["fn"], eps) @ w["emb"].T
+            for got in (whole, mixed, chunks):
+                util.assert_close(dtype, got[rid], want, rid)
+    finally:
+        registry.unregister_architecture("ToyOrderForCausalLM")
