@@ -404,3 +404,97 @@ def test_a_layer_run_twice_a_shared_cache_and_a_window_group(gpu, dtype):
                 util.assert_close(dtype, got[rid], want, rid)
     finally:
         registry.unregister_architecture("ToyOrderForCausalLM")
+
+
+# --------------------------------------------------------------- a toy routed feed-forward
+def test_toy_feed_forward_with_routing_beside_the_frameworks_parts(gpu):
+    """A feed-forward defined here: a float32 router picks one of three small SwiGLU experts per
+    token (the experts are the framework's own SwiGLU parts; the routing is a few torch calls).
+    Layer 0 uses it, layer 1 the dense SwiGLU: feed-forwards differ layer by layer.  Because the
+    choice is per token, cutting and batching change nothing."""
+    from tuff_amd.config.base import ModelConfig
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.models import registry
+    from tuff_amd.models.decoder import DecoderModel
+    from tuff_amd.parts.base import FEED_FORWARDS, FeedForward, WeightDecl
+    from tuff_amd.parts.block import PreNormBlock
+    from tuff_amd.parts.ffn import SwiGLU
+    from tuff_amd.parts.norm import RMSNorm
+    from tuff_amd.parts.shortconv import ShortConvMixer
+    from tuff_amd.weights.random_init import random_weights
+    d, F, E, V, K, eps = 48, 40, 3, 131, 3, 1e-5
+
+    class RoutedSwiGLU(FeedForward):
+        def __init__(self, d, F, n_experts, prefix):
+            self.router = f"{prefix}.router"
+            self.experts = [SwiGLU(d, F, names={k: f"{prefix}.e{e}.{k}" for k in ("gate", "up", "down")})
+                            for e in range(n_experts)]
+            self.d, self.E = d, n_experts
+
+        def weight_decls(self):
+            return [WeightDecl(self.router, (self.E, self.d))] + [x for e in self.experts for x in e.weight_decls()]
+
+        def kernel_modules(self):
+            return [m for e in self.experts for m in e.kernel_modules()]
+
+        def bind(self, weights, rt):
+            self.rt, self.w_router = rt, weights[self.router].float()
+            for e in self.experts:
+                e.bind(weights, rt)
+
+        def forward(self, h, ctx, residual):
+            choice = (h.float() @ self.w_router.T).argmax(-1)                 # router logits in float32
+            for e, expert in enumerate(self.experts):
+                rows = torch.nonzero(choice == e).flatten()
+                if rows.numel():
+                    part = torch.zeros(rows.numel(), self.d, dtype=torch.float32, device=h.device)
+                    expert.forward(h[rows].contiguous(), ctx, part)
+                    residual[rows] += part
+
+    @dataclasses.dataclass
+    class RoutedConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyRoutedForCausalLM"
+        vocab_size: int
+
+    def build(cfg):
+        def mixer(i):
+            return ShortConvMixer(d, K, names={"in_proj": f"l{i}.in", "conv": f"l{i}.conv", "out_proj": f"l{i}.out"})
+        ffs = [FEED_FORWARDS.get("toy_routed")(d, F, E, "l0.moe"),
+               SwiGLU(d, 2 * F, names={"gate": "l1.g", "up": "l1.u", "down": "l1.d"})]
+        blocks = [PreNormBlock(RMSNorm(d, eps, f"l{i}.n1"), mixer(i), RMSNorm(d, eps, f"l{i}.n2"), ffs[i]) for i in range(2)]
+        return DecoderModel(vocab_size=cfg.vocab_size, hidden_size=d, embedding=WeightDecl("emb", (cfg.vocab_size, d)),
+                            blocks=blocks, final_norm=RMSNorm(d, eps, "fn"))
+
+    FEED_FORWARDS.register("toy_routed", RoutedSwiGLU)
+    registry.register_architecture("ToyRoutedForCausalLM", RoutedConfig, build)
+    try:
+        cfg = registry.config_from_dict({"architectures": ["ToyRoutedForCausalLM"], "vocab_size": V})
+        model = registry.build_model(cfg)
+        weights = random_weights(model.weight_decls(), 6, torch.float32, "cpu", stored_dtype=torch.float32)
+        weights["l0.moe.router"] = weights["l0.moe.router"] * 40          # clear choices: no ties to argue about
+        eng = Engine(model, {k: v.to(gpu) for k, v in weights.items()}, dtype="float32", max_tokens=256)
+        reqs = {"a": util.rand_tokens(33, V, 1), "b": util.rand_tokens(20, V, 2), "c": util.rand_tokens(9, V, 3)}
+        whole = util.run_plan(eng, util.plan_whole(reqs))
+        mixed = util.run_plan(eng, util.plan_mixed(reqs, seed=2, decode_tail=5))
+        w = {k: v.double() for k, v in weights.items()}
+        used = set()
+        for rid, toks in reqs.items():
+            x = w["emb"][toks]
+            for i in range(2):
+                x = x + plain.short_conv(plain.rms_norm(x, w[f"l{i}.n1"], eps), w[f"l{i}.in"], w[f"l{i}.conv"], w[f"l{i}.out"])
+                h = plain.rms_norm(x, w[f"l{i}.n2"], eps)
+                if i == 0:
+                    choice = (h @ w["l0.moe.router"].T).argmax(-1)
+                    used |= set(choice.tolist())
+                    y = torch.stack([plain.swiglu(h[t:t + 1], w[f"l0.moe.e{int(c)}.gate"], w[f"l0.moe.e{int(c)}.up"],
+                                                  w[f"l0.moe.e{int(c)}.down"])[0] for t, c in enumerate(choice)])
+                else:
+                    y = plain.swiglu(h, w["l1.g"], w["l1.u"], w["l1.d"])
+                x = x + y
+            want = plain.rms_norm(x, w["fn"], eps) @ w["emb"].T
+            util.assert_close_f32(whole[rid], want, rid)
+            util.assert_close_f32(mixed[rid], want, rid)
+        assert len(used) == E                                             # every expert was chosen by some token
+    finally:
+        registry.unregister_architecture("ToyRoutedForCausalLM")
+        FEED_FORWARDS.unregister("toy_routed")
