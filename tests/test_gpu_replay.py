@@ -48,6 +48,14 @@ def test_whole(gpu, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_feed_forward_width_that_is_no_multiple_of_8(gpu, dtype):
+    reqs = requests_for("D")
+    check_plan("D", dtype, util.plan_whole(reqs), reqs)
+    plan = util.plan_mixed(reqs, seed=4)
+    check_plan("D", dtype, plan, reqs, max_tokens=util.live_tokens_peak(plan))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_head_then_single_tokens(gpu, name, dtype):
     reqs = requests_for(name)

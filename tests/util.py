@@ -34,7 +34,13 @@ TINY_C = dict(
     hidden_size=240, num_attention_heads=3, num_key_value_heads=3,
     block_ff_dim=328, block_auto_adjust_ff_dim=False, vocab_size=777, rope_theta=500000.0,
     conv_L_cache=2, norm_eps=3e-6, tie_word_embeddings=True, max_position_embeddings=1024)
-CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 5)}
+# a feed-forward width that is no multiple of 8 (the bfloat16 kernels read 16 bytes at a time)
+TINY_D = dict(
+    architectures=["Lfm2ForCausalLM"], num_hidden_layers=2, layer_types=["full_attention", "conv"],
+    hidden_size=32, num_attention_heads=2, num_key_value_heads=1,
+    block_ff_dim=100, block_auto_adjust_ff_dim=False, vocab_size=333, rope_theta=10000.0,
+    conv_L_cache=3, norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=512)
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 5), "D": (TINY_D, 9)}
 
 _TMP = tempfile.TemporaryDirectory(prefix="tuff_amd_tests_")
 

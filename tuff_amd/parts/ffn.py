@@ -5,6 +5,8 @@ interleaved and the activation is the product's epilogue.
 """
 from __future__ import annotations
 
+import torch
+
 from ..csrc import ops
 from .base import FEED_FORWARDS, FeedForward, Runtime
 from .linear import Linear
@@ -20,19 +22,37 @@ class SwiGLU(FeedForward):
                  aliases: dict[str, tuple] | None = None):
         """names: checkpoint names of 'gate' [F, d], 'up' [F, d], 'down' [d, F]."""
         self.d, self.F = int(hidden_size), int(ffn_dim)
-        al = aliases or {}
-        self.gate_up = Linear([names["gate"], names["up"]], self.d, [self.F, self.F],
+        self._names, self._al = dict(names), aliases or {}
+        self._make(self.F)
+        self._decls = self.gate_up.weight_decls() + self.down.weight_decls()
+
+    def _make(self, width: int) -> None:
+        names, al = self._names, self._al
+        self.gate_up = Linear([names["gate"], names["up"]], self.d, [width, width],
                               aliases=[al.get("gate", ()), al.get("up", ())], swiglu_pair=True)
-        self.down = Linear(names["down"], self.F, self.d, aliases=[al.get("down", ())])
+        self.down = Linear(names["down"], width, self.d, aliases=[al.get("down", ())])
+        self.width = width
 
     def weight_decls(self):
-        return self.gate_up.weight_decls() + self.down.weight_decls()
+        return self._decls
 
     def kernel_modules(self):
         return ["elementwise"]
 
     def bind(self, weights, rt: Runtime):
         self.rt = rt
+        names = self._names
+        g, u, dn = (weights[names[k]] for k in ("gate", "up", "down"))
+        if self.F % 8 and all(t.dtype == torch.bfloat16 for t in (g, u, dn)):
+            # The bfloat16 matrix kernels read 16 bytes at a time along the inner size.  A width that is
+            # no multiple of 8 is filled up with zero rows of gate and up (silu(0) * 0 = 0, exactly) and
+            # zero columns of down: the same function.
+            pad = -self.F % 8
+            weights = dict(weights)
+            weights[names["gate"]] = torch.cat([g, g.new_zeros(pad, self.d)])
+            weights[names["up"]] = torch.cat([u, u.new_zeros(pad, self.d)])
+            weights[names["down"]] = torch.cat([dn, dn.new_zeros(self.d, pad)], dim=1).contiguous()
+            self._make(self.F + pad)
         self.gate_up.bind(weights, rt)
         self.down.bind(weights, rt)
 
@@ -41,6 +61,6 @@ class SwiGLU(FeedForward):
             act = self.gate_up.forward(h, swiglu=True)          # silu(gate) * up in the product's epilogue
         else:
             gu = self.gate_up.forward(h)
-            act = self.rt.empty(h.shape[0], self.F, dtype=gu.dtype)
+            act = self.rt.empty(h.shape[0], self.width, dtype=gu.dtype)
             ops.swiglu(gu, act)
         self.down.forward(act, accumulate_into=residual)
