@@ -213,3 +213,33 @@ def test_command_line(gpu, tmp_path):
     assert _tuff("--model", folder, "--prompt-ids", ids, "-n", "5000").returncode == 2
     assert _tuff("--model", str(tmp_path), "--prompt-ids", ids).returncode == 1
     assert _tuff("--model", folder, "--inspect").returncode == 0
+
+
+def test_command_line_jobs(gpu, tmp_path):
+    """--jobs: the model is loaded once; every line is a run of its own with its own output files,
+    exit code and environment (src/main.c:1921-2093)."""
+    folder = util.model_folder("A", "float32")
+    V = util.TINY_A["vocab_size"]
+    a, b = util.rand_tokens(9, V, 3), util.rand_tokens(14, V, 4)
+    ids = lambda p: ",".join(map(str, p))
+    alone = [_tuff("--model", folder, "--dtype", "fp32", "--prompt-ids", ids(p), "--dump-tokens", "-n", "10").stdout
+             for p in (a, b)]
+    jobs = tmp_path / "jobs.txt"
+    o = [tmp_path / f"o{i}" for i in range(4)]
+    jobs.write_text(
+        "# two runs, a usage error, and a run with an assignment in front\n"
+        f"--prompt-ids {ids(a)} --dump-tokens -n 10 --out {o[0]} --err {tmp_path / 'e0'} --status {tmp_path / 's0'}\n"
+        "\n"
+        f"--prompt-ids '{' '.join(map(str, b))}' --dump-tokens -n 10 --out {o[1]}\n"
+        f"--dump-tokens -n 10 --out {o[2]} --status {tmp_path / 's2'}\n"
+        f"TUFF_TEST_MARK=1 --prompt-ids {ids(a)} --dump-tokens -n 10 --out {o[3]} --err {tmp_path / 'e3'}\n")
+    p = _tuff("--model", folder, "--dtype", "fp32", "--jobs", str(jobs))
+    assert p.returncode == 2, p.stderr                       # the first code that was not 0
+    assert "4 job(s), 1 failed" in p.stderr
+    said = p.stderr + (tmp_path / "e0").read_text() + (tmp_path / "e3").read_text()
+    assert said.count("model ready") == 1 and said.count("reusing the loaded model") == 2      # job 3 never got that far
+    assert o[0].read_text() == alone[0] and o[1].read_text() == alone[1] and o[3].read_text() == alone[0]
+    assert (tmp_path / "s0").read_text().strip() == "0" and (tmp_path / "s2").read_text().strip() == "2"
+    assert (tmp_path / "e0").read_text().strip().endswith("JOB_EXIT=0")
+    assert "reusing the loaded model" in (tmp_path / "e3").read_text()
+    assert "TUFF_TEST_MARK" not in os.environ

@@ -6,6 +6,7 @@ vocabulary.
     tuff --model DIR --prompt-ids p.txt --dump-tokens -n 32
     tuff --model DIR --prompt-ids p.txt --teacher-force ref.txt --dump-logits out.bin --tf-batch 4
     tuff --random config.json --seed 2 --inspect
+    tuff --model DIR --jobs jobs.txt            (the model is loaded once, every line is a run)
 
 Exit codes as in the reference: 0 ok, 1 mismatch or model error, 2 usage, 3 engine or IO failure.
 """
@@ -60,6 +61,11 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--num-pages", type=int, default=None)
     ap.add_argument("--ignore-eos", action="store_true")
+    ap.add_argument("--jobs", metavar="FILE", help="one job a line: [NAME=value ...] <tuff arguments> [--out F] [--err F] "
+                                                    "[--status F]; the model is loaded once")
+    ap.add_argument("--out", help="in a job: the job's standard output goes to this file")
+    ap.add_argument("--err", help="in a job: the job's standard error goes to this file")
+    ap.add_argument("--status", help="in a job: the job's exit code is written to this file")
     return ap
 
 
@@ -78,6 +84,90 @@ def _inspect(cfg, model, out=sys.stdout) -> None:
 
 
 def main(argv=None) -> int:
+    argv = list(sys.argv[1:] if argv is None else argv)
+    if "--jobs" in argv:
+        return _run_jobs(argv)
+    return _run(argv, {})
+
+
+def _run_jobs(argv: list) -> int:
+    """`--jobs FILE` as in the reference (src/main.c:1921-2093): one process, one model load, many
+    jobs.  A job's command line is this invocation's arguments (without --jobs) followed by the
+    line's; leading NAME=value tokens are its environment (restored afterwards); --out/--err take its
+    output, the last line of its standard error is JOB_EXIT=<code>, --status gets the code.  Blank
+    lines and lines starting with '#' are skipped.  Returns 0 if every job did, else the first
+    job's code that was not 0."""
+    import contextlib
+    import shlex
+    i = argv.index("--jobs")
+    if i + 1 >= len(argv):
+        print("tuff: --jobs needs a file", file=sys.stderr)
+        return 2
+    path, defaults = argv[i + 1], argv[:i] + argv[i + 2:]
+    try:
+        with open(path) as f:
+            lines = f.readlines()
+    except OSError as e:
+        print(f"tuff: cannot open the jobs file: {e}", file=sys.stderr)
+        return 2
+    loaded: dict = {}
+    overall = njob = nfail = 0
+    for line in lines:
+        if not line.strip() or line.lstrip().startswith("#"):
+            continue
+        njob += 1
+        rc, env, job_args = 0, {}, []
+        try:
+            tokens = shlex.split(line)
+        except ValueError as e:
+            print(f"tuff: jobs: line {njob}: {e}", file=sys.stderr)
+            tokens, rc = [], 2
+        while tokens and "=" in tokens[0] and (tokens[0][0].isalpha() or tokens[0][0] == "_") \
+                and tokens[0].split("=", 1)[0].replace("_", "a").isalnum():
+            name, value = tokens.pop(0).split("=", 1)
+            env[name] = value
+        job_args = defaults + tokens
+
+        def last(opt):
+            hits = [k for k in range(len(job_args) - 1) if job_args[k] == opt]
+            return job_args[hits[-1] + 1] if hits else None
+        out_path, err_path, status_path = last("--out"), last("--err"), last("--status")
+        saved = {k: os.environ.get(k) for k in env}
+        os.environ.update(env)
+        with contextlib.ExitStack() as stack:
+            fo = stack.enter_context(open(out_path, "w")) if out_path else None
+            fe = stack.enter_context(open(err_path, "w")) if err_path else None
+            if fo:
+                stack.enter_context(contextlib.redirect_stdout(fo))
+            if fe:
+                stack.enter_context(contextlib.redirect_stderr(fe))
+            if rc == 0:
+                try:
+                    rc = _run(job_args, loaded)
+                except Exception as e:                       # noqa: BLE001 - a job must not take the runner down
+                    print(f"tuff: {type(e).__name__}: {e}", file=sys.stderr)
+                    rc = 3
+            sys.stdout.flush()
+            print(f"JOB_EXIT={rc}", file=sys.stderr)
+            sys.stderr.flush()
+        for k, v in saved.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+        if status_path:
+            with open(status_path, "w") as f:
+                f.write(f"{rc}\n")
+        print(f"tuff: job {njob}: exit {rc}" + (f" err={err_path}" if err_path else ""), file=sys.stderr)
+        if rc != 0:
+            nfail += 1
+            overall = overall or rc
+    print(f"tuff: jobs: {njob} job(s), {nfail} failed", file=sys.stderr)
+    return overall
+
+
+def _run(argv: list, loaded: dict) -> int:
+    """One run.  `loaded` keeps the engine from one run of a job file to the next."""
     ap = build_parser()
     try:
         args = ap.parse_args(argv)
@@ -141,12 +231,22 @@ def main(argv=None) -> int:
         ctx = min(args.ctx, getattr(cfg, "max_position_embeddings", args.ctx))
         pages = args.num_pages or args.max_num_seqs * -(-ctx // args.page_size)
         kw = dict(dtype=args.dtype, page_size=args.page_size, num_pages=pages, max_requests=args.max_num_seqs)
-        t0 = time.time()
-        if args.random:
-            eng = Engine.from_config(cfg, args.seed, **kw)
+        key = (os.path.abspath(args.random or args.model), bool(args.random), args.seed if args.random else None,
+               tuple(sorted(kw.items())))
+        if loaded.get("key") == key:
+            eng = loaded["engine"]
+            for rid in eng.manager.live():                   # a run that failed may have left requests behind
+                eng.end(rid)
+            print(f"tuff: jobs: reusing the loaded model {args.random or args.model}", file=sys.stderr)
         else:
-            eng = Engine.from_folder(args.model, **kw)
-        print(f"tuff: model ready in {time.time() - t0:.2f} s", file=sys.stderr)
+            loaded.clear()
+            t0 = time.time()
+            if args.random:
+                eng = Engine.from_config(cfg, args.seed, **kw)
+            else:
+                eng = Engine.from_folder(args.model, **kw)
+            loaded.update(key=key, engine=eng)
+            print(f"tuff: model ready in {time.time() - t0:.2f} s", file=sys.stderr)
     except Exception as e:                                   # noqa: BLE001 - reported, then exit code
         print(f"tuff: {type(e).__name__}: {e}", file=sys.stderr)
         return 1 if type(e).__name__ in ("WeightsError", "ConfigError") else 3
