@@ -1,4 +1,5 @@
-"""Compiles the HIP sources of this folder for gfx950 with hipcc, one shared library a source.
+"""Compiles the HIP sources of this folder for gfx950 with hipcc, one shared library a source,
+and the plain C interface (capi.cpp, host code only) with the C++ compiler against libpython.
 
 A library is rebuilt when the hash of its source, the shared header and the flags differs
 from the one recorded beside it; otherwise the built file is loaded as it is.  Libraries go
@@ -38,6 +39,11 @@ MODULES = {
     "sampling": "sampling.hip",
 }
 
+# Host-only libraries: name -> (source, further files whose change makes it stale)
+HOST_MODULES = {
+    "amd": ("capi.cpp", ["../../include/tuff_amd.h"]),     # libtuff_amd.so, the plain C interface
+}
+
 
 class BuildError(RuntimeError):
     pass
@@ -69,12 +75,32 @@ def _writable_dir() -> str:
     raise BuildError("no writable folder for the compiled kernels; set TUFF_AMD_BUILD_DIR")
 
 
+def _host_command() -> list[str]:
+    """Compiler and flags for a host-only library that embeds the Python interpreter."""
+    import sysconfig
+    cxx = next((c for c in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"),
+                            shutil.which("clang++"), "/opt/rocm/llvm/bin/clang++") if c and shutil.which(c)), None)
+    if cxx is None:
+        raise BuildError("no C++ compiler found (looked at $CXX, g++, c++, clang++)")
+    v = sysconfig.get_config_vars()
+    libdirs = [d for d in (v.get("LIBPL"), v.get("LIBDIR")) if d]
+    return ([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall",
+             "-I", sysconfig.get_paths()["include"]]
+            + [f"-L{d}" for d in libdirs] + [f"-Wl,-rpath,{d}" for d in libdirs[1:]]
+            + [f"-lpython{v['LDVERSION']}", "-ldl", "-lpthread"])
+
+
 def _source_hash(module: str) -> str:
     h = hashlib.sha256()
-    for fn in [MODULES[module]] + HEADERS:
+    if module in HOST_MODULES:
+        src, more = HOST_MODULES[module]
+        files, flags = [src] + more, _host_command()
+    else:
+        files, flags = [MODULES[module]] + HEADERS, FLAGS
+    for fn in files:
         with open(os.path.join(HERE, fn), "rb") as f:
             h.update(f.read())
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(flags).encode())
     return h.hexdigest()
 
 
@@ -105,15 +131,21 @@ def _say(msg: str) -> None:
 
 def compile_module(module: str, quiet: bool = False) -> str:
     """Compiles one module unconditionally and returns the path of the library."""
-    if module not in MODULES:
-        raise BuildError(f"unknown kernel module '{module}'; known: {sorted(MODULES)}")
-    src = os.path.join(HERE, MODULES[module])
+    if module not in MODULES and module not in HOST_MODULES:
+        raise BuildError(f"unknown module '{module}'; known: {sorted(MODULES) + sorted(HOST_MODULES)}")
+    host = module in HOST_MODULES
+    name = HOST_MODULES[module][0] if host else MODULES[module]
+    src = os.path.join(HERE, name)
     out_dir = _writable_dir()
     out = os.path.join(out_dir, f"libtuff_{module}.so")
     tmp = os.path.join(out_dir, f".libtuff_{module}.{os.getpid()}.{threading.get_ident()}.so")
-    cmd = [_hipcc()] + FLAGS + ["-I", HERE, "-o", tmp, src]
+    if host:
+        cmd = _host_command()
+        cmd = cmd[:1] + [src, "-o", tmp] + cmd[1:]          # libraries after the source that needs them
+    else:
+        cmd = [_hipcc()] + FLAGS + ["-I", HERE, "-o", tmp, src]
     if not quiet:
-        _say(f"compiling {MODULES[module]} for {ARCH} ...")
+        _say(f"compiling {name}" + ("" if host else f" for {ARCH}") + " ...")
     env = dict(os.environ)
     env.setdefault("HOME", out_dir)            # hipcc wants somewhere to keep temporaries
     t0 = time.time()
@@ -123,7 +155,7 @@ def compile_module(module: str, quiet: bool = False) -> str:
     def ticker():
         while not done.wait(10.0):
             if not quiet:
-                _say(f"  still compiling {MODULES[module]} ({time.time() - t0:.0f} s)")
+                _say(f"  still compiling {name} ({time.time() - t0:.0f} s)")
     th = threading.Thread(target=ticker, daemon=True)
     th.start()
     log, _ = proc.communicate()
@@ -133,7 +165,7 @@ def compile_module(module: str, quiet: bool = False) -> str:
             os.unlink(tmp)
         except OSError:
             pass
-        raise BuildError(f"hipcc failed on {MODULES[module]} (exit {proc.returncode}):\n{log}")
+        raise BuildError(f"{os.path.basename(cmd[0])} failed on {name} (exit {proc.returncode}):\n{log}")
     os.replace(tmp, out)
     with open(out + ".hash.tmp", "w") as f:
         f.write(_source_hash(module))
@@ -154,8 +186,9 @@ def ensure_built(module: str) -> str:
 def build_all(force: bool = True, jobs: int = 8) -> dict[str, str]:
     """Compiles every module (in parallel).  With force=False only the missing or stale ones."""
     from concurrent.futures import ThreadPoolExecutor
-    todo = [m for m in MODULES if force or find_built(m) is None]
-    out = {m: find_built(m) for m in MODULES if m not in todo}
+    every = list(MODULES) + list(HOST_MODULES)
+    todo = [m for m in every if force or find_built(m) is None]
+    out = {m: find_built(m) for m in every if m not in todo}
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo) or 1))) as ex:
         for m, path in zip(todo, ex.map(compile_module, todo)):
             out[m] = path

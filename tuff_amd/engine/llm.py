@@ -67,50 +67,15 @@ class LLM:
                          max_model_len=self.ctx_size, eos_token_id=eos)
 
     def run(self, sched: Scheduler, on_step=None) -> None:
-        """Steps until every request of the scheduler has finished.
-
-        While the requests only decode, the next step is started before the tokens of the
-        current one have reached the host: it takes them from the sampler's output on the device
-        (`run_ahead`).  The host then accounts for a step while the GPU runs the next one."""
-        steps = tokens = ahead_steps = 0
-
-        def start(batch, device_tokens=None):
-            entries = [StepEntry(s.request.id, s.tokens, [len(s.tokens) - 1] if s.samples else [])
-                       for s in batch]
-            logits = self.engine.step(entries, device_tokens)
-            sampling = [s.request for s in batch if s.samples]
-            pending = self.sampler.launch(logits, [r.sampler for r in sampling]) if sampling else None
-            return sampling, pending
-
-        under_way = None                                  # a step started ahead: (batch, sampling, pending)
-        while under_way is not None or sched.has_unfinished():
-            if under_way is None:
-                batch = sched.schedule()
-                if not batch:
-                    if sched.has_unfinished():
-                        raise RuntimeError("the scheduler made no progress: no request fits the cache")
-                    break
-                sampling, pending = start(batch)
-            else:
-                batch, sampling, pending = under_way
-                under_way = None
-            if self.run_ahead and pending is not None and len(sampling) == len(batch) \
-                    and not any(self.sampler.needs_history(r.sampler) for r in sampling):
-                nxt = sched.schedule_ahead(batch)
-                if nxt is not None:
-                    under_way = (nxt,) + start(nxt, pending.out)
-                    ahead_steps += 1
-            sampled = {}
-            if pending is not None:
-                sampled = {r.id: t for r, t in zip(sampling, pending.tokens())}
-            live = [s for s in batch if s.request.status != "finished"]
-            sched.update(batch, sampled)
-            steps += 1
-            tokens += sum(len(s.tokens) for s in live)
+        """Steps until every request of the scheduler has finished."""
+        loop = Loop(self, sched)
+        while True:
+            done = loop.step()
+            if done is None:
+                break
             if on_step is not None:
-                on_step(live, {s.request.id: sampled[s.request.id] for s in live if s.samples})
-        self.last_stats = {"steps": steps, "tokens_run": tokens, "preemptions": sched.num_preemptions,
-                           "steps_started_ahead": ahead_steps}
+                on_step(*done)
+        self.last_stats = loop.stats()
 
     def generate(self, prompts: Sequence[Sequence[int]], params=None) -> list[Generation]:
         """prompts: token id lists.  params: one SamplingParams for all, or one per prompt."""
@@ -127,3 +92,60 @@ class LLM:
             sched.add(r)
         self.run(sched)
         return [Generation(r.id, r.prompt, list(r.output), r.finish_reason or "", r.preemptions) for r in reqs]
+
+
+class Loop:
+    """The run loop, one step a call: scheduler -> step -> sampler -> scheduler.
+
+    While the requests only decode, the next step is started before the tokens of the
+    current one have reached the host: it takes them from the sampler's output on the device
+    (`run_ahead`).  The host then accounts for a step while the GPU runs the next one.
+    Requests may be added to the scheduler between calls."""
+
+    def __init__(self, llm: "LLM", sched: Scheduler):
+        self.llm, self.sched = llm, sched
+        self.under_way = None                             # a step started ahead: (batch, sampling, pending)
+        self.steps = self.tokens = self.ahead_steps = 0
+
+    def _start(self, batch, device_tokens=None):
+        entries = [StepEntry(s.request.id, s.tokens, [len(s.tokens) - 1] if s.samples else [])
+                   for s in batch]
+        logits = self.llm.engine.step(entries, device_tokens)
+        sampling = [s.request for s in batch if s.samples]
+        pending = self.llm.sampler.launch(logits, [r.sampler for r in sampling]) if sampling else None
+        return sampling, pending
+
+    def step(self):
+        """Runs one step and accounts for it.  Returns (the Scheduled entries whose requests were
+        still live, {request id: token drawn}), or None when nothing is left to do."""
+        sched, sampler = self.sched, self.llm.sampler
+        if self.under_way is None:
+            if not sched.has_unfinished():
+                return None
+            batch = sched.schedule()
+            if not batch:
+                if sched.has_unfinished():
+                    raise RuntimeError("the scheduler made no progress: no request fits the cache")
+                return None
+            sampling, pending = self._start(batch)
+        else:
+            batch, sampling, pending = self.under_way
+            self.under_way = None
+        if self.llm.run_ahead and pending is not None and len(sampling) == len(batch) \
+                and not any(sampler.needs_history(r.sampler) for r in sampling):
+            nxt = sched.schedule_ahead(batch)
+            if nxt is not None:
+                self.under_way = (nxt,) + self._start(nxt, pending.out)
+                self.ahead_steps += 1
+        sampled = {}
+        if pending is not None:
+            sampled = {r.id: t for r, t in zip(sampling, pending.tokens())}
+        live = [s for s in batch if s.request.status != "finished"]
+        sched.update(batch, sampled)
+        self.steps += 1
+        self.tokens += sum(len(s.tokens) for s in live)
+        return live, {s.request.id: sampled[s.request.id] for s in live if s.samples}
+
+    def stats(self) -> dict:
+        return {"steps": self.steps, "tokens_run": self.tokens, "preemptions": self.sched.num_preemptions,
+                "steps_started_ahead": self.ahead_steps}
