@@ -193,6 +193,28 @@ def test_recorded_decode_steps_equal_eager_steps(gpu, dtype):
     util.assert_close(dtype, got["y"][mask], full[mask], "y")
 
 
+def test_layers_of_full_size_float32_against_the_plain_implementation(gpu):
+    """Layers with the sizes of a 1.2B model, float32, against the plain implementation: whole, a
+    head then single tokens, and two requests mixed in portions."""
+    name = "F"
+    V = util.FULL_SIZE_LAYERS["vocab_size"]
+    reqs = {"a": util.rand_tokens(70, V, 21), "b": util.rand_tokens(37, V, 22)}
+    from tuff_amd.engine.engine import Engine
+    folder = util.model_folder(name, "bfloat16")            # both paths read these bfloat16 weights
+    eng = Engine.from_folder(folder, dtype="float32", page_size=16, max_tokens=256)
+    want = {rid: util.plain_logits(name, toks, "bfloat16") for rid, toks in reqs.items()}
+    for plan in (util.plan_whole(reqs), util.plan_tail(reqs, 8), util.plan_mixed(reqs, seed=2, decode_tail=6)):
+        got = util.run_plan(eng, plan)
+        eng.manager.check()
+        for rid in reqs:
+            util.assert_close_f32(got[rid], want[rid], f"full-size float32 {rid}")
+    del eng
+    eng16 = Engine.from_folder(folder, dtype="bfloat16", page_size=16, max_tokens=256)
+    got16 = util.run_plan(eng16, util.plan_whole(reqs))
+    for rid in reqs:
+        util.assert_close_bf16(got16[rid], want[rid], f"full-size bfloat16 {rid}")
+
+
 def test_layers_of_full_size_bfloat16_against_float32(gpu):
     """Layers with the sizes of a 1.2B model (hidden 2048, 32 query and 8 kv heads of 64, feed-forward
     8192, vocabulary 65536; two conv layers and an attention layer): the bfloat16 kernels chosen at
