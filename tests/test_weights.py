@@ -169,3 +169,21 @@ def test_missing_file():
     _, _, decls = model_and_decls("A")
     with pytest.raises(loader.WeightsError):
         loader.load_weights("/nonexistent/folder", decls, torch.bfloat16, "cpu")
+
+
+def test_tile_major_weight_layout():
+    """The order the matrix kernels stream a bfloat16 weight in: piece l of block (t, b) is row
+    16 t + l % 16, k 32 b + 8 (l // 16) .. + 7; zero outside the matrix; rows() gives it back."""
+    from tuff_amd.csrc import ops
+    for N, K in ((50, 40), (16, 32), (33, 96)):
+        w = torch.randn(N, K).to(torch.bfloat16)
+        t = ops.tile_weight(w)
+        assert t.shape == (N, K) and t.blocks.shape == (-(-N // 16), -(-K // 32), 64, 8)
+        for tile, blk, piece in ((0, 0, 0), (t.blocks.shape[0] - 1, t.blocks.shape[1] - 1, 63), (1 % t.blocks.shape[0], 0, 37)):
+            row, k = 16 * tile + piece % 16, 32 * blk + 8 * (piece // 16)
+            want = torch.zeros(8, dtype=torch.bfloat16)
+            if row < N:
+                n = max(0, min(8, K - k))
+                want[:n] = w[row, k:k + n]
+            assert torch.equal(t.blocks[tile, blk, piece], want), (N, K, tile, blk, piece)
+        assert torch.equal(t.rows(), w)

@@ -188,6 +188,50 @@ def fill_u32(t: torch.Tensor, value: int = 0) -> None:
 
 
 # ------------------------------------------------------------------------------ GEMM
+class TiledWeight:
+    """A bfloat16 weight [N, K] in the order the matrix kernels stream it: blocks of 16 rows x 32 k,
+    [ceil(N/16)][ceil(K/32)] of them, each 1 KB with piece l of 16 bytes = row l % 16,
+    k 8 (l // 16) .. 8 (l // 16) + 7; rows and k beyond the matrix are zero."""
+
+    def __init__(self, blocks: torch.Tensor, N: int, K: int):
+        self.blocks, self.shape = blocks, (int(N), int(K))
+        self.dtype, self.device = blocks.dtype, blocks.device
+
+    def data_ptr(self) -> int:
+        return self.blocks.data_ptr()
+
+    def rows(self) -> torch.Tensor:
+        """The weight back in row-major order [N, K] (a copy)."""
+        N, K = self.shape
+        t = self.blocks.view(-1, self.blocks.shape[1], 4, 16, 8).permute(0, 3, 1, 2, 4)
+        return t.reshape(t.shape[0] * 16, -1)[:N, :K].contiguous()
+
+
+def tile_weight(w: torch.Tensor) -> TiledWeight:
+    """The tile-major copy of a row-major bfloat16 weight [N, K].  Made once when a weight is bound."""
+    if w.dim() != 2 or w.dtype != torch.bfloat16:
+        raise KernelError(f"tile_weight: a bfloat16 matrix is needed, got {w.dtype} {tuple(w.shape)}")
+    N, K = w.shape
+    Np, Kp = -(-N // 16) * 16, -(-K // 32) * 32
+    if (Np, Kp) != (N, K):
+        padded = torch.zeros(Np, Kp, dtype=w.dtype, device=w.device)
+        padded[:N, :K] = w
+        w = padded
+    blocks = w.view(Np // 16, 16, Kp // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
+    return TiledWeight(blocks.view(Np // 16, Kp // 32, 64, 8), N, K)
+
+
+def _tiled(w, N: int, K: int) -> TiledWeight:
+    """w as the bfloat16 kernels take it.  A plain tensor is converted on the spot (tests and single
+    calls; the parts bind tiled weights)."""
+    if not isinstance(w, TiledWeight):
+        _gpu("w", w, torch.bfloat16, (N, K))
+        w = tile_weight(w)
+    if not w.blocks.is_cuda or not w.blocks.is_contiguous() or w.shape != (N, K):
+        raise KernelError(f"w: a tiled weight {(N, K)} on the GPU is needed, got {w.shape} on {w.device}")
+    return w
+
+
 def _bf16_mode(out: torch.Tensor, accumulate: bool, swiglu: bool, M: int, N: int) -> int:
     if swiglu:
         if accumulate or out.dtype != torch.bfloat16 or N % 2:
@@ -214,8 +258,10 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     M, K = x.shape
     N = w.shape[0]
     _gpu("x", x)
-    _gpu("w", w, x.dtype, (N, K))
     if x.dtype == torch.float32:
+        if isinstance(w, TiledWeight):
+            raise KernelError("gemm: float32 activations with a tiled bfloat16 weight")
+        _gpu("w", w, x.dtype, (N, K))
         if out.dtype != torch.float32 or swiglu:
             raise KernelError("gemm: float32 operands need a float32 output and have no fused epilogue")
         _gpu("out", out, shape=(M, N))
@@ -226,6 +272,7 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         raise KernelError(f"gemm: unsupported operand type {x.dtype}")
     if K % 8 != 0:
         raise KernelError(f"gemm: the bfloat16 kernels need an inner size that is a multiple of 8, got {K}")
+    w = _tiled(w, N, K)
     mode = _bf16_mode(out, accumulate, swiglu, M, N)
     ws_floats = _gemm_workspace(M, N, K)
     ws = torch.empty(ws_floats, dtype=torch.float32, device=x.device) if ws_floats else None
@@ -246,7 +293,7 @@ def gemm_normed(x: torch.Tensor, norm_w: torch.Tensor, eps: float, w: torch.Tens
     N = w.shape[0]
     _gpu("x", x, torch.float32)
     _gpu("norm_w", norm_w, torch.float32, (K,))
-    _gpu("w", w, torch.bfloat16, (N, K))
+    w = _tiled(w, N, K)
     _opt("rows", rows, torch.int32, (M,))
     if M > NORMED_MAX_ROWS or K > NORMED_MAX_K or K % 8:
         raise KernelError(f"gemm_normed: at most {NORMED_MAX_ROWS} rows and an inner size that is a multiple of 8 "
@@ -276,7 +323,7 @@ def gemm_accum_emit(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, ne
     M, K = x.shape
     N = w.shape[0]
     _gpu("x", x, torch.bfloat16)
-    _gpu("w", w, torch.bfloat16, (N, K))
+    w = _tiled(w, N, K)
     _gpu("residual", residual, torch.float32, (M, N))
     _gpu("next_norm_w", next_norm_w, torch.float32, (N,))
     _gpu("xw", xw, torch.bfloat16, (M, N))
@@ -296,7 +343,7 @@ def gemm_scaled(xw: torch.Tensor, ss: torch.Tensor, eps: float, w: torch.Tensor,
     N = w.shape[0]
     _gpu("xw", xw, torch.bfloat16)
     _gpu("ss", ss, torch.float32, (None, 16))
-    _gpu("w", w, torch.bfloat16, (N, K))
+    w = _tiled(w, N, K)
     if M > NORMED_MAX_ROWS or K % 8:
         raise KernelError(f"gemm_scaled: at most {NORMED_MAX_ROWS} rows, inner size a multiple of 8")
     mode = _bf16_mode(out, accumulate, swiglu, M, N)

@@ -118,6 +118,12 @@ class DecoderModel:
         self._head_cast: Optional[torch.Tensor] = None
         if self.head.dtype != rt.dtype and self.head.dtype != torch.float32:
             raise TypeError(f"head weight of type {self.head.dtype} in a {rt.dtype} run")
+        if self.head.dtype == torch.bfloat16:
+            # the matrix kernels stream a tile-major copy; a tied embedding keeps its rows for the lookup
+            if self.hidden_size % 8 != 0:
+                raise ValueError(f"the bfloat16 matrix kernels need a hidden size that is a multiple of 8, "
+                                 f"got {self.hidden_size}")
+            self.head = ops.tile_weight(self.head)
 
     # --------------------------------------------------------------------- forward
     def forward(self, ctx, cache_views: dict[int, object]) -> Optional[torch.Tensor]:

@@ -26,7 +26,7 @@ class Linear:
         self.in_features, self.outs = int(in_features), [int(o) for o in outs]
         self.out_features = sum(self.outs)
         self.aliases = [tuple(a) for a in aliases] if aliases else [()] * len(self.names)
-        self.weight: Optional[torch.Tensor] = None
+        self.weight = None            # bound: ops.TiledWeight (bfloat16) or a float32 tensor [out, in]
         self.swiglu_pair = bool(swiglu_pair)
         if self.swiglu_pair and (len(self.names) != 2 or self.outs[0] != self.outs[1]):
             raise ValueError("a SwiGLU pair is two tensors of one shape")
@@ -49,9 +49,11 @@ class Linear:
                 self.interleaved = True
             else:
                 self.weight = torch.cat(ws, dim=0).contiguous()
-        if self.weight.dtype == torch.bfloat16 and self.in_features % 8 != 0:
-            raise ValueError(f"{self.names[0]}: the bfloat16 matrix kernels need an input size that is a "
-                             f"multiple of 8, got {self.in_features}")
+        if self.weight.dtype == torch.bfloat16:
+            if self.in_features % 8 != 0:
+                raise ValueError(f"{self.names[0]}: the bfloat16 matrix kernels need an input size that is a "
+                                 f"multiple of 8, got {self.in_features}")
+            self.weight = ops.tile_weight(self.weight)       # the order the kernels stream it in
 
     def forward(self, x, *, out_dtype: Optional[torch.dtype] = None,
                 accumulate_into: Optional[torch.Tensor] = None, swiglu: bool = False) -> Optional[torch.Tensor]:
