@@ -120,7 +120,9 @@ def test_gemm_with_the_norm_inside(gpu, M, N, K, use_rows):
         assert torch.equal(one[0], out[M - 1])
 
 
-@pytest.mark.parametrize("M,d,K1,N2", [(1, 64, 192, 512), (8, 2048, 8192, 6144), (16, 240, 328, 777 * 2), (5, 96, 96, 40)])
+@pytest.mark.parametrize("M,d,K1,N2", [(1, 64, 192, 512), (8, 2048, 8192, 6144), (16, 240, 328, 777 * 2), (5, 96, 96, 40),
+                                       (17, 96, 96, 40), (40, 2048, 8192, 6144), (64, 240, 328, 777 * 2), (33, 64, 192, 512),
+                                       (64, 2048, 2048, 65536)])
 def test_gemm_that_prepares_the_next_norm(gpu, M, d, K1, N2):
     """residual += a @ w1.T leaves bf16(residual * norm weight) and per-tile row sums of squares;
     the next product scales its rows by them: together rmsnorm(residual) @ w2.T."""
@@ -133,7 +135,7 @@ def test_gemm_that_prepares_the_next_norm(gpu, M, d, K1, N2):
     eps = 1e-5
     res = res0.to(gpu)
     xw = torch.empty(M, d, dtype=torch.bfloat16, device=gpu)
-    ss = torch.full((ops.gemm_emit_tiles(d, K1), 16), float("nan"), device=gpu)
+    ss = torch.full(ops.gemm_emit_layout(M, d, K1), float("nan"), device=gpu)
     ops.gemm_accum_emit(a.to(gpu), w1.to(gpu), res, nw.to(gpu), xw, ss)
     want_res = res0.double() + a.double() @ w1.double().T
     assert (res.cpu().double() - want_res).abs().max() <= 1e-5 * float(want_res.abs().max()) + 1e-6 * K1

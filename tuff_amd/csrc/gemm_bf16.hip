@@ -15,7 +15,8 @@
 // The skinny kernels stream each weight byte once from HBM straight into MFMA operands.  Where
 // N alone gives too little parallelism to fill 256 CUs, skinny16 uses more waves a workgroup
 // (8 or 16, partials added in wave order through LDS) and skinny64 splits K over workgroups
-// (partial tiles in a work space, added in slice order by a second kernel).  The cut depends
+// (partial tiles in a work space, added in slice order by a second kernel, which also does the
+// epilogue).  The cut depends
 // on N and K only, never on M, so the order of additions is fixed.
 //
 // All use v_mfma_f32_16x16x32_bf16.  Lane l of a wave supplies row (l % 16) of an operand tile
@@ -456,15 +457,21 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
 // 16 < M <= 64.  grid (tiles of 64 columns, K slices).  Wave w owns columns 16w..16w+15 of the
 // tile and all MT row tiles.  The X rows of a K chunk (128 wide) go through LDS once for the
 // four waves, double buffered; W goes from HBM to registers one chunk ahead.  With more than
-// one K slice the partial tiles go to a work space and a second kernel adds them in slice order.
+// one K slice, or when the epilogue has to leave the next norm's operand, the partial tiles go to
+// a work space and splitk_finish_kernel adds them in slice order and does the epilogue.
+// NORM_SCALED as above, with the sums of squares per tile of 64 columns: ss_in [n_ss][64].
 constexpr int SK_NT = 256;
 constexpr int XS_STRIDE = SK_CHUNK + 8;             // bf16 elements; 272 bytes: conflict-free 16-byte reads
 
-template <int MT, int MODE>
+template <int MT, int MODE, int NORM>
 __global__ __launch_bounds__(SK_NT) void gemm_bf16_skinny64_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                                    void* __restrict__ Y, int M, int N, int K, int chunks_per_slice,
-                                                                   float* __restrict__ ws) {
+                                                                   float* __restrict__ ws, bool to_ws,
+                                                                   const float* __restrict__ ss_in, int n_ss, float eps) {
+    static_assert(NORM != NORM_INSIDE, "the norm inside is for at most 16 rows");
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16 * XS_STRIDE];
+    __shared__ float ss_parts[4][64];
+    __shared__ float scale_lds[64];
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
     const int r16 = lane % 16, g = lane / 16;
     const int tile = blockIdx.x, slice = blockIdx.y, n_slices = gridDim.y;
@@ -512,9 +519,17 @@ __global__ __launch_bounds__(SK_NT) void gemm_bf16_skinny64_kernel(const bf16_t*
     if (c_begin < c_end) {
         load_x(c_begin);
         load_w4(c_begin, b0);
-        store_x(0);
     }
+    if (NORM == NORM_SCALED && !to_ws) {
+        // thread -> (row tid % 64, part tid / 64): part p adds the tiles p, p + 4, ... of its row
+        float t = 0.f;
+        for (int j = tid / 64; j < n_ss; j += 4) t += ss_in[(long long)j * 64 + tid % 64];
+        ss_parts[tid / 64][tid % 64] = t;
+    }
+    if (c_begin < c_end) store_x(0);
     __syncthreads();
+    if (NORM == NORM_SCALED && !to_ws && tid < 64)    // read in the epilogue, behind the barriers of the loop
+        scale_lds[tid] = 1.0f / sqrtf((ss_parts[0][tid] + ss_parts[1][tid] + ss_parts[2][tid] + ss_parts[3][tid]) / (float)K + eps);
     for (int c = c_begin; c < c_end; c += 2) {
         // chunk c from buffer 0 / b0, chunk c+1 from buffer 1 / b1
         const bool more1 = c + 1 < c_end, more2 = c + 2 < c_end;
@@ -531,7 +546,7 @@ __global__ __launch_bounds__(SK_NT) void gemm_bf16_skinny64_kernel(const bf16_t*
     }
 
     const long long col = (long long)tile * 64 + wave * 16 + r16;
-    if (n_slices > 1) {
+    if (to_ws) {
         // partial tile of this slice: ws[slice][row][col]
         if (col >= N) return;
         float* mine = ws + (long long)slice * (MT * 16) * N;
@@ -546,40 +561,92 @@ __global__ __launch_bounds__(SK_NT) void gemm_bf16_skinny64_kernel(const bf16_t*
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const long long row = i * 16 + g * 4 + e;
-            const float v = acc[i][e];
+            float v = acc[i][e];
+            if (NORM == NORM_SCALED) v *= scale_lds[row];
             const float partner = (MODE == OUT_SWIGLU) ? __shfl_xor(v, 1, WAVE) : 0.f;
             store_elem<MODE>(Y, row, col, M, N, v, partner);
         }
 }
 
-// Y (=|+=) sum over slices, in slice order, of ws[slice][row][col]; rows_padded rows a slice.
-template <int MODE>
-__global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* __restrict__ Y, int M, int N, int rows_padded,
-                                     int n_slices) {
-    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (MODE == OUT_SWIGLU) {
-        const int F = N / 2;
-        if (i >= (long long)M * F) return;
-        const long long row = i / F, f = i - row * F;
-        float gt = 0.f, up = 0.f;
-        for (int s = 0; s < n_slices; ++s) {
-            const float* p = ws + ((long long)s * rows_padded + row) * N + 2 * f;
-            gt += p[0];
-            up += p[1];
-        }
-        ((bf16_t*)Y)[i] = (bf16_t)silu_mul(gt, up);
-        return;
+// Finishes a product whose partial tiles lie in the work space: v = sum over slices, in slice
+// order, of ws[slice][row][col] (rows_padded rows a slice), scaled per row for NORM_SCALED, then the
+// epilogue of MODE; with EMIT, Y += v and from the new Y the operand of the norm that follows, as
+// in the kernel for at most 16 rows, with sums of squares per tile of 64 columns: emit_ss [tiles][64].
+// grid (tiles of 64 columns, groups of 16 rows), 256 threads: thread -> row tid / 16 of the group and
+// four neighbouring columns.
+struct FinishExtra {
+    const float* ss_in = nullptr; int n_ss = 0; float eps = 0.f; int K = 0;                 // NORM_SCALED
+    const float* emit_nw = nullptr; bf16_t* emit_xw = nullptr; float* emit_ss = nullptr;   // EMIT
+};
+
+template <int MODE, int NORM, bool EMIT>
+__global__ __launch_bounds__(256) void splitk_finish_kernel(const float* __restrict__ ws, void* __restrict__ Y, int M, int N,
+                                                            int rows_padded, int n_slices, FinishExtra ex) {
+    static_assert(!EMIT || MODE == OUT_F32_ACCUM, "the emitting epilogue adds into the residual stream");
+    const int tid = threadIdx.x, q = tid % 16;
+    const long long row = (long long)blockIdx.y * 16 + tid / 16;
+    const long long col = (long long)blockIdx.x * 64 + q * 4;
+    float scale = 1.f;
+    if (NORM == NORM_SCALED) {
+        // the sixteen threads of a row add the tiles q, q + 16, ... and then each other, in a fixed butterfly
+        float t = 0.f;
+        for (int j = q; j < ex.n_ss; j += 16) t += ex.ss_in[(long long)j * 64 + row];
+        t += __shfl_xor(t, 1, WAVE);
+        t += __shfl_xor(t, 2, WAVE);
+        t += __shfl_xor(t, 4, WAVE);
+        t += __shfl_xor(t, 8, WAVE);
+        scale = 1.0f / sqrtf(t / (float)ex.K + ex.eps);
     }
-    if (i >= (long long)M * N) return;
-    float v = 0.f;
-    for (int s = 0; s < n_slices; ++s) v += ws[(long long)s * rows_padded * N + i];
-    store_out<MODE>(Y, i, v);
+    const bool whole = N % 4 == 0 && col + 3 < N;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    if (row < M) {
+        for (int s = 0; s < n_slices; ++s) {
+            const float* p = ws + ((long long)s * rows_padded + row) * N + col;
+            if (whole) {
+                const f32x4 t = *(const f32x4*)p;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] += t[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) if (col + e < N) v[e] += p[e];
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] *= scale;
+    float sq = 0.f;
+    if (row < M) {
+        if (MODE == OUT_SWIGLU) {
+            bf16_t* out = (bf16_t*)Y + row * (N / 2) + col / 2;
+            if (col + 1 < N) out[0] = (bf16_t)silu_mul(v[0], v[1]);
+            if (col + 3 < N) out[1] = (bf16_t)silu_mul(v[2], v[3]);
+        } else if (EMIT) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (col + e < N) {
+                    const float y = ((const float*)Y)[row * N + col + e] + v[e];
+                    ((float*)Y)[row * N + col + e] = y;
+                    ex.emit_xw[row * N + col + e] = (bf16_t)(y * ex.emit_nw[col + e]);
+                    sq = fmaf(y, y, sq);
+                }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) if (col + e < N) store_out<MODE>(Y, row * N + col + e, v[e]);
+        }
+    }
+    if (EMIT) {
+        sq += __shfl_xor(sq, 1, WAVE);
+        sq += __shfl_xor(sq, 2, WAVE);
+        sq += __shfl_xor(sq, 4, WAVE);
+        sq += __shfl_xor(sq, 8, WAVE);
+        if (q == 0) ex.emit_ss[(long long)blockIdx.x * 64 + row] = sq;      // rows M .. 63 of the tile: zero
+    }
 }
 
 struct SkinnyPlan { int tiles, waves, slices, chunks_per_slice, cols; long long ws_floats; };
 
 // How a skinny product is cut.  Depends on N and K (and on which of the two kernels M selects).
-SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16) {
+SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16, bool emit = false) {
     const int nchunks = ceil_div(K, SK_CHUNK);
     SkinnyPlan p;
     p.slices = 1; p.chunks_per_slice = nchunks; p.ws_floats = 0; p.waves = 4;
@@ -604,7 +671,7 @@ SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16) {
         s = max(1, min(s, nchunks / 2));
         p.chunks_per_slice = ceil_div(nchunks, s);
         p.slices = ceil_div(nchunks, p.chunks_per_slice);
-        p.ws_floats = p.slices > 1 ? (long long)p.slices * mt * 16 * N : 0;
+        p.ws_floats = (p.slices > 1 || emit) ? (long long)p.slices * mt * 16 * N : 0;
     }
     return p;
 }
@@ -647,24 +714,47 @@ int launch_skinny16_mode(const void* X, const bf16_t* W, void* Y, int M, int N, 
     return -3;
 }
 
+// 16 < M <= 64.  ws: the work space tuff_gemm_bf16_workspace asks for.
+template <int MODE, int NORM, bool EMIT>
+int launch_skinny64(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, float* ws, const FinishExtra& ex,
+                    hipStream_t stream) {
+    const SkinnyPlan p = plan_skinny(M, N, K, 16, EMIT);
+    dim3 grid(p.tiles, p.slices), block(SK_NT);
+    const bool to_ws = p.ws_floats > 0;
+    if (to_ws && !ws) return -4;
+    const int mt = ceil_div(M, 16);
+#define GO(MT) hipLaunchKernelGGL((gemm_bf16_skinny64_kernel<MT, MODE, NORM>), grid, block, 0, stream, X, W, Y, M, N, K, \
+                                  p.chunks_per_slice, ws, to_ws, ex.ss_in, ex.n_ss, ex.eps)
+    if (mt == 2) GO(2); else if (mt == 3) GO(3); else GO(4);
+#undef GO
+    if (to_ws) {
+        int rc = launch_status();
+        if (rc) return rc;
+        // the emitting epilogue writes the sums of squares of all 64 rows of a tile (zero beyond M)
+        hipLaunchKernelGGL((splitk_finish_kernel<MODE, NORM, EMIT>), dim3(p.tiles, EMIT ? 4 : mt), dim3(256), 0, stream,
+                           (const float*)ws, Y, M, N, mt * 16, p.slices, ex);
+    }
+    return launch_status();
+}
+
+template <int NORM>
+int launch_skinny64_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, int mode, float* ws,
+                         const FinishExtra& ex, hipStream_t stream) {
+    if (mode == OUT_BF16) return launch_skinny64<OUT_BF16, NORM, false>(X, W, Y, M, N, K, ws, ex, stream);
+    if (mode == OUT_F32) return launch_skinny64<OUT_F32, NORM, false>(X, W, Y, M, N, K, ws, ex, stream);
+    if (mode == OUT_F32_ACCUM) return launch_skinny64<OUT_F32_ACCUM, NORM, false>(X, W, Y, M, N, K, ws, ex, stream);
+    if (mode == OUT_SWIGLU) {
+        if (N % 2) return -2;
+        return launch_skinny64<OUT_SWIGLU, NORM, false>(X, W, Y, M, N, K, ws, ex, stream);
+    }
+    return -3;
+}
+
 template <int MODE>
 int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, float* ws, hipStream_t stream) {
     if (M <= 16) return launch_skinny16<MODE, NORM_NONE, false>(X, W, Y, M, N, K, Skinny16Extra(), stream);
     if (M <= 64) {
-        const SkinnyPlan p = plan_skinny(M, N, K);
-        dim3 grid(p.tiles, p.slices), block(SK_NT);
-        if (p.slices > 1 && !ws) return -4;
-#define GO(MT) hipLaunchKernelGGL((gemm_bf16_skinny64_kernel<MT, MODE>), grid, block, 0, stream, X, W, Y, M, N, K, p.chunks_per_slice, ws)
-        const int mt = ceil_div(M, 16);
-        if (mt == 2) GO(2); else if (mt == 3) GO(3); else GO(4);
-#undef GO
-        if (p.slices > 1) {
-            int rc = launch_status();
-            if (rc) return rc;
-            const long long n = (long long)M * (MODE == OUT_SWIGLU ? N / 2 : N);
-            hipLaunchKernelGGL((splitk_reduce_kernel<MODE>), dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, stream,
-                               (const float*)ws, Y, M, N, mt * 16, p.slices);
-        }
+        return launch_skinny64<MODE, NORM_NONE, false>(X, W, Y, M, N, K, ws, FinishExtra(), stream);
     } else {
         // Large blocks where they give most CUs one.  Of the small ones a CU holds two if there are
         // enough; if not, a block is alone on its CU and hides the memory's latency by itself, with
@@ -690,15 +780,21 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
 }
 }  // namespace
 
-// Tiles of columns a product of at most 16 rows is cut into: the first dimension of the sums of
-// squares tuff_gemm_bf16_accum_emit leaves.
-TUFF_EXPORT int tuff_gemm_bf16_emit_tiles(int N, int K) { return plan_skinny(1, N, K).tiles; }
+// How the sums of squares of tuff_gemm_bf16_accum_emit are laid out for a product of M rows:
+// *tiles tiles of columns, *rows rows each (16 for M <= 16, 64 for M <= 64).
+TUFF_EXPORT int tuff_gemm_bf16_emit_layout(int M, int N, int K, int* tiles, int* rows) {
+    if (M > 64) return -2;
+    *tiles = plan_skinny(M, N, K).tiles;
+    *rows = M <= 16 ? 16 : 64;
+    return 0;
+}
 
 // Work space a product of this shape needs: *ws_floats float32 for partial tiles (0: none).
-TUFF_EXPORT int tuff_gemm_bf16_workspace(int M, int N, int K, long long* ws_floats) {
+// emit: for tuff_gemm_bf16_accum_emit.
+TUFF_EXPORT int tuff_gemm_bf16_workspace(int M, int N, int K, int emit, long long* ws_floats) {
     *ws_floats = 0;
     if (M > 64 || M <= 16 || N <= 0) return 0;
-    *ws_floats = plan_skinny(M, N, K).ws_floats;
+    *ws_floats = plan_skinny(M, N, K, 16, emit != 0).ws_floats;
     return 0;
 }
 
@@ -731,25 +827,37 @@ TUFF_EXPORT int tuff_gemm_bf16_normed(const float* X, const int* rows, const flo
     return launch_skinny16_mode<NORM_INSIDE>(X, (const bf16_t*)W, Y, M, N, K, mode, x, stream);
 }
 
-// For M <= 16 rows:  Y += X W^T, and from the new Y (the residual stream, float32 [M, N]) the
-// operand of the RMSNorm that follows: xw = bf16(Y * next_norm_w) [M, N] and ss [ceil(N/16)][16],
-// the sums of squares of each row over each tile of 16 columns.
+// For M <= 64 rows:  Y += X W^T, and from the new Y (the residual stream, float32 [M, N]) the
+// operand of the RMSNorm that follows: xw = bf16(Y * next_norm_w) [M, N] and ss [tiles][rows] (as
+// tuff_gemm_bf16_emit_layout says), the sums of squares of each row over each tile of columns.
+// ws: for M > 16, the work space tuff_gemm_bf16_workspace(M, N, K, 1) asks for.
 TUFF_EXPORT int tuff_gemm_bf16_accum_emit(const void* X, const void* W, float* Y, int M, int N, int K,
-                                          const float* next_norm_w, void* xw, float* ss, hipStream_t stream) {
+                                          const float* next_norm_w, void* xw, float* ss, float* ws, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (K % 8 != 0 || M > 16) return -2;
-    Skinny16Extra x;
+    if (K % 8 != 0 || M > 64) return -2;
+    if (M <= 16) {
+        Skinny16Extra x;
+        x.emit_nw = next_norm_w; x.emit_xw = (bf16_t*)xw; x.emit_ss = ss;
+        return launch_skinny16<OUT_F32_ACCUM, NORM_NONE, true>(X, (const bf16_t*)W, Y, M, N, K, x, stream);
+    }
+    FinishExtra x;
     x.emit_nw = next_norm_w; x.emit_xw = (bf16_t*)xw; x.emit_ss = ss;
-    return launch_skinny16<OUT_F32_ACCUM, NORM_NONE, true>(X, (const bf16_t*)W, Y, M, N, K, x, stream);
+    return launch_skinny64<OUT_F32_ACCUM, NORM_NONE, true>((const bf16_t*)X, (const bf16_t*)W, Y, M, N, K, ws, x, stream);
 }
 
-// For M <= 16 rows:  Y (=|+=) (XW W^T) scaled per row by 1 / sqrt(sum_t ss[t][row] / K + eps), with
-// XW and ss as tuff_gemm_bf16_accum_emit leaves them (n_ss tiles).
+// For M <= 64 rows:  Y (=|+=) (XW W^T) scaled per row by 1 / sqrt(sum_t ss[t][row] / K + eps), with
+// XW and ss as tuff_gemm_bf16_accum_emit leaves them for the same M (n_ss tiles).
+// ws: for M > 16, the work space tuff_gemm_bf16_workspace(M, N, K, 0) asks for.
 TUFF_EXPORT int tuff_gemm_bf16_scaled(const void* XW, const float* ss, int n_ss, float eps, const void* W, void* Y,
-                                      int M, int N, int K, int mode, hipStream_t stream) {
+                                      int M, int N, int K, int mode, float* ws, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (K % 8 != 0 || M > 16 || n_ss < 1) return -2;
-    Skinny16Extra x;
-    x.ss_in = ss; x.n_ss = n_ss; x.eps = eps;
-    return launch_skinny16_mode<NORM_SCALED>(XW, (const bf16_t*)W, Y, M, N, K, mode, x, stream);
+    if (K % 8 != 0 || M > 64 || n_ss < 1) return -2;
+    if (M <= 16) {
+        Skinny16Extra x;
+        x.ss_in = ss; x.n_ss = n_ss; x.eps = eps;
+        return launch_skinny16_mode<NORM_SCALED>(XW, (const bf16_t*)W, Y, M, N, K, mode, x, stream);
+    }
+    FinishExtra x;
+    x.ss_in = ss; x.n_ss = n_ss; x.eps = eps; x.K = K;
+    return launch_skinny64_mode<NORM_SCALED>((const bf16_t*)XW, (const bf16_t*)W, Y, M, N, K, mode, ws, x, stream);
 }

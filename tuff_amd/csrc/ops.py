@@ -37,12 +37,12 @@ _SIGNATURES = {
     },
     "gemm_bf16": {
         "tuff_gemm_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
-        "tuff_gemm_bf16_workspace": [_c_int, _c_int, _c_int, ctypes.POINTER(_c_ll)],
-        "tuff_gemm_bf16_emit_tiles": [_c_int, _c_int],
+        "tuff_gemm_bf16_workspace": [_c_int, _c_int, _c_int, _c_int, ctypes.POINTER(_c_ll)],
+        "tuff_gemm_bf16_emit_layout": [_c_int, _c_int, _c_int, ctypes.POINTER(_c_int), ctypes.POINTER(_c_int)],
         "tuff_gemm_bf16_accum_emit": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
-                                      _c_void_p, _c_void_p],
+                                      _c_void_p, _c_void_p, _c_void_p],
         "tuff_gemm_bf16_scaled": [_c_void_p, _c_void_p, _c_int, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
-                                  _c_int, _c_void_p],
+                                  _c_int, _c_void_p, _c_void_p],
         "tuff_gemm_bf16_normed": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
                                   _c_int, _c_void_p],
     },
@@ -274,13 +274,13 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         raise KernelError(f"gemm: the bfloat16 kernels need an inner size that is a multiple of 8, got {K}")
     w = _tiled(w, N, K)
     mode = _bf16_mode(out, accumulate, swiglu, M, N)
-    ws_floats = _gemm_workspace(M, N, K)
-    ws = torch.empty(ws_floats, dtype=torch.float32, device=x.device) if ws_floats else None
+    ws = _gemm_workspace(M, N, K, x.device)
     _check(load("gemm_bf16").tuff_gemm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, mode,
                                             None if ws is None else ws.data_ptr(), _stream()), "gemm_bf16")
 
 
-NORMED_MAX_ROWS, NORMED_MAX_K = 16, 8192
+NORMED_MAX_ROWS, NORMED_MAX_K = 16, 8192      # gemm_normed: the norm inside the product's kernel
+EMIT_MAX_ROWS = 64                            # gemm_accum_emit / gemm_scaled
 
 
 def gemm_normed(x: torch.Tensor, norm_w: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor, *,
@@ -304,21 +304,24 @@ def gemm_normed(x: torch.Tensor, norm_w: torch.Tensor, eps: float, w: torch.Tens
         out.data_ptr(), M, N, K, mode, _stream()), "gemm_bf16_normed")
 
 
-_emit_tiles: dict = {}
+_emit_layouts: dict = {}
 
 
-def gemm_emit_tiles(N: int, K: int) -> int:
-    """Tiles of columns gemm_accum_emit cuts a product with N outputs and inner size K into."""
-    key = (N, K)
-    if key not in _emit_tiles:
-        _emit_tiles[key] = int(load("gemm_bf16").tuff_gemm_bf16_emit_tiles(N, K))
-    return _emit_tiles[key]
+def gemm_emit_layout(M: int, N: int, K: int) -> tuple:
+    """(tiles, rows): shape of the sums of squares gemm_accum_emit leaves for a product of M rows
+    with N outputs and inner size K."""
+    key = (M <= 16, N, K)
+    if key not in _emit_layouts:
+        t, r = _c_int(0), _c_int(0)
+        _check(load("gemm_bf16").tuff_gemm_bf16_emit_layout(M, N, K, ctypes.byref(t), ctypes.byref(r)), "gemm_emit_layout")
+        _emit_layouts[key] = (int(t.value), int(r.value))
+    return _emit_layouts[key]
 
 
-def gemm_accum_emit(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, next_norm_w: torch.Tensor,
+def gemm_accum_emit(x: torch.Tensor, w, residual: torch.Tensor, next_norm_w: torch.Tensor,
                     xw: torch.Tensor, ss: torch.Tensor) -> None:
-    """residual += x @ w.T for at most 16 rows, and for the RMSNorm that follows: xw = the new
-    residual times next_norm_w as bfloat16, ss [gemm_emit_tiles(N, K), 16] = per-tile sums of squares
+    """residual += x @ w.T for at most 64 rows, and for the RMSNorm that follows: xw = the new
+    residual times next_norm_w as bfloat16, ss [gemm_emit_layout(M, N, K)] = per-tile sums of squares
     of each row."""
     M, K = x.shape
     N = w.shape[0]
@@ -327,44 +330,50 @@ def gemm_accum_emit(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, ne
     _gpu("residual", residual, torch.float32, (M, N))
     _gpu("next_norm_w", next_norm_w, torch.float32, (N,))
     _gpu("xw", xw, torch.bfloat16, (M, N))
-    _gpu("ss", ss, torch.float32, (gemm_emit_tiles(N, K), 16))
-    if M > NORMED_MAX_ROWS or K % 8:
-        raise KernelError(f"gemm_accum_emit: at most {NORMED_MAX_ROWS} rows, inner size a multiple of 8")
+    if M > EMIT_MAX_ROWS or K % 8:
+        raise KernelError(f"gemm_accum_emit: at most {EMIT_MAX_ROWS} rows, inner size a multiple of 8")
+    _gpu("ss", ss, torch.float32, gemm_emit_layout(M, N, K))
+    ws = _gemm_workspace(M, N, K, x.device, emit=True)
     _check(load("gemm_bf16").tuff_gemm_bf16_accum_emit(x.data_ptr(), w.data_ptr(), residual.data_ptr(), M, N, K,
                                                        next_norm_w.data_ptr(), xw.data_ptr(), ss.data_ptr(),
-                                                       _stream()), "gemm_bf16_accum_emit")
+                                                       None if ws is None else ws.data_ptr(), _stream()),
+           "gemm_bf16_accum_emit")
 
 
-def gemm_scaled(xw: torch.Tensor, ss: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor, *,
+def gemm_scaled(xw: torch.Tensor, ss: torch.Tensor, eps: float, w, out: torch.Tensor, *,
                 accumulate: bool = False, swiglu: bool = False) -> None:
-    """out (=|+=) rmsnorm(x) @ w.T from what gemm_accum_emit left: xw = bf16(x * norm weight) and the
-    per-tile sums of squares ss; each row of the product is scaled by 1 / sqrt(sum(ss) / K + eps)."""
+    """out (=|+=) rmsnorm(x) @ w.T from what gemm_accum_emit left for the same number of rows:
+    xw = bf16(x * norm weight) and the per-tile sums of squares ss; each row of the product is
+    scaled by 1 / sqrt(sum(ss) / K + eps)."""
     M, K = xw.shape
     N = w.shape[0]
     _gpu("xw", xw, torch.bfloat16)
-    _gpu("ss", ss, torch.float32, (None, 16))
+    if M > EMIT_MAX_ROWS or K % 8:
+        raise KernelError(f"gemm_scaled: at most {EMIT_MAX_ROWS} rows, inner size a multiple of 8")
+    _gpu("ss", ss, torch.float32, (None, 16 if M <= 16 else 64))
     w = _tiled(w, N, K)
-    if M > NORMED_MAX_ROWS or K % 8:
-        raise KernelError(f"gemm_scaled: at most {NORMED_MAX_ROWS} rows, inner size a multiple of 8")
     mode = _bf16_mode(out, accumulate, swiglu, M, N)
+    ws = _gemm_workspace(M, N, K, xw.device)
     _check(load("gemm_bf16").tuff_gemm_bf16_scaled(xw.data_ptr(), ss.data_ptr(), ss.shape[0], float(eps), w.data_ptr(),
-                                                   out.data_ptr(), M, N, K, mode, _stream()), "gemm_bf16_scaled")
+                                                   out.data_ptr(), M, N, K, mode,
+                                                   None if ws is None else ws.data_ptr(), _stream()), "gemm_bf16_scaled")
 
 
 _plans: dict = {}
 
 
-def _gemm_workspace(M: int, N: int, K: int) -> int:
-    """float32 elements of work space a bfloat16 product of this shape needs (0: none)."""
+def _gemm_workspace(M: int, N: int, K: int, device, emit: bool = False) -> Optional[torch.Tensor]:
+    """The float32 work space a bfloat16 product of this shape needs, or None.  Taken anew for every
+    call: the allocator hands the same block out again."""
     if M <= 16 or M > 64:
-        return 0
-    key = (M, N, K)
+        return None
+    key = (M, N, K, emit)
     n = _plans.get(key)
     if n is None:
         a = _c_ll(0)
-        load("gemm_bf16").tuff_gemm_bf16_workspace(M, N, K, ctypes.byref(a))
+        load("gemm_bf16").tuff_gemm_bf16_workspace(M, N, K, int(emit), ctypes.byref(a))
         n = _plans[key] = int(a.value)
-    return n
+    return torch.empty(n, dtype=torch.float32, device=device) if n else None
 
 
 # ----------------------------------------------------------------- q/k/v post-processing

@@ -133,9 +133,12 @@ class DecoderModel:
         x = torch.empty(ctx.T, self.hidden_size, dtype=torch.float32, device=rt.device)
         ops.embed_rows(self.embedding, ctx.tokens, x)
         all_rows = ctx.n_logits == ctx.T and bool(ctx.host.get("logit_rows_identity", False))
+        # the final norm inside the head's product (at most 16 rows), or, when every row is wanted,
+        # from the row scales the last block leaves (at most 64)
         head_fused = (hasattr(self.final_norm, "pending") and self.head.dtype == torch.bfloat16
-                      and 0 < ctx.n_logits <= ops.NORMED_MAX_ROWS and self.hidden_size <= ops.NORMED_MAX_K
-                      and self.hidden_size % 8 == 0)
+                      and self.hidden_size % 8 == 0 and ctx.n_logits > 0
+                      and (ctx.n_logits <= ops.NORMED_MAX_ROWS and self.hidden_size <= ops.NORMED_MAX_K
+                           or all_rows and ctx.n_logits <= ops.EMIT_MAX_ROWS))
         for i, run in enumerate(self.schedule):
             block = self.blocks[run.block]
             if getattr(block, "takes_next_norm", False):
@@ -155,9 +158,10 @@ class DecoderModel:
             p = fn.pending(x, None if all_rows else ctx.logit_rows)
             if p.pre is not None:
                 ops.gemm_scaled(p.pre[0], p.pre[1], fn.eps, self.head, logits)
-            else:
+                return logits
+            if ctx.n_logits <= ops.NORMED_MAX_ROWS and self.hidden_size <= ops.NORMED_MAX_K:
                 ops.gemm_normed(x, fn.weight_f32, fn.eps, self.head, logits, rows=ctx.logit_rows)
-            return logits
+                return logits
         h = self.final_norm.forward(x, rows=ctx.logit_rows)
         if h.dtype != self.head.dtype:
             h32 = torch.empty(h.shape, dtype=torch.float32, device=rt.device)

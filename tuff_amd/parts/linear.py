@@ -67,8 +67,10 @@ class Linear:
         pending = x if isinstance(x, PendingNorm) else None
         if pending is not None:
             T = pending.shape[0]
-            fused = (w.dtype == torch.bfloat16 and T <= ops.NORMED_MAX_ROWS
-                     and self.in_features <= ops.NORMED_MAX_K and self.in_features % 8 == 0)
+            # the row scales left by the product before (any T up to 64), or the norm inside this product
+            fused = w.dtype == torch.bfloat16 and self.in_features % 8 == 0 and (
+                T <= ops.EMIT_MAX_ROWS if pending.pre is not None
+                else T <= ops.NORMED_MAX_ROWS and self.in_features <= ops.NORMED_MAX_K)
             if not fused:
                 x, pending = pending.tensor(), None
         if pending is None:
@@ -95,10 +97,10 @@ class Linear:
         if accumulate_into is not None:
             nxt = getattr(accumulate_into, "_tuff_next_norm", None)
             if (nxt is not None and pending is None and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
-                    and T <= ops.NORMED_MAX_ROWS):
+                    and T <= ops.EMIT_MAX_ROWS):
                 # the norm that follows reads the sum just made: leave it its operand and row sums
                 xw = torch.empty(T, self.out_features, dtype=torch.bfloat16, device=dev)
-                ss = torch.empty(ops.gemm_emit_tiles(self.out_features, self.in_features), 16, dtype=torch.float32, device=dev)
+                ss = torch.empty(ops.gemm_emit_layout(T, self.out_features, self.in_features), dtype=torch.float32, device=dev)
                 ops.gemm_accum_emit(x, w, accumulate_into, nxt.weight_f32, xw, ss)
                 nxt.announce_operand(accumulate_into, xw, ss)
                 return None
