@@ -109,17 +109,20 @@ def run_decode(llm, cfg, batch: int, ctx_end: int, steps: int, warmup: int, seed
 
 def run_prefill(llm, cfg, tokens: int, repeats: int = 3):
     import torch
+    from tuff_amd.csrc import ops
     from tuff_amd.engine.batch import StepEntry
     eng = llm.engine
     g = torch.Generator().manual_seed(SEED + 1)
     best = None
+    picked = torch.empty(1, dtype=torch.int32, device=eng.device)
     for i in range(repeats + 1):
         prompt = torch.randint(0, cfg.vocab_size, (tokens,), generator=g).tolist()
         eng.begin(("prefill", i))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         logits = eng.step([StepEntry(("prefill", i), prompt, [tokens - 1])])
-        nxt = int(torch.argmax(logits[0]))                # the first generated token reaches the host
+        ops.argmax(logits, picked)
+        nxt = int(picked.cpu()[0])                        # the first generated token reaches the host
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         eng.end(("prefill", i))
