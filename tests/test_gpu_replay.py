@@ -252,3 +252,48 @@ def test_layers_of_full_size_bfloat16_against_float32(gpu):
     top = torch.topk(outs["float32"], 2, dim=-1).values
     clear = (top[:, 0] - top[:, 1]) > 0.05 * float(outs["float32"].std())
     assert (outs["bfloat16"].argmax(-1) == outs["float32"].argmax(-1))[clear].all()
+
+
+def random_configuration(seed: int) -> dict:
+    """A small configuration whose every size and option is drawn from the seed."""
+    import random
+    rng = random.Random(seed)
+    heads = rng.choice([1, 2, 3, 4, 6, 8])
+    kv = rng.choice([h for h in range(1, heads + 1) if heads % h == 0])
+    hd = rng.choice([16, 24, 32, 40, 48, 64, 80, 128])
+    layers = rng.randint(2, 5)
+    types = [rng.choice(["conv", "full_attention"]) for _ in range(layers)]
+    types[rng.randrange(layers)] = "full_attention"
+    types[(types.index("full_attention") + 1) % layers] = "conv"
+    return dict(
+        architectures=["Lfm2ForCausalLM"], num_hidden_layers=layers, layer_types=types,
+        hidden_size=heads * hd, num_attention_heads=heads, num_key_value_heads=kv,
+        block_ff_dim=rng.choice([40, 72, 100, 136, 200, 333]), block_auto_adjust_ff_dim=False,
+        vocab_size=rng.randint(90, 1500), rope_theta=rng.choice([1e4, 5e5, 1e6]), conv_L_cache=rng.randint(2, 5),
+        norm_eps=rng.choice([1e-5, 1e-6, 3e-6]), tie_word_embeddings=rng.random() < 0.5, max_position_embeddings=512)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", [11, 12, 13, 14, 15])
+def test_configurations_drawn_at_random(gpu, tmp_path, seed, dtype):
+    """Configurations whose sizes nobody chose (head counts and sizes, groups, widths that are no
+    multiple of 8, vocabulary, conv length, layer order), under the mixed plan, against the plain
+    implementation."""
+    import random
+    from plain.lfm2_plain import forward_logits, read_model
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.models.registry import config_from_dict
+    from tuff_amd.weights.random_init import write_random_model
+    raw = random_configuration(seed)
+    stored = stored_for(dtype)
+    folder = str(tmp_path / "model")
+    write_random_model(config_from_dict(raw), folder, seed, getattr(torch, stored))
+    cfg, w = read_model(folder)
+    rng = random.Random(seed)
+    reqs = {f"q{i}": util.rand_tokens(rng.randint(3, 120), raw["vocab_size"], seed * 10 + i) for i in range(5)}
+    plan = util.plan_mixed(reqs, seed=seed)
+    eng = Engine.from_folder(folder, dtype=dtype, page_size=rng.choice([16, 32]), max_tokens=util.live_tokens_peak(plan) + 64)
+    got = util.run_plan(eng, plan)
+    eng.manager.check()
+    for rid, toks in reqs.items():
+        util.assert_close(dtype, got[rid], forward_logits(cfg, w, toks), f"seed {seed} {raw} {rid}")
