@@ -106,7 +106,14 @@ def loaded_modules() -> list[str]:
     return sorted(_libs)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """Handle of torch's current stream on the current device (the stream a graph is being
+    recorded on, inside a recording).  Called once a launch, so through the cheapest way there is."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -128,7 +135,7 @@ def _gpu(name: str, t: torch.Tensor, dtype=None, shape=None) -> int:
         raise KernelError(f"{name}: tensor must be contiguous (shape {tuple(t.shape)}, stride {t.stride()})")
     if dtype is not None and t.dtype != dtype:
         raise KernelError(f"{name}: expected {dtype}, got {t.dtype}")
-    if shape is not None:
+    if shape is not None and tuple(shape) != t.shape:        # torch.Size compares equal to a tuple
         if len(shape) != t.dim() or any(s is not None and s != g for s, g in zip(shape, t.shape)):
             raise KernelError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
     return t.data_ptr()

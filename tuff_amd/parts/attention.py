@@ -113,7 +113,8 @@ class AttentionMixer(Mixer):
         key = ("query_blocks", G, nb)
         blocks = ctx.host.get(key)
         if blocks is None:
-            blocks = torch.from_numpy(ops.query_blocks(ctx.host["q_len"], G, nb)).to(device)
+            # through pinned memory, so that the host does not wait for the stream
+            blocks = torch.from_numpy(ops.query_blocks(ctx.host["q_len"], G, nb)).pin_memory().to(device, non_blocking=True)
             ctx.host[key] = blocks
         return blocks
 
