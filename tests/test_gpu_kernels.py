@@ -39,6 +39,7 @@ def test_gemm_f32(gpu, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(1, 16, 8), (5, 1000, 96), (17, 33, 40), (64, 777, 240), (65, 130, 136),
                                    (200, 300, 328), (300, 64, 2048), (128, 128, 64), (2, 2048, 8192),
+                                   (72, 2048, 8192), (512, 2050, 2048), (130, 1026, 1000),
                                    (33, 100, 2048), (64, 2048, 8192), (20, 64, 1024), (48, 200, 512), (16, 24, 4096),
                                    (8, 6144, 2048),
                                    # each shape of block of the tiled kernel, with ragged edges and a partial last step
@@ -71,6 +72,7 @@ def test_gemm_bf16(gpu, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(1, 32, 64), (8, 512, 240), (16, 6144, 2048), (5, 200, 96), (64, 384, 256),
                                    (40, 2050, 2048), (300, 130, 136), (2048, 512, 128), (1100, 8200, 72),
+                                   (200, 384, 1024), (72, 4100, 2048),
                                    (1030, 8202, 136), (1100, 4002, 200)])
 def test_gemm_bf16_swiglu_epilogue(gpu, M, N, K):
     """Rows of w are gate and up rows interleaved; the output is silu(gate) * up."""

@@ -118,7 +118,8 @@ __device__ __forceinline__ void store_quad(void* Y, long long row, long long col
 
 template <int TM, int TN, int WAVES_M, int WAVES_N, int AHEAD, int MODE>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_tiled_kernel(
-        const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, int M, int N, int K) {
+        const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, int M, int N, int K,
+        int steps_per_slice, float* __restrict__ ws) {
     constexpr int NT = 64 * WAVES_M * WAVES_N;
     constexpr int BM = 16 * TM * WAVES_M, BN = 16 * TN * WAVES_N;
     constexpr int PA = BM * CHUNKS / NT, PB = BN * CHUNKS / NT;     // 16-byte pieces of X and of W a thread moves a step
@@ -162,7 +163,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_tiled_kernel
     // Memory answers later than a step lasts, so the operands of AHEAD steps are on their way at
     // any time, each in a register set of its own; a set is free again once it went into LDS.
     bf16x8 ra[AHEAD][PA], rb[AHEAD][PB];
+    // gridDim.z > 1: the block walks only its slice of K and leaves a float32 partial block in the work
+    // space, ws[slice][row][col]; splitk_finish_kernel adds the slices and does the epilogue.
     const int nk = (K + TBK - 1) / TBK;
+    const int kt_begin = blockIdx.z * steps_per_slice, kt_end = min(nk, kt_begin + steps_per_slice);
 
     auto load_global = [&](auto set_tag, int kt) {
         constexpr int set = decltype(set_tag)::value;
@@ -224,22 +228,31 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_tiled_kernel
     };
 
     // set s holds step s, later step s + AHEAD, ...; step kt + 1 is filled in while step kt is multiplied
-    static_for<AHEAD>([&](auto s) { load_global(s, decltype(s)::value); });
+    static_for<AHEAD>([&](auto s) { load_global(s, kt_begin + decltype(s)::value); });
 #pragma unroll
     for (int p = 0; p < PA + PB; ++p) store_piece(std::integral_constant<int, 0>(), 0, p);
     __syncthreads();
-    for (int kt0 = 0; kt0 < nk; kt0 += AHEAD) {
+    for (int kt0 = kt_begin; kt0 < kt_end; kt0 += AHEAD) {
         static_for<AHEAD>([&](auto u) {
             constexpr int set = decltype(u)::value;
             const int kt = kt0 + set;
-            if (kt < nk) {
+            if (kt < kt_end) {
                 load_global(u, kt + AHEAD);
-                multiply(kt & 1, std::integral_constant<int, (set + 1) % AHEAD>());
+                multiply((kt - kt_begin) & 1, std::integral_constant<int, (set + 1) % AHEAD>());
                 __syncthreads();
             }
         });
     }
 
+    if (gridDim.z > 1) {
+        float* mine = ws + (long long)blockIdx.z * M * N;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                store_quad<OUT_F32>(mine, m0 + wm + i * 16 + r16, n0 + wn + j * 16 + g * 4, M, N, acc[i][j]);
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -676,6 +689,27 @@ SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16, bool emit = fals
     return p;
 }
 
+// How a product of more than 64 rows is cut: shape 0: 256 x 256 blocks; 1: 128 x 128 blocks, two a CU;
+// 2: 128 x 128 blocks, one a CU, four register sets.  Depends on the sizes only.
+struct TiledPlan { int shape, slices, steps_per_slice; long long ws_floats; };
+
+TiledPlan plan_tiled(int M, int N, int K) {
+    const long long large = (long long)ceil_div(N, 256) * ceil_div(M, 256);
+    const long long small = (long long)ceil_div(N, 128) * ceil_div(M, 128);
+    const int nk = ceil_div(K, TBK);
+    TiledPlan t;
+    t.shape = large >= 160 ? 0 : small > 256 ? 1 : 2;
+    t.slices = 1; t.steps_per_slice = nk; t.ws_floats = 0;
+    if (t.shape == 2 && small <= 128) {
+        // as many slices as give every CU at most one block, at least eight steps a slice
+        int s = max(1, min((int)(256 / small), nk / 8));
+        t.steps_per_slice = ceil_div(nk, s);
+        t.slices = ceil_div(nk, t.steps_per_slice);
+        if (t.slices > 1) t.ws_floats = (long long)t.slices * M * N;
+    }
+    return t;
+}
+
 struct Skinny16Extra {
     const float* norm_w = nullptr; float eps = 0.f; const int* rows = nullptr;       // NORM_INSIDE
     const float* ss_in = nullptr; int n_ss = 0;                                      // NORM_SCALED (+ eps)
@@ -758,9 +792,10 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
     } else {
         // Large blocks where they give most CUs one.  Of the small ones a CU holds two if there are
         // enough; if not, a block is alone on its CU and hides the memory's latency by itself, with
-        // the operands of four steps under way.
-        const long long large = (long long)ceil_div(N, 256) * ceil_div(M, 256);
-        const long long small = (long long)ceil_div(N, 128) * ceil_div(M, 128);
+        // the operands of four steps under way.  Where even the small blocks are fewer than half the
+        // CUs (few rows, narrow output), K is cut into slices, a block a slice.
+        const TiledPlan t = plan_tiled(M, N, K);
+        if (t.slices > 1 && !ws) return -4;
 #define TILED(TM, TN, WM, WN, AHEAD) do { \
             auto kern = gemm_bf16_tiled_kernel<TM, TN, WM, WN, AHEAD, MODE>; \
             constexpr int bm = 16 * TM * WM, bn = 16 * TN * WN, lds = 2 * (bm + bn) * TBK * 2; \
@@ -769,12 +804,19 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
                 if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -1; \
                 set = true; \
             } \
-            hipLaunchKernelGGL(kern, dim3(ceil_div(N, bn), ceil_div(M, bm)), dim3(64 * WM * WN), lds, stream, X, W, Y, M, N, K); \
+            hipLaunchKernelGGL(kern, dim3(ceil_div(N, bn), ceil_div(M, bm), t.slices), dim3(64 * WM * WN), lds, stream, \
+                               X, W, Y, M, N, K, t.steps_per_slice, ws); \
         } while (0)
-        if (large >= 160) TILED(8, 4, 2, 4, 1);
-        else if (small > 256) TILED(4, 2, 2, 4, 1);
+        if (t.shape == 0) TILED(8, 4, 2, 4, 1);
+        else if (t.shape == 1) TILED(4, 2, 2, 4, 1);
         else TILED(4, 2, 2, 4, 4);
 #undef TILED
+        if (t.slices > 1) {
+            int rc = launch_status();
+            if (rc) return rc;
+            hipLaunchKernelGGL((splitk_finish_kernel<MODE, NORM_NONE, false>), dim3(ceil_div(N, 64), ceil_div(M, 16)), dim3(256), 0,
+                               stream, (const float*)ws, Y, M, N, M, t.slices, FinishExtra());
+        }
     }
     return launch_status();
 }
@@ -793,8 +835,8 @@ TUFF_EXPORT int tuff_gemm_bf16_emit_layout(int M, int N, int K, int* tiles, int*
 // emit: for tuff_gemm_bf16_accum_emit.
 TUFF_EXPORT int tuff_gemm_bf16_workspace(int M, int N, int K, int emit, long long* ws_floats) {
     *ws_floats = 0;
-    if (M > 64 || M <= 16 || N <= 0) return 0;
-    *ws_floats = plan_skinny(M, N, K, 16, emit != 0).ws_floats;
+    if (M <= 16 || N <= 0) return 0;
+    *ws_floats = M <= 64 ? plan_skinny(M, N, K, 16, emit != 0).ws_floats : plan_tiled(M, N, K).ws_floats;
     return 0;
 }
 

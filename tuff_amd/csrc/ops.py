@@ -372,7 +372,7 @@ _plans: dict = {}
 def _gemm_workspace(M: int, N: int, K: int, device, emit: bool = False) -> Optional[torch.Tensor]:
     """The float32 work space a bfloat16 product of this shape needs, or None.  Taken anew for every
     call: the allocator hands the same block out again."""
-    if M <= 16 or M > 64:
+    if M <= 16:
         return None
     key = (M, N, K, emit)
     n = _plans.get(key)
