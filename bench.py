@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """Serving benchmark on one MI355X: decode tokens a second of the LFM2.5-1.2B shape with random
-weights (BASELINE.json configs[2]), plus the 2,048-token prefill and decode at batch 1 and 64.
+weights (16 layers, 6 of them attention; hidden 2048), plus the 2,048-token prefill and decode at batch 1 and 64.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
 
@@ -21,7 +21,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0                                   # MI355X HBM3E, published
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}           # dense MFMA, published
 
-# BASELINE.json configs[2]: LFM2.5-1.2B shape
+# the config.json of the LFM2.5-1.2B shape
 SHAPE = dict(
     architectures=["Lfm2ForCausalLM"], num_hidden_layers=16, full_attn_idxs=[2, 5, 8, 10, 12, 14],
     hidden_size=2048, num_attention_heads=32, num_key_value_heads=8, block_ff_dim=12288,
