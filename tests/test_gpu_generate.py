@@ -243,3 +243,37 @@ def test_command_line_jobs(gpu, tmp_path):
     assert (tmp_path / "e0").read_text().strip().endswith("JOB_EXIT=0")
     assert "reusing the loaded model" in (tmp_path / "e3").read_text()
     assert "TUFF_TEST_MARK" not in os.environ
+
+
+@pytest.mark.parametrize("name,seed", [("A", 3), ("B", 7), ("C", 18)])
+def test_scheduler_scenarios_drawn_at_random(gpu, name, seed):
+    """Requests, options, pool size, budget and slots drawn from a seed (greedy and seeded draws,
+    repetition penalty, end tokens on and off, pools small enough to preempt, starting steps early
+    on and off): in float32 every request generates what it generates alone."""
+    import random
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.engine.llm import LLM
+    from tuff_amd.sampling.params import SamplingParams
+    V = util.CONFIGS[name][0]["vocab_size"]
+    folder = util.model_folder(name, "float32")
+    alone = LLM(engine=Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=256, max_requests=2),
+                max_num_seqs=1, ctx_size=400)
+    rng = random.Random(seed)
+    n = rng.randint(3, 12)
+    prompts = [util.rand_tokens(rng.randint(2, 90), V, seed * 100 + i) for i in range(n)]
+    params = [SamplingParams(max_new_tokens=rng.randint(1, 40), ignore_eos=rng.random() < 0.7,
+                             temp=rng.choice([0.0, 0.0, 0.8]), top_k=rng.choice([0, 20]), seed=rng.randint(1, 99),
+                             repeat_penalty=rng.choice([1.0, 1.0, 1.2])) for _ in range(n)]
+    pages = rng.randint(9, 30)
+    llm = LLM(engine=Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=pages, max_requests=rng.randint(2, 5)),
+              max_num_seqs=rng.randint(2, 5), max_batched_tokens=rng.choice([16, 48, 200]), ctx_size=400,
+              run_ahead=rng.random() < 0.7)
+    got = llm.generate(prompts, params)
+    llm.engine.manager.check()
+    assert not llm.engine.manager.live()
+    for i, (p, sp, g) in enumerate(zip(prompts, params, got)):
+        if g.finish_reason == "capacity":
+            assert -(-(len(p) + sp.max_new_tokens) // 16) > pages
+            continue
+        want = alone.generate([p], sp)[0]
+        assert (g.token_ids, g.finish_reason) == (want.token_ids, want.finish_reason), (seed, i, g.preemptions)
