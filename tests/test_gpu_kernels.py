@@ -272,6 +272,62 @@ def test_qkv_post(gpu, H, Hkv, hd, ps, dt):
     assert (k2.cpu().double().reshape(T, Hkv, hd) - wantk).abs().max() <= tol * float(wantk.abs().max())
 
 
+@pytest.mark.parametrize("ps", [16, 32, 64])
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_qkv_post_heads_of_64(gpu, dt, ps):
+    """The kernel for heads of 64 channels: sixteen lanes a token, v rows of sixteen tokens written in
+    runs.  Slots as a prompt gives them (runs of whole pages from a page's start), runs that begin in
+    the middle of a page, scattered slots, a last group of fewer than sixteen tokens, slots that are
+    not to be written; against the plain formulas, and bit for bit against the same tokens in steps
+    of 1, 5 and 16."""
+    from tuff_amd.csrc import ops
+    H, Hkv, hd, eps, base = 6, 3, 64, 1e-6, 1000000.0
+    T = 16 * 7 + 5
+    qkv = _r(T, (H + 2 * Hkv) * hd, seed=21, dtype=dt)
+    qw, kw = 1 + _r(hd, seed=22, scale=0.1), 1 + _r(hd, seed=23, scale=0.1)
+    pos = (torch.arange(T, dtype=torch.int32) * 3 + 2) % 1500
+    n_pages = 40
+    slots = torch.empty(T, dtype=torch.int64)
+    slots[0:32] = torch.arange(32) + 5 * ps                 # two whole groups from a page's start
+    slots[32:48] = torch.arange(16) + 9 * ps + 8             # a run that begins in the middle of a page
+    slots[48:64] = torch.randperm(16, generator=torch.Generator().manual_seed(2)) + 11 * ps   # one page, shuffled
+    slots[64:112] = torch.arange(48) + 20 * ps               # pages in a row
+    slots[112:] = torch.arange(5) + 30 * ps                  # the last, short group
+    write = torch.ones(T, dtype=torch.bool)
+    write[70] = False
+    slot_arg = torch.where(write, slots, torch.full_like(slots, -1)).to(torch.int32)
+    inv_freq = (base ** (-2 * torch.arange(hd // 2, dtype=torch.float64) / hd)).float()
+    dev = lambda x: x.to(gpu)
+
+    def run(step):
+        kc = torch.zeros(n_pages, Hkv, ps, hd, dtype=dt, device=gpu)
+        vc = torch.zeros(n_pages, Hkv, hd, ps, dtype=dt, device=gpu)
+        q = torch.empty(T, H * hd, dtype=dt, device=gpu)
+        for a in range(0, T, step):
+            b = min(T, a + step)
+            ops.qkv_post(dev(qkv[a:b]), q[a:b], H=H, Hkv=Hkv, hd=hd, positions=dev(pos[a:b]), eps=eps, q_norm_w=dev(qw),
+                         k_norm_w=dev(kw), inv_freq=dev(inv_freq), rotary_dim=hd, k_cache=kc, v_cache=vc,
+                         slot_mapping=dev(slot_arg[a:b]), page_size=ps)
+        return q, kc, vc
+    q, kc, vc = run(T)
+    x = qkv.double()
+    qs, ks, vs = x[:, :H * hd].reshape(T, H, hd), x[:, H * hd:(H + Hkv) * hd].reshape(T, Hkv, hd), x[:, (H + Hkv) * hd:].reshape(T, Hkv, hd)
+    want_q = plain.rope_neox(plain.rms_norm(qs, qw.double(), eps), pos, base)
+    want_k = plain.rope_neox(plain.rms_norm(ks, kw.double(), eps), pos, base)
+    tol = 2e-4 if dt == torch.float32 else 2 ** -7
+    assert (q.cpu().double().reshape(T, H, hd) - want_q).abs().max() <= tol * float(want_q.abs().max())
+    flat_k = kc.cpu().double().permute(0, 2, 1, 3).reshape(n_pages * ps, Hkv, hd)
+    flat_v = vc.cpu().double().permute(0, 3, 1, 2).reshape(n_pages * ps, Hkv, hd)
+    assert (flat_k[slots[write]] - want_k[write]).abs().max() <= tol * float(want_k.abs().max())
+    assert torch.equal(flat_v[slots[write]], vs[write])
+    untouched = torch.ones(n_pages * ps, dtype=torch.bool)
+    untouched[slots[write]] = False
+    assert (flat_k[untouched] == 0).all() and (flat_v[untouched] == 0).all()
+    for step in (1, 5, 16):
+        q2, k2, v2 = run(step)
+        assert torch.equal(q, q2) and torch.equal(kc, k2) and torch.equal(vc, v2), f"steps of {step} differ"
+
+
 def test_qkv_post_many_tokens_equal_few(gpu):
     """With many tokens a wave takes several heads of a token in turn; the result is, bit for
     bit, that of the same tokens in small steps."""

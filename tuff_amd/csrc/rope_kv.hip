@@ -14,6 +14,25 @@
 namespace {
 constexpr int MAX_PER_LANE = 4;            // head sizes up to 256
 
+// Four neighbouring elements as float32, and back (8 bytes of bfloat16 or 16 of float32 at once).
+__device__ __forceinline__ void load4(const bf16_t* p, float (&v)[4]) {
+    const bf16x4 t = *(const bf16x4*)p;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = (float)t[e];
+}
+__device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
+    const f32x4 t = *(const f32x4*)p;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = t[e];
+}
+__device__ __forceinline__ void store4(bf16_t* p, const float (&v)[4]) {
+    bf16x4 t = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+    *(bf16x4*)p = t;
+}
+__device__ __forceinline__ void store4(float* p, const float (&v)[4]) {
+    *(f32x4*)p = f32x4{v[0], v[1], v[2], v[3]};
+}
+
 // A workgroup of four waves takes one token; wave w the heads_per_wave heads from
 // (blockIdx.y * 4 + w) * heads_per_wave on (q heads, then k heads, then v heads).  The angles of a
 // token are the same for all its heads and are computed once a wave.
@@ -122,6 +141,124 @@ __global__ __launch_bounds__(POST_WAVES * WAVE) void qkv_post_kernel(
     }
 }
 
+// The same for heads of 64 channels with the half-split rotation over the whole head, laid out for
+// many tokens.  Two kinds of workgroups in one launch:
+//  * q and k: sixteen lanes take one token and walk a share of its heads; lane l holds the channels
+//    4l .. 4l+3 of a head (one 8-byte load for bfloat16), the norm's sum of squares is a butterfly over
+//    the sixteen lanes, the rotation's partner channel j +- 32 sits in lane l ^ 8, and the token's
+//    cosines and sines are computed once for all its heads.
+//  * v: a workgroup takes sixteen consecutive tokens, brings their v rows into LDS and writes, for
+//    every (kv head, channel), the sixteen positions in one run where the tokens fill a run of sixteen
+//    slots from a multiple of sixteen (the usual case in a prompt), else one by one: V is kept with a
+//    channel's positions contiguous, and a token alone can only write it two bytes at a time.
+// Whatever the number of tokens in the step, a token's values go through the same arithmetic.
+constexpr int P64_GROUPS = 16;                       // sixteen-lane groups a workgroup
+constexpr int P64_TOKENS = 16;                       // tokens a v workgroup
+
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void qkv_post64_kernel(
+    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const TW* __restrict__ q_norm_w, const TW* __restrict__ k_norm_w, float eps, const float* __restrict__ inv_freq,
+    const int* __restrict__ positions, const int* __restrict__ slot_mapping,
+    int n_tokens, int H, int Hkv, int page_size, int shares, int qk_blocks) {
+    constexpr int HD = 64;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const int tid = threadIdx.x;
+    const int row_width = (H + 2 * Hkv) * HD;
+    if ((int)blockIdx.x < qk_blocks) {
+        const int l = tid % 16, grp = tid / 16;
+        const long long item = (long long)blockIdx.x * P64_GROUPS + grp;      // (token, share of its heads)
+        const int t = (int)(item / shares), share = (int)(item % shares);
+        if (t >= n_tokens) return;
+        const int n_heads = k_cache ? H + Hkv : H;
+        const int per = (n_heads + shares - 1) / shares;
+        const int head_begin = share * per, head_end = min(n_heads, head_begin + per);
+        const float pos = (float)positions[t];
+        const bool first = l < 8;
+        float rc[4], rs[4], wq[4], wk[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float a = pos * inv_freq[(4 * l + e) & 31];
+            rc[e] = cosf(a);
+            rs[e] = sinf(a);
+            wq[e] = q_norm_w ? to_f32(q_norm_w[4 * l + e]) : 1.f;
+            wk[e] = k_norm_w ? to_f32(k_norm_w[4 * l + e]) : 1.f;
+        }
+        long long slot = -1;
+        if (k_cache) slot = slot_mapping[t];
+        const T* row = qkv + (long long)t * row_width + 4 * l;
+        for (int head = head_begin; head < head_end; ++head) {
+            const bool is_q = head < H;
+            float v[4];
+            load4(row + (long long)head * HD, v);
+            float ss = v[0] * v[0];
+            ss = fmaf(v[1], v[1], ss);
+            ss = fmaf(v[2], v[2], ss);
+            ss = fmaf(v[3], v[3], ss);
+            ss += __shfl_xor(ss, 8, WAVE);
+            ss += __shfl_xor(ss, 4, WAVE);
+            ss += __shfl_xor(ss, 2, WAVE);
+            ss += __shfl_xor(ss, 1, WAVE);
+            if (is_q ? q_norm_w != nullptr : k_norm_w != nullptr) {
+                const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * inv * (is_q ? wq[e] : wk[e]);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float other = __shfl_xor(v[e], 8, WAVE);
+                const float x0 = first ? v[e] : other, x1 = first ? other : v[e];
+                v[e] = first ? (x0 * rc[e] - x1 * rs[e]) : (x0 * rs[e] + x1 * rc[e]);
+            }
+            if (is_q) store4(q_out + ((long long)t * H + head) * HD + 4 * l, v);
+            else if (slot >= 0) {
+                const long long page = slot / page_size, off = slot % page_size;
+                store4(k_cache + ((page * Hkv + (head - H)) * page_size + off) * HD + 4 * l, v);
+            }
+        }
+        return;
+    }
+    // v: tokens t0 .. t0 + 15
+    T* vt = (T*)lds_raw;                                   // [16 tokens][Hkv * 64]
+    const int t0 = ((int)blockIdx.x - qk_blocks) * P64_TOKENS;
+    const int width = Hkv * HD, n_here = min(P64_TOKENS, n_tokens - t0);
+    for (int p = tid * 4; p < P64_TOKENS * width; p += 256 * 4) {
+        const int i = p / width, c = p % width;
+        if (i < n_here) {
+            float x[4];
+            load4(qkv + (long long)(t0 + i) * row_width + (long long)(H + Hkv) * HD + c, x);
+            store4(vt + p, x);
+        }
+    }
+    __shared__ int slots[P64_TOKENS];
+    if (tid < P64_TOKENS) slots[tid] = tid < n_here ? slot_mapping[t0 + tid] : -1;
+    __syncthreads();
+    const int s0 = slots[0];
+    bool run = n_here == P64_TOKENS && s0 >= 0 && s0 % 16 == 0;
+#pragma unroll
+    for (int i = 1; i < P64_TOKENS; ++i) run = run && slots[i] == s0 + i;
+    for (int p = tid; p < width; p += 256) {               // p = kv head * 64 + channel
+        const int kvh = p / HD, ch = p % HD;
+        if (run) {
+            const long long page = s0 / page_size, off = s0 % page_size;
+            T* dst = v_cache + ((page * Hkv + kvh) * HD + ch) * page_size + off;
+            T vals[P64_TOKENS];
+#pragma unroll
+            for (int i = 0; i < P64_TOKENS; ++i) vals[i] = vt[i * width + p];
+            constexpr int PIECES = P64_TOKENS * (int)sizeof(T) / 16;
+#pragma unroll
+            for (int q = 0; q < PIECES; ++q) ((uint4*)dst)[q] = ((const uint4*)vals)[q];
+        } else {
+            for (int i = 0; i < n_here; ++i) {
+                const long long slot = slots[i];
+                if (slot < 0) continue;
+                const long long page = slot / page_size, off = slot % page_size;
+                v_cache[((page * Hkv + kvh) * HD + ch) * page_size + off] = vt[i * width + p];
+            }
+        }
+    }
+}
+
 // Copies already encoded k and v rows [T, Hkv, hd] into the paged cache.
 template <typename T>
 __global__ __launch_bounds__(WAVE) void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v,
@@ -151,6 +288,27 @@ TUFF_EXPORT int tuff_qkv_post(const void* qkv, void* q_out, void* k_out, void* k
                               int n_tokens, int H, int Hkv, int hd, int page_size, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (hd > MAX_PER_LANE * WAVE || rotary_dim > hd || (rotary_dim % 2) != 0) return -2;
+    if (hd == 64 && inv_freq && rotary_dim == 64 && !interleaved && !k_out && page_size % 16 == 0) {
+        // shares of a token's heads: enough sixteen-lane groups for the chip, whole heads each
+        const int n_heads = k_cache ? H + Hkv : H;
+        int shares = 1;
+        while (shares < n_heads && (long long)n_tokens * shares < 8192) shares *= 2;
+        shares = min(shares, n_heads);
+        const int qk_blocks = (int)ceil_div_ll((long long)n_tokens * shares, P64_GROUPS);
+        const int v_blocks = k_cache ? ceil_div(n_tokens, P64_TOKENS) : 0;
+        const size_t esize = dt == DT_F32 ? 4 : 2;
+        const size_t lds = k_cache ? (size_t)P64_TOKENS * Hkv * 64 * esize : 0;
+        if (lds > 64 * 1024) return -2;
+#define LAUNCH64(T, TW) hipLaunchKernelGGL((qkv_post64_kernel<T, TW>), dim3(qk_blocks + v_blocks), dim3(256), lds, stream, \
+        (const T*)qkv, (T*)q_out, (T*)k_cache, (T*)v_cache, (const TW*)q_norm_w, (const TW*)k_norm_w, eps, inv_freq, \
+        positions, slot_mapping, n_tokens, H, Hkv, page_size, shares, qk_blocks)
+        if (dt == DT_F32 && norm_dt == DT_F32) LAUNCH64(float, float);
+        else if (dt == DT_F32) LAUNCH64(float, bf16_t);
+        else if (norm_dt == DT_F32) LAUNCH64(bf16_t, float);
+        else LAUNCH64(bf16_t, bf16_t);
+#undef LAUNCH64
+        return launch_status();
+    }
     const int heads = k_cache ? H + 2 * Hkv : (k_out ? H + Hkv : H);
     // few tokens: a wave a head; many: several heads a wave, so that workgroups stay in the thousands
     const long long waves = (long long)n_tokens * heads;
