@@ -147,8 +147,8 @@ __global__ __launch_bounds__(POST_WAVES * WAVE) void qkv_post_kernel(
 //    4l .. 4l+3 of a head (one 8-byte load for bfloat16), the norm's sum of squares is a butterfly over
 //    the sixteen lanes, the rotation's partner channel j +- 32 sits in lane l ^ 8, and the token's
 //    cosines and sines are computed once for all its heads.
-//  * v: a workgroup takes sixteen consecutive tokens, brings their v rows into LDS and writes, for
-//    every (kv head, channel), the sixteen positions in one run where the tokens fill a run of sixteen
+//  * v: a workgroup takes sixteen consecutive tokens and one kv head, brings the rows into LDS and
+//    writes, for every channel, the sixteen positions in one run where the tokens fill a run of sixteen
 //    slots from a multiple of sixteen (the usual case in a prompt), else one by one: V is kept with a
 //    channel's positions contiguous, and a token alone can only write it two bytes at a time.
 // Whatever the number of tokens in the step, a token's values go through the same arithmetic.
@@ -162,7 +162,6 @@ __global__ __launch_bounds__(256) void qkv_post64_kernel(
     const int* __restrict__ positions, const int* __restrict__ slot_mapping,
     int n_tokens, int H, int Hkv, int page_size, int shares, int qk_blocks) {
     constexpr int HD = 64;
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const int tid = threadIdx.x;
     const int row_width = (H + 2 * Hkv) * HD;
     if ((int)blockIdx.x < qk_blocks) {
@@ -218,43 +217,44 @@ __global__ __launch_bounds__(256) void qkv_post64_kernel(
         }
         return;
     }
-    // v: tokens t0 .. t0 + 15
-    T* vt = (T*)lds_raw;                                   // [16 tokens][Hkv * 64]
-    const int t0 = ((int)blockIdx.x - qk_blocks) * P64_TOKENS;
-    const int width = Hkv * HD, n_here = min(P64_TOKENS, n_tokens - t0);
-    for (int p = tid * 4; p < P64_TOKENS * width; p += 256 * 4) {
-        const int i = p / width, c = p % width;
+    // v: tokens t0 .. t0 + 15 of one kv head
+    __shared__ __attribute__((aligned(16))) T vt[P64_TOKENS][HD];
+    __shared__ int slots[P64_TOKENS];
+    const int vb = (int)blockIdx.x - qk_blocks;
+    const int t0 = (vb / Hkv) * P64_TOKENS, kvh = vb % Hkv;
+    const int n_here = min(P64_TOKENS, n_tokens - t0);
+    {
+        const int i = tid / 16, c = (tid % 16) * 4;          // 16 tokens x 16 pieces of four channels
         if (i < n_here) {
             float x[4];
-            load4(qkv + (long long)(t0 + i) * row_width + (long long)(H + Hkv) * HD + c, x);
-            store4(vt + p, x);
+            load4(qkv + (long long)(t0 + i) * row_width + (long long)(H + Hkv + kvh) * HD + c, x);
+            store4(&vt[i][c], x);
         }
     }
-    __shared__ int slots[P64_TOKENS];
     if (tid < P64_TOKENS) slots[tid] = tid < n_here ? slot_mapping[t0 + tid] : -1;
     __syncthreads();
     const int s0 = slots[0];
     bool run = n_here == P64_TOKENS && s0 >= 0 && s0 % 16 == 0;
 #pragma unroll
     for (int i = 1; i < P64_TOKENS; ++i) run = run && slots[i] == s0 + i;
-    for (int p = tid; p < width; p += 256) {               // p = kv head * 64 + channel
-        const int kvh = p / HD, ch = p % HD;
-        if (run) {
+    if (run) {
+        if (tid < HD) {                                      // a channel a thread: its sixteen positions in one run
             const long long page = s0 / page_size, off = s0 % page_size;
-            T* dst = v_cache + ((page * Hkv + kvh) * HD + ch) * page_size + off;
+            T* dst = v_cache + ((page * Hkv + kvh) * HD + tid) * page_size + off;
             T vals[P64_TOKENS];
 #pragma unroll
-            for (int i = 0; i < P64_TOKENS; ++i) vals[i] = vt[i * width + p];
+            for (int i = 0; i < P64_TOKENS; ++i) vals[i] = vt[i][tid];
             constexpr int PIECES = P64_TOKENS * (int)sizeof(T) / 16;
 #pragma unroll
             for (int q = 0; q < PIECES; ++q) ((uint4*)dst)[q] = ((const uint4*)vals)[q];
-        } else {
-            for (int i = 0; i < n_here; ++i) {
-                const long long slot = slots[i];
-                if (slot < 0) continue;
-                const long long page = slot / page_size, off = slot % page_size;
-                v_cache[((page * Hkv + kvh) * HD + ch) * page_size + off] = vt[i * width + p];
-            }
+        }
+    } else {
+        const int ch = tid % HD;
+        for (int i = tid / HD; i < n_here; i += 256 / HD) {
+            const long long slot = slots[i];
+            if (slot < 0) continue;
+            const long long page = slot / page_size, off = slot % page_size;
+            v_cache[((page * Hkv + kvh) * HD + ch) * page_size + off] = vt[i][ch];
         }
     }
 }
@@ -295,11 +295,8 @@ TUFF_EXPORT int tuff_qkv_post(const void* qkv, void* q_out, void* k_out, void* k
         while (shares < n_heads && (long long)n_tokens * shares < 8192) shares *= 2;
         shares = min(shares, n_heads);
         const int qk_blocks = (int)ceil_div_ll((long long)n_tokens * shares, P64_GROUPS);
-        const int v_blocks = k_cache ? ceil_div(n_tokens, P64_TOKENS) : 0;
-        const size_t esize = dt == DT_F32 ? 4 : 2;
-        const size_t lds = k_cache ? (size_t)P64_TOKENS * Hkv * 64 * esize : 0;
-        if (lds > 64 * 1024) return -2;
-#define LAUNCH64(T, TW) hipLaunchKernelGGL((qkv_post64_kernel<T, TW>), dim3(qk_blocks + v_blocks), dim3(256), lds, stream, \
+        const int v_blocks = k_cache ? ceil_div(n_tokens, P64_TOKENS) * Hkv : 0;
+#define LAUNCH64(T, TW) hipLaunchKernelGGL((qkv_post64_kernel<T, TW>), dim3(qk_blocks + v_blocks), dim3(256), 0, stream, \
         (const T*)qkv, (T*)q_out, (T*)k_cache, (T*)v_cache, (const TW*)q_norm_w, (const TW*)k_norm_w, eps, inv_freq, \
         positions, slot_mapping, n_tokens, H, Hkv, page_size, shares, qk_blocks)
         if (dt == DT_F32 && norm_dt == DT_F32) LAUNCH64(float, float);
