@@ -30,27 +30,50 @@ TUFF_EXPORT int tuff_embed_rows(const void* table, int table_dt, const int* toke
 // -------------------------------------------------------------------- RMSNorm
 // y_i = x_i * (1 / sqrt(mean_j x_j^2 + eps)) * w_i   (src/lfm25_gpu.cu:235,244).
 // `rows` (optional) gathers input rows: output row r is the norm of x[rows[r]].
-// Per-thread strided partial sums -> wave butterfly -> wave partials in order.
-template <typename TW, typename TO>
-__global__ void rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ w,
-                               TO* __restrict__ out, const int* __restrict__ rows, int d, float eps) {
+// Per-thread strided partial sums -> wave butterfly -> wave partials in order; which elements a
+// thread takes depends on d alone (multiples of 4: four neighbours a step).
+template <typename TW, typename TO, bool VEC>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ w,
+                                                      TO* __restrict__ out, const int* __restrict__ rows, int d, float eps) {
     __shared__ float scratch[4];
     const int r = blockIdx.x;
     const long long src = rows ? rows[r] : r;
     const float* xr = x + src * (long long)d;
+    TO* o = out + (long long)r * d;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < d; i += 256) { const float v = xr[i]; ss += v * v; }
+    if (VEC) {
+        // d is a multiple of 4: four neighbouring elements a thread and step, 16-byte loads
+        for (int i = threadIdx.x * 4; i < d; i += 1024) {
+            const f32x4 v = *(const f32x4*)(xr + i);
+            ss = fmaf(v[0], v[0], ss); ss = fmaf(v[1], v[1], ss); ss = fmaf(v[2], v[2], ss); ss = fmaf(v[3], v[3], ss);
+        }
+    } else {
+        for (int i = threadIdx.x; i < d; i += 256) { const float v = xr[i]; ss += v * v; }
+    }
     const float total = block_sum<4>(ss, scratch);
     const float inv = 1.0f / sqrtf(total / (float)d + eps);
-    TO* o = out + (long long)r * d;
-    for (int i = threadIdx.x; i < d; i += 256) o[i] = from_f32<TO>(xr[i] * inv * to_f32(w[i]));
+    if (VEC) {
+        for (int i = threadIdx.x * 4; i < d; i += 1024) {
+            const f32x4 v = *(const f32x4*)(xr + i);
+            TO y[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) y[e] = from_f32<TO>(v[e] * inv * to_f32(w[i + e]));
+            if (sizeof(TO) == 2) *(uint2*)(o + i) = *(const uint2*)y;
+            else *(uint4*)(o + i) = *(const uint4*)y;
+        }
+    } else {
+        for (int i = threadIdx.x; i < d; i += 256) o[i] = from_f32<TO>(xr[i] * inv * to_f32(w[i]));
+    }
 }
 
 TUFF_EXPORT int tuff_rmsnorm(const float* x, const void* w, int w_dt, void* out, int out_dt,
                              const int* rows, int n_rows, int d, float eps, hipStream_t stream) {
     if (n_rows <= 0) return 0;
     dim3 grid(n_rows), block(256);
-#define LAUNCH(TW, TO) hipLaunchKernelGGL((rmsnorm_kernel<TW, TO>), grid, block, 0, stream, x, (const TW*)w, (TO*)out, rows, d, eps)
+#define LAUNCH(TW, TO) do { \
+        if (d % 4 == 0) hipLaunchKernelGGL((rmsnorm_kernel<TW, TO, true>), grid, block, 0, stream, x, (const TW*)w, (TO*)out, rows, d, eps); \
+        else hipLaunchKernelGGL((rmsnorm_kernel<TW, TO, false>), grid, block, 0, stream, x, (const TW*)w, (TO*)out, rows, d, eps); \
+    } while (0)
     if (w_dt == DT_F32 && out_dt == DT_F32) LAUNCH(float, float);
     else if (w_dt == DT_F32 && out_dt == DT_BF16) LAUNCH(float, bf16_t);
     else if (w_dt == DT_BF16 && out_dt == DT_F32) LAUNCH(bf16_t, float);
