@@ -51,11 +51,12 @@ __global__ void shortconv_fwd_kernel(const T* __restrict__ bcx, const TW* __rest
 
 // The same for bfloat16 activations, eight channels a thread (16-byte loads and stores); d must
 // be a multiple of 8.  Every channel goes through the chain of operations of the kernel above.
-template <typename TW>
+template <typename TW, int KT>                    // KT: the kernel length if it is 2, 3 or 4, else 0 (read K)
 __global__ void shortconv_fwd_vec_kernel(const bf16_t* __restrict__ bcx, const TW* __restrict__ conv_w,
                                          const float* __restrict__ state, bf16_t* __restrict__ out,
                                          const int* __restrict__ req_of_token, const int* __restrict__ q_start,
-                                         const int* __restrict__ state_slot, int d, int K) {
+                                         const int* __restrict__ state_slot, int d, int K_arg) {
+    const int K = KT ? KT : K_arg;
     const int t = blockIdx.x;
     const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
     if (c >= d) return;
@@ -63,8 +64,18 @@ __global__ void shortconv_fwd_vec_kernel(const bf16_t* __restrict__ bcx, const T
     const int t0 = q_start[r];
     const int i = t - t0;
     const float* st = state + (long long)state_slot[r] * (K - 1) * d;
+    // the taps of the thread's eight channels are 8 K neighbouring weights: with a known K they come
+    // in whole pieces of eight
+    float wl[KT ? 8 * KT : 1];
+    if (KT) {
+#pragma unroll
+        for (int p = 0; p < KT; ++p)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) wl[p * 8 + e] = to_f32(conv_w[(long long)c * KT + p * 8 + e]);
+    }
     float y[8];
-    for (int k = 0; k < K; ++k) {
+#pragma unroll
+    for (int k = 0; k < (KT ? KT : 1) * (KT ? 1 : K); ++k) {
         const int src = i - (K - 1) + k;
         float u[8];
         if (src >= 0) {
@@ -80,7 +91,7 @@ __global__ void shortconv_fwd_vec_kernel(const bf16_t* __restrict__ bcx, const T
         }
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float w = to_f32(conv_w[(long long)(c + e) * K + k]);
+            const float w = KT ? wl[e * (KT ? KT : 1) + k] : to_f32(conv_w[(long long)(c + e) * K + k]);
             y[e] = (k == 0) ? u[e] * w : fmaf(u[e], w, y[e]);
         }
     }
@@ -160,12 +171,12 @@ TUFF_EXPORT int tuff_shortconv_fwd(const void* bcx, const void* conv_w, int w_dt
     if (dt == DT_BF16 && d % 8 == 0 && n_tokens > 16) {
         const int threads = d / 8 < 256 ? ((d / 8 + 63) / 64) * 64 : 256;
         dim3 vblock(threads), vgrid(n_tokens, ceil_div(d / 8, threads));
-        if (w_dt == DT_F32)
-            hipLaunchKernelGGL(shortconv_fwd_vec_kernel<float>, vgrid, vblock, 0, stream, (const bf16_t*)bcx, (const float*)conv_w,
-                               state, (bf16_t*)out, req_of_token, q_start, state_slot, d, K);
-        else
-            hipLaunchKernelGGL(shortconv_fwd_vec_kernel<bf16_t>, vgrid, vblock, 0, stream, (const bf16_t*)bcx, (const bf16_t*)conv_w,
-                               state, (bf16_t*)out, req_of_token, q_start, state_slot, d, K);
+#define VEC(TW, KT) hipLaunchKernelGGL((shortconv_fwd_vec_kernel<TW, KT>), vgrid, vblock, 0, stream, (const bf16_t*)bcx, (const TW*)conv_w, \
+                                          state, (bf16_t*)out, req_of_token, q_start, state_slot, d, K)
+#define VEC_K(TW) do { if (K == 2) VEC(TW, 2); else if (K == 3) VEC(TW, 3); else if (K == 4) VEC(TW, 4); else VEC(TW, 0); } while (0)
+        if (w_dt == DT_F32) VEC_K(float); else VEC_K(bf16_t);
+#undef VEC_K
+#undef VEC
         return launch_status();
     }
     dim3 block(256), grid(n_tokens, ceil_div(d, 256));
