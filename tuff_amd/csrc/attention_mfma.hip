@@ -262,7 +262,10 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
 constexpr int COMBINE_MAX_PARTS = 2048;
 
 // Up to 64 partitions: lane p keeps (m_p, l_p) in registers, weights travel by shuffle; no LDS.
-// Same arithmetic as the general kernel below.
+// Same arithmetic as the general kernel below.  PER: channels a lane (head size / 64, rounded up);
+// the partial outputs of BATCH partitions are asked for at once, so that a context of 8192 positions
+// with heads of 64 is one trip to memory.
+template <int PER, int BATCH>
 __global__ __launch_bounds__(WAVE) void attn_combine64_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                                               bf16_t* __restrict__ out, const int* __restrict__ positions,
                                                               int H, int hd, int window, int n_parts) {
@@ -282,32 +285,34 @@ __global__ __launch_bounds__(WAVE) void attn_combine64_kernel(const float* __res
     const float w_l = valid ? __expf(m_l - M) : 0.f;
     const float wl_l = w_l * (valid ? l_l : 0.f);
     const float* o = ws_o + row * n_parts * hd;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    float acc[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) acc[j] = 0.f;
     float L = 0.f;                                         // both sums run over p in ascending order
     // The loads below do not wait for the position: rows of partitions the token does not have
     // exist too (unwritten); their weight is zero and they are skipped by a select, not a product.
-    for (int i0 = 0; i0 < n_parts; i0 += 8) {
-        float ov[8][4];
+    for (int i0 = 0; i0 < n_parts; i0 += BATCH) {
+        float ov[BATCH][PER];
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
+        for (int u = 0; u < BATCH; ++u)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < PER; ++j) {
                 const int d = lane + j * WAVE;
                 ov[u][j] = (i0 + u < n_parts && d < hd) ? o[(long long)(i0 + u) * hd + d] : 0.f;
             }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
+        for (int u = 0; u < BATCH; ++u) {
             const float w = __shfl(w_l, i0 + u, WAVE);
             L += __shfl(wl_l, i0 + u, WAVE);
             if (w > 0.f) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[j] = fmaf(w, ov[u][j], acc[j]);
+                for (int j = 0; j < PER; ++j) acc[j] = fmaf(w, ov[u][j], acc[j]);
             }
         }
     }
     const float inv = 1.0f / L;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < PER; ++j) {
         const int d = lane + j * WAVE;
         if (d < hd) out[row * hd + d] = (bf16_t)(acc[j] * inv);
     }
@@ -394,10 +399,14 @@ TUFF_EXPORT int tuff_attention_mfma(const void* q, const void* k_cache, const vo
 #undef GO
     int rc = launch_status();
     if (rc) return rc;
-    if (n_parts <= WAVE)
-        hipLaunchKernelGGL(attn_combine64_kernel, dim3((unsigned)((long long)n_tokens * H)), dim3(WAVE), 0, stream,
-                           (const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, H, hd, window, n_parts);
-    else
+    if (n_parts <= WAVE) {
+#define COMBINE(PER, BATCH) hipLaunchKernelGGL((attn_combine64_kernel<PER, BATCH>), dim3((unsigned)((long long)n_tokens * H)), dim3(WAVE), \
+                                               0, stream, (const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, H, hd, window, n_parts)
+        if (hd <= 64) { if (n_parts <= 8) COMBINE(1, 8); else if (n_parts <= 16) COMBINE(1, 16); else COMBINE(1, 32); }
+        else if (hd <= 128) { if (n_parts <= 8) COMBINE(2, 8); else COMBINE(2, 16); }
+        else COMBINE(4, 8);
+#undef COMBINE
+    } else
         hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)((long long)n_tokens * H)), dim3(WAVE), 0, stream,
                            (const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, H, hd, window, n_parts);
     return launch_status();
