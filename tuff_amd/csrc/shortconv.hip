@@ -134,17 +134,27 @@ __global__ void shortconv_decode_kernel(const T* __restrict__ bcx, const TW* __r
     if (c >= d) return;
     float* st = state + (long long)state_slot[r] * (K - 1) * d;
     const T* row = bcx + (long long)r * 3 * d;
-    const float u = to_f32(row[c]) * to_f32(row[2 * d + c]);
-    float y = 0.f;
-    for (int k = 0; k < K - 1; ++k) {
-        const float s = st[(long long)k * d + c];
-        const float w = to_f32(conv_w[(long long)c * K + k]);
-        y = (k == 0) ? s * w : fmaf(s, w, y);
-        if (k > 0) st[(long long)(k - 1) * d + c] = s;
+    // every load first (a store into the state in between would hold the loads after it back), then
+    // the chain, then the stores
+    float s[MAX_TAPS], w[MAX_TAPS];
+#pragma unroll
+    for (int k = 0; k < MAX_TAPS; ++k) {
+        s[k] = k < K - 1 ? st[(long long)k * d + c] : 0.f;
+        w[k] = k < K - 1 ? to_f32(conv_w[(long long)c * K + k]) : 0.f;
     }
-    y = fmaf(u, to_f32(conv_w[(long long)c * K + K - 1]), y);
+    const float w_last = to_f32(conv_w[(long long)c * K + K - 1]);
+    const float u = to_f32(row[c]) * to_f32(row[2 * d + c]);
+    const float gate = to_f32(row[d + c]);
+    float y = 0.f;
+#pragma unroll
+    for (int k = 0; k < MAX_TAPS; ++k)
+        if (k < K - 1) y = (k == 0) ? s[k] * w[k] : fmaf(s[k], w[k], y);
+    y = fmaf(u, w_last, y);
+#pragma unroll
+    for (int k = 1; k < MAX_TAPS; ++k)
+        if (k < K - 1) st[(long long)(k - 1) * d + c] = s[k];
     st[(long long)(K - 2) * d + c] = u;
-    out[(long long)r * d + c] = from_f32<T>(to_f32(row[d + c]) * y);
+    out[(long long)r * d + c] = from_f32<T>(gate * y);
 }
 }  // namespace
 
