@@ -613,13 +613,25 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const float* __restr
     const bool whole = N % 4 == 0 && col + 3 < N;
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     if (row < M) {
-        for (int s = 0; s < n_slices; ++s) {
-            const float* p = ws + ((long long)s * rows_padded + row) * N + col;
-            if (whole) {
-                const f32x4 t = *(const f32x4*)p;
+        if (whole) {
+            // the slices of a step of eight are asked for together and added in their order
+            const long long stride = (long long)rows_padded * N;
+            const float* p0 = ws + row * N + col;
+            for (int s0 = 0; s0 < n_slices; s0 += 8) {
+                f32x4 t[8];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] += t[e];
-            } else {
+                for (int u = 0; u < 8; ++u)
+                    if (s0 + u < n_slices) t[u] = *(const f32x4*)(p0 + (s0 + u) * stride);
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    if (s0 + u < n_slices) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] += t[u][e];
+                    }
+            }
+        } else {
+            for (int s = 0; s < n_slices; ++s) {
+                const float* p = ws + ((long long)s * rows_padded + row) * N + col;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) if (col + e < N) v[e] += p[e];
             }
