@@ -107,13 +107,14 @@ def loaded_modules() -> list[str]:
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_get_device = getattr(torch._C, "_cuda_getDevice", None) or torch.cuda.current_device
 
 
 def _stream() -> int:
     """Handle of torch's current stream on the current device (the stream a graph is being
     recorded on, inside a recording).  Called once a launch, so through the cheapest way there is."""
     if _raw_stream is not None:
-        return _raw_stream(torch.cuda.current_device())
+        return _raw_stream(_get_device())
     return torch.cuda.current_stream().cuda_stream
 
 

@@ -12,6 +12,7 @@ from __future__ import annotations
 import math
 from typing import Optional
 
+import numpy as np
 import torch
 
 from ..csrc import ops
@@ -109,14 +110,43 @@ class AttentionMixer(Mixer):
         self.out.forward(o, accumulate_into=residual)
 
     @staticmethod
-    def _blocks(ctx, G, nb, device):
-        key = ("query_blocks", G, nb)
+    def _upload(array, device):
+        """Through pinned memory, so that the host does not wait for the stream."""
+        return torch.from_numpy(array).pin_memory().to(device, non_blocking=True)
+
+    @classmethod
+    def _blocks(cls, ctx, G, nb, device, skip_single: bool = False):
+        key = ("query_blocks", G, nb, skip_single)
         blocks = ctx.host.get(key)
         if blocks is None:
-            # through pinned memory, so that the host does not wait for the stream
-            blocks = torch.from_numpy(ops.query_blocks(ctx.host["q_len"], G, nb)).pin_memory().to(device, non_blocking=True)
-            ctx.host[key] = blocks
+            q_len = ctx.host["q_len"]
+            if skip_single:
+                q_len = np.where(q_len == 1, 0, q_len)
+            blocks = ctx.host[key] = cls._upload(ops.query_blocks(q_len, G, nb), device)
         return blocks
+
+    @classmethod
+    def _single_token_runs(cls, ctx, G, device):
+        """Runs of neighbouring requests with one token each in a step that also holds portions:
+        [(first token, tokens, block list, request records relative to the first token, longest
+        context)], made once a step.  Only where a request's heads fit one block of 16 columns."""
+        key = ("single_token_runs", G)
+        runs = ctx.host.get(key)
+        if runs is None:
+            runs = []
+            q_len, ctx_len = ctx.host["q_len"], ctx.host["ctx_len"]
+            if G <= 16 and (q_len == 1).any():
+                start = np.concatenate([[0], np.cumsum(q_len)[:-1]])
+                single = np.concatenate([[False], q_len == 1, [False]])
+                edges = np.flatnonzero(single[1:] != single[:-1])          # run r_lo .. r_hi - 1 for every pair
+                for r_lo, r_hi in zip(edges[0::2], edges[1::2]):
+                    tok_lo = int(start[r_lo])
+                    info = np.stack([start - tok_lo, q_len, ctx_len - q_len, ctx_len], axis=1).astype(np.int32)
+                    blocks = np.stack([np.arange(r_lo, r_hi), np.zeros(r_hi - r_lo, dtype=np.int64)], axis=1).astype(np.int32)
+                    runs.append((tok_lo, int(r_hi - r_lo), cls._upload(blocks, device), cls._upload(info, device),
+                                 int(ctx_len[r_lo:r_hi].max())))
+            ctx.host[key] = runs
+        return runs
 
     def attend(self, q, o, ctx, cache, g) -> None:
         G = self.H // self.Hkv
@@ -125,9 +155,17 @@ class AttentionMixer(Mixer):
                           page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len, window=self.window or 0,
                           scale=self.scale)
             if ctx.max_q_len > 1:
-                # prompt portions in the step: blocks of columns walk over their keys through LDS
+                # prompt portions in the step: blocks of columns walk over their keys through LDS.
+                # Requests with a single token beside them (runs of neighbours in the step's order) go
+                # the way of a step of single tokens: one workgroup walking all keys of such a request
+                # would be the longest of the step.
                 nb = ops.attention_prefill_block_columns(self.hd) // 16
-                ops.attention_prefill(q, cache.k, cache.v, o, blocks=self._blocks(ctx, G, nb, q.device), **common)
+                runs = self._single_token_runs(ctx, G, q.device)
+                ops.attention_prefill(q, cache.k, cache.v, o, blocks=self._blocks(ctx, G, nb, q.device, skip_single=bool(runs)),
+                                      **common)
+                for tok_lo, n, blocks, info, ctx_len in runs:
+                    ops.attention_mfma(q[tok_lo:tok_lo + n], cache.k, cache.v, o[tok_lo:tok_lo + n], blocks=blocks, nb=1,
+                                       positions=ctx.positions[tok_lo:tok_lo + n], **dict(common, req_info=info, max_ctx_len=ctx_len))
                 return
             # single tokens: the keys of a request are split over many waves, then merged
             nb = 1 if G <= 16 else (2 if G <= 32 else 4)
