@@ -549,6 +549,33 @@ def test_attention_long_context(gpu):
         _check_step(case, reqs, out2.cpu().double().reshape(T, H, hd), H, hd, window, ("prefill", window))
 
 
+@pytest.mark.parametrize("H,Hkv,hd,ps", [(4, 2, 64, 16), (3, 1, 80, 32), (2, 2, 128, 16)])
+@pytest.mark.parametrize("window", [0, 700])
+def test_attention_prefill_key_segments(gpu, H, Hkv, hd, ps, window, monkeypatch):
+    """A short portion far into long requests: few blocks of columns, so the keys are cut into
+    segments, a workgroup a segment, and the segments merged.  Against the plain formula, and against
+    the same step without segments (to the rounding of one merge).  One request is shorter than a
+    segment, one ends inside a segment, stale pages hold NaN."""
+    from tuff_amd.csrc import ops
+    reqs = [(5000, 40), (2100, 30), (300, 17), (0, 5)]
+    case = _mixed_step_case(gpu, reqs, H, Hkv, hd, ps)
+    T = case["q"].shape[0]
+    cols = ops.attention_prefill_block_columns(hd)
+    blocks = torch.from_numpy(ops.query_blocks(case["q_len"], H // Hkv, cols // 16)).to(gpu)
+    outs = {}
+    for segments in (False, True):
+        out = torch.full((T, H * hd), float("nan"), dtype=torch.bfloat16, device=gpu)
+        ops.attention_prefill(case["q"].to(gpu), case["kc"], case["vc"], out, block_table=case["table"],
+                              blocks=blocks, req_info=case["req_info"], H=H, Hkv=Hkv, hd=hd, page_size=ps,
+                              max_ctx_len=case["max_ctx_len"], window=window,
+                              positions=case["positions"] if segments else None)
+        outs[segments] = out.cpu().double().reshape(T, H, hd)
+        _check_step(case, reqs, outs[segments], H, hd, window, f"segments {segments}")
+    assert blocks.shape[0] * Hkv < ops.PREFILL_MIN_WORKGROUPS and case["max_ctx_len"] >= 2 * ops.PREFILL_MIN_SEGMENT
+    # the two ways differ in rounding only
+    assert (outs[True] - outs[False]).abs().max() <= 2 ** -7 * float(outs[False].abs().max())
+
+
 @pytest.mark.parametrize("kernel", ["mfma", "prefill"])
 def test_attention_matrix_kernels_find_a_far_key_and_the_window_edge(gpu, kernel):
     """One key among a thousand matches the query: the output is that key's value row, wherever

@@ -268,7 +268,7 @@ constexpr int COMBINE_MAX_PARTS = 2048;
 template <int PER, int BATCH>
 __global__ __launch_bounds__(WAVE) void attn_combine64_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                                               bf16_t* __restrict__ out, const int* __restrict__ positions,
-                                                              int H, int hd, int window, int n_parts) {
+                                                              int H, int hd, int window, int n_parts, int part_keys) {
     const long long row = blockIdx.x;                      // token * H + head
     const int lane = threadIdx.x;
     float m_l = -INFINITY, l_l = 0.f;
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(WAVE) void attn_combine64_kernel(const float* __res
     }
     const int pos = positions[row / H];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int p_lo = lo / PART, p_hi = pos / PART;
+    const int p_lo = lo / part_keys, p_hi = pos / part_keys;
     const bool valid = lane >= p_lo && lane <= p_hi && l_l > 0.f;
     const float M = wave_max(valid ? m_l : -INFINITY);
     const float w_l = valid ? __expf(m_l - M) : 0.f;
@@ -320,13 +320,13 @@ __global__ __launch_bounds__(WAVE) void attn_combine64_kernel(const float* __res
 
 __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                                             bf16_t* __restrict__ out, const int* __restrict__ positions,
-                                                            int H, int hd, int window, int n_parts) {
+                                                            int H, int hd, int window, int n_parts, int part_keys) {
     __shared__ float wts[COMBINE_MAX_PARTS], wls[COMBINE_MAX_PARTS];
     const long long row = blockIdx.x;                      // token * H + head
     const int lane = threadIdx.x;
     const int pos = positions[row / H];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int p_lo = lo / PART, np = pos / PART - p_lo + 1;
+    const int p_lo = lo / part_keys, np = pos / part_keys - p_lo + 1;
     const float* ml = ws_ml + (row * n_parts + p_lo) * 2;
     float M = -INFINITY;
     for (int i = lane; i < np; i += WAVE) M = fmaxf(M, ml[i * 2 + 1] > 0.f ? ml[i * 2] : -INFINITY);
@@ -368,6 +368,25 @@ void launch_partition(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16
 }
 }  // namespace
 
+// Merges, for every (token, head) of n_tokens tokens, the partial results of its partitions of
+// part_keys keys each.
+static int launch_merge(const float* ws_o, const float* ws_ml, bf16_t* out, const int* positions, int n_tokens, int H, int hd,
+                 int window, int n_parts, int part_keys, hipStream_t stream) {
+    const dim3 grid((unsigned)((long long)n_tokens * H));
+    if (n_parts <= WAVE) {
+#define COMBINE(PER, BATCH) hipLaunchKernelGGL((attn_combine64_kernel<PER, BATCH>), grid, dim3(WAVE), 0, stream, ws_o, ws_ml, out, \
+                                               positions, H, hd, window, n_parts, part_keys)
+        if (hd <= 64) { if (n_parts <= 8) COMBINE(1, 8); else if (n_parts <= 16) COMBINE(1, 16); else COMBINE(1, 32); }
+        else if (hd <= 128) { if (n_parts <= 8) COMBINE(2, 8); else COMBINE(2, 16); }
+        else COMBINE(4, 8);
+#undef COMBINE
+    } else {
+        hipLaunchKernelGGL(attn_combine_kernel, grid, dim3(WAVE), 0, stream, ws_o, ws_ml, out, positions, H, hd, window, n_parts,
+                           part_keys);
+    }
+    return launch_status();
+}
+
 // Query blocks are listed by the host: block b holds the columns blk[b].y .. +16*nb-1 of request
 // blk[b].x (a request's columns are numbered (token - its first token) * G + head within the kv
 // group); blk == null: block b is request b from column 0 (every request fits one block).
@@ -399,15 +418,16 @@ TUFF_EXPORT int tuff_attention_mfma(const void* q, const void* k_cache, const vo
 #undef GO
     int rc = launch_status();
     if (rc) return rc;
-    if (n_parts <= WAVE) {
-#define COMBINE(PER, BATCH) hipLaunchKernelGGL((attn_combine64_kernel<PER, BATCH>), dim3((unsigned)((long long)n_tokens * H)), dim3(WAVE), \
-                                               0, stream, (const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, H, hd, window, n_parts)
-        if (hd <= 64) { if (n_parts <= 8) COMBINE(1, 8); else if (n_parts <= 16) COMBINE(1, 16); else COMBINE(1, 32); }
-        else if (hd <= 128) { if (n_parts <= 8) COMBINE(2, 8); else COMBINE(2, 16); }
-        else COMBINE(4, 8);
-#undef COMBINE
-    } else
-        hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)((long long)n_tokens * H)), dim3(WAVE), 0, stream,
-                           (const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, H, hd, window, n_parts);
-    return launch_status();
+    return launch_merge((const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, n_tokens, H, hd, window, n_parts, PART,
+                        stream);
+}
+
+// The merge alone, for partial results that another kernel left in the same layout (ws_o
+// [tokens * H * n_parts * hd], ws_ml [tokens * H * n_parts * 2] = (reference exponent, sum); partition
+// p of a row holds the keys p * part_keys .. (p + 1) * part_keys - 1).
+TUFF_EXPORT int tuff_attention_merge(const float* ws_o, const float* ws_ml, void* out, const int* positions, int n_tokens,
+                                     int H, int hd, int window, int n_parts, int part_keys, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (hd > 256 || n_parts < 1 || n_parts > COMBINE_MAX_PARTS || part_keys < 1) return -2;
+    return launch_merge(ws_o, ws_ml, (bf16_t*)out, positions, n_tokens, H, hd, window, n_parts, part_keys, stream);
 }

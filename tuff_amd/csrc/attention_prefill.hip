@@ -45,7 +45,8 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ block_table, int max_blocks,
     const int2* __restrict__ blk, const int4* __restrict__ req_info,
-    int H, int Hkv, int hd, int page_size, int window, float scale_log2e) {
+    int H, int Hkv, int hd, int page_size, int window, float scale_log2e,
+    int seg_keys, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
     constexpr int KC = HDP / 32;          // 32-wide chunks of the head dimension
     constexpr int DB = HDP / 16;          // 16-wide blocks of output channels
     constexpr int HC = HDP / 8;           // 16-byte chunks of a K row
@@ -71,8 +72,14 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     const int last_col = min(ncols, col0 + CB) - 1;
     const int pos_max = pos0 + last_col / G;
     const int lo_min = window > 0 ? max(0, pos0 + col0 / G - window + 1) : 0;
-    const int key_start = lo_min / STEP * STEP;
-    const int nsteps = (pos_max - key_start) / STEP + 1;
+    // gridDim.z > 1: the keys are cut into segments of seg_keys (a multiple of STEP), a workgroup a
+    // segment; it leaves what it has summed, unnormalised, with its reference exponent and sum in
+    // the work space, for the kernel that merges the partitions of single-token steps.
+    const int seg = blockIdx.z, n_segs = gridDim.z;
+    const int seg_begin = n_segs > 1 ? seg * seg_keys : 0;
+    const int key_last = n_segs > 1 ? min(pos_max, seg_begin + seg_keys - 1) : pos_max;
+    const int key_start = max(lo_min / STEP * STEP, seg_begin);
+    const int nsteps = key_last >= key_start ? (key_last - key_start) / STEP + 1 : 0;
 
     // ---- this wave's columns
     const int wcol0 = col0 + wave * NBW * 16;
@@ -112,6 +119,17 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         l_run[nb] = 0.f;
 #pragma unroll
         for (int db = 0; db < DB; ++db) o[db][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    if (nsteps == 0) {                     // a segment beyond the block's keys: nothing summed
+#pragma unroll
+        for (int nb = 0; nb < NBW; ++nb)
+            if (qrow[nb] >= 0 && g == 0) {
+                const long long slot = qrow[nb] * n_segs + seg;
+                ws_ml[slot * 2] = -INFINITY;
+                ws_ml[slot * 2 + 1] = 0.f;
+            }
+        return;
     }
 
     // ---- page numbers: lane i holds the page of granule (16 keys) gran_base + i; 64 granules = 16 steps
@@ -318,6 +336,17 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         l += __shfl_xor(l, 16, WAVE);
         l += __shfl_xor(l, 32, WAVE);
         if (qrow[nb] < 0) continue;
+        if (n_segs > 1) {
+            const long long slot = qrow[nb] * n_segs + seg;
+            // the merge works with natural exponents: reference 2^m = e^(m ln 2)
+            if (g == 0) { ws_ml[slot * 2] = m_run[nb] * 0.6931471805599453f; ws_ml[slot * 2 + 1] = l; }
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const int dim = db * 16 + 4 * g;
+                if (dim < hd) *(f32x4*)(ws_o + slot * hd + dim) = o[db][nb];
+            }
+            continue;
+        }
         const float inv = 1.0f / l;
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
@@ -334,7 +363,7 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
 template <int HDP, int NBW, int AHEAD>
 int launch(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, bf16_t* out,
            const int* bt, int max_blocks, const int2* blk, const int4* req_info,
-           int H, int Hkv, int hd, int ps, int window, float scale_log2e) {
+           int H, int Hkv, int hd, int ps, int window, float scale_log2e, int seg_keys, float* ws_o, float* ws_ml) {
     auto kern = attn_prefill_kernel<HDP, NBW, AHEAD>;
     constexpr int lds = 2 * (STEP * (HDP + 8) + HDP * VROW) * 2;
     static bool set = false;
@@ -343,7 +372,7 @@ int launch(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, con
         set = true;
     }
     hipLaunchKernelGGL(kern, grid, dim3(NT), lds, stream, q, kc, vc, out, bt, max_blocks, blk, req_info,
-                       H, Hkv, hd, ps, window, scale_log2e);
+                       H, Hkv, hd, ps, window, scale_log2e, seg_keys, ws_o, ws_ml);
     return launch_status();
 }
 }  // namespace
@@ -355,20 +384,27 @@ TUFF_EXPORT int tuff_attention_prefill_block_columns(int hd) { return hd <= 128 
 // of request blk[b].x (a request's columns are numbered (token - its first token) * G + head
 // within the kv group); blk == null: block b is request b from column 0.
 // req_info [R]: (first token of the request in the step, its tokens, position of the first, -).
+// n_segs > 1: the keys are cut into segments of seg_keys (a multiple of 64) and `out` is not written:
+// the partial results go to ws_o [tokens * H * n_segs * hd] and ws_ml [tokens * H * n_segs * 2] in the
+// layout of the single-token kernel's partitions, to be merged by tuff_attention_merge with
+// part_keys = seg_keys.
 TUFF_EXPORT int tuff_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
                                        const int* block_table, int max_blocks, const int* blk, int n_qblocks,
                                        const int* req_info, int H, int Hkv, int hd, int page_size, int window,
-                                       float scale, hipStream_t stream) {
+                                       float scale, int n_segs, int seg_keys, float* ws_o, float* ws_ml,
+                                       hipStream_t stream) {
     if (n_qblocks <= 0) return 0;
     if (hd > 256 || hd % 8 != 0 || page_size % 16 != 0 || Hkv <= 0 || H % Hkv != 0) return -2;
     if (Hkv > 65535 || !(scale > 0.f)) return -2;
+    if (n_segs < 1 || n_segs > 65535) return -2;
+    if (n_segs > 1 && (seg_keys <= 0 || seg_keys % STEP != 0 || !ws_o || !ws_ml)) return -2;
     const bf16_t* Q = (const bf16_t*)q;
     const bf16_t* K = (const bf16_t*)k_cache;
     const bf16_t* V = (const bf16_t*)v_cache;
-    dim3 grid(n_qblocks, Hkv);
+    dim3 grid(n_qblocks, Hkv, n_segs);
     const float sl = scale * 1.4426950408889634f;
 #define GO(HDP, NBW, AHEAD) return launch<HDP, NBW, AHEAD>(grid, stream, Q, K, V, (bf16_t*)out, block_table, max_blocks, (const int2*)blk, \
-                                             (const int4*)req_info, H, Hkv, hd, page_size, window, sl)
+                                             (const int4*)req_info, H, Hkv, hd, page_size, window, sl, seg_keys, ws_o, ws_ml)
     if (hd <= 32) GO(32, 2, 3);
     else if (hd <= 64) GO(64, 2, 3);
     else if (hd <= 96) GO(96, 2, 2);

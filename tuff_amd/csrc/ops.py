@@ -63,10 +63,13 @@ _SIGNATURES = {
         "tuff_attention_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                                 _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p],
+        "tuff_attention_merge": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                 _c_void_p],
     },
     "attention_prefill": {
         "tuff_attention_prefill": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
-                                   _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p],
+                                   _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
+                                   _c_void_p, _c_void_p, _c_void_p],
         "tuff_attention_prefill_block_columns": [_c_int],
     },
     "shortconv": {
@@ -519,12 +522,20 @@ def attention_prefill_block_columns(hd: int) -> int:
     return 128 if hd <= 128 else 64
 
 
+PREFILL_MIN_WORKGROUPS = 192     # fewer than this: the keys are cut into segments, a workgroup a segment
+PREFILL_MIN_SEGMENT = 1024       # keys; shorter segments are not worth their merge
+
+
 def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info,
-                      H, Hkv, hd, page_size, max_ctx_len, window=0, scale=None) -> None:
+                      H, Hkv, hd, page_size, max_ctx_len, window=0, scale=None, positions=None) -> None:
     """Matrix-core attention for steps with prompt portions: a workgroup walks over all keys of a
     block of query columns, keys and values staged through LDS; writes `out` directly.
     blocks: int32 [n_blocks, 2] from query_blocks(q_len, G, attention_prefill_block_columns(hd) // 16),
-    or None when every request's columns fit one block (block b = request b)."""
+    or None when every request's columns fit one block (block b = request b).
+    positions (int32 [T], optional): with them, a step with few blocks and long contexts (a short
+    portion far into a long prompt) cuts the keys into segments, a workgroup a segment, and merges the
+    segments' results as a step of single tokens merges its partitions.  Then every row of `out` is
+    written, also those of tokens no block covers (with meaningless values)."""
     T = q.shape[0]
     if not attention_mfma_supported(q.dtype, hd, page_size):
         raise KernelError(f"attention_prefill: needs bfloat16, a head size that is a multiple of 8 (got {hd}) "
@@ -553,10 +564,27 @@ def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info
         _gpu("blocks", blocks, torch.int32, (nblk, 2))
     if scale is None:
         scale = 1.0 / math.sqrt(hd)
+    n_segs, seg_keys, ws_o, ws_ml = 1, 0, None, None
+    workgroups = nblk * Hkv
+    if positions is not None and 0 < workgroups < PREFILL_MIN_WORKGROUPS and int(max_ctx_len) >= 2 * PREFILL_MIN_SEGMENT:
+        want = min(-(-2 * PREFILL_MIN_WORKGROUPS // workgroups), int(max_ctx_len) // PREFILL_MIN_SEGMENT, 64)
+        seg_keys = -(-(-(-int(max_ctx_len) // want)) // 64) * 64
+        n_segs = -(-int(max_ctx_len) // seg_keys)
+    if n_segs > 1:
+        _gpu("positions", positions, torch.int32, (T,))
+        ws_o = torch.empty(T * H * n_segs * hd, dtype=torch.float32, device=q.device)
+        ws_ml = torch.empty(T * H * n_segs * 2, dtype=torch.float32, device=q.device)
+    else:
+        n_segs, seg_keys = 1, 0
     _check(load("attention_prefill").tuff_attention_prefill(
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
         block_table.data_ptr(), block_table.shape[1], None if blocks is None else blocks.data_ptr(), nblk,
-        req_info.data_ptr(), H, Hkv, hd, page_size, int(window or 0), float(scale), _stream()), "attention_prefill")
+        req_info.data_ptr(), H, Hkv, hd, page_size, int(window or 0), float(scale), n_segs, seg_keys,
+        None if ws_o is None else ws_o.data_ptr(), None if ws_ml is None else ws_ml.data_ptr(), _stream()), "attention_prefill")
+    if n_segs > 1:
+        _check(load("attention_mfma").tuff_attention_merge(ws_o.data_ptr(), ws_ml.data_ptr(), out.data_ptr(), positions.data_ptr(),
+                                                           T, H, hd, int(window or 0), n_segs, seg_keys, _stream()),
+               "attention_merge")
 
 
 def query_blocks(q_len, G: int, nb: int):

@@ -161,8 +161,9 @@ class AttentionMixer(Mixer):
                 # would be the longest of the step.
                 nb = ops.attention_prefill_block_columns(self.hd) // 16
                 runs = self._single_token_runs(ctx, G, q.device)
+                # (first: with key segments it writes every row of o, the single tokens' rows come after)
                 ops.attention_prefill(q, cache.k, cache.v, o, blocks=self._blocks(ctx, G, nb, q.device, skip_single=bool(runs)),
-                                      **common)
+                                      positions=ctx.positions, **common)
                 for tok_lo, n, blocks, info, ctx_len in runs:
                     ops.attention_mfma(q[tok_lo:tok_lo + n], cache.k, cache.v, o[tok_lo:tok_lo + n], blocks=blocks, nb=1,
                                        positions=ctx.positions[tok_lo:tok_lo + n], **dict(common, req_info=info, max_ctx_len=ctx_len))
