@@ -131,6 +131,68 @@ def run_prefill(llm, cfg, tokens: int, repeats: int = 3):
     return best
 
 
+# Two serving runs through the scheduler, on other shapes of the architecture: many requests of very
+# different lengths, prompts in portions beside decoding requests.
+SCENARIOS = {
+    "lfm2-2.6b": dict(
+        config=dict(architectures=["Lfm2ForCausalLM"], num_hidden_layers=30,
+                    full_attn_idxs=[2, 6, 10, 14, 18, 21, 24, 27], hidden_size=2048, num_attention_heads=32,
+                    num_key_value_heads=8, block_ff_dim=16128, block_auto_adjust_ff_dim=True, block_multiple_of=256,
+                    vocab_size=65536, rope_theta=1000000.0, conv_L_cache=3, norm_eps=1e-5, tie_word_embeddings=True,
+                    max_position_embeddings=16384),
+        seed=3, requests=32, at_a_time=32, budget=2048, new_tokens=256, prompts=("uniform", 128, 4096)),
+    "lfm2-700m-long": dict(
+        config=dict(architectures=["Lfm2ForCausalLM"], num_hidden_layers=16, full_attn_idxs=[2, 5, 8, 10, 12, 14],
+                    hidden_size=1536, num_attention_heads=24, num_key_value_heads=8, block_ff_dim=6912,
+                    block_auto_adjust_ff_dim=False, vocab_size=65536, rope_theta=1000000.0, conv_L_cache=3,
+                    norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=32768),
+        seed=4, requests=64, at_a_time=64, budget=512, new_tokens=64, prompts=("log-uniform", 16, 30000)),
+}
+
+
+def run_scenario(name: str, dtype: str) -> dict:
+    import math
+    import random
+    import torch
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.engine.llm import LLM
+    from tuff_amd.models.registry import config_from_dict
+    from tuff_amd.sampling.params import SamplingParams
+    sc = SCENARIOS[name]
+    cfg = config_from_dict(sc["config"])
+    rng = random.Random(sc["seed"])
+    kind, lo, hi = sc["prompts"]
+    if kind == "uniform":
+        lens = [rng.randint(lo, hi) for _ in range(sc["requests"])]
+    else:
+        lens = [int(math.exp(rng.uniform(math.log(lo), math.log(hi)))) for _ in range(sc["requests"])]
+    new = sc["new_tokens"]
+    pages = sum(-(-(n + new) // 16) for n in lens) + 64
+    eng = Engine.from_config(cfg, sc["seed"], dtype=dtype, page_size=16, num_pages=pages, max_requests=sc["at_a_time"])
+    llm = LLM(engine=eng, max_num_seqs=sc["at_a_time"], max_batched_tokens=sc["budget"],
+              ctx_size=cfg.max_position_embeddings, ignore_eos=True)
+    g = torch.Generator().manual_seed(SEED)
+    prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=g).tolist() for n in lens]
+    best = None
+    for _ in range(2):                                     # the first run warms up
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        outs = llm.generate(prompts, SamplingParams(max_new_tokens=new, ignore_eos=True))
+        torch.cuda.synchronize()
+        best = time.perf_counter() - t0
+        if not all(len(o.token_ids) == new for o in outs):
+            raise RuntimeError("a request of the scenario did not run to its end")
+    total = sum(lens) + len(lens) * new
+    st = llm.last_stats
+    return {"metric": f"tokens/s through the scheduler, prompts and generated ({name})", "value": round(total / best, 1),
+            "unit": "tokens/s", "n_gpus": 1, "seconds": round(best, 3), "generated_per_s": round(len(lens) * new / best, 1),
+            "dtype": dtype, "data": "synthetic: seeded random weights, uniform random token ids",
+            "config": {"scenario": name, "requests": len(lens), "at_a_time": sc["at_a_time"], "prompt_tokens": sum(lens),
+                       "longest_prompt": max(lens), "new_tokens_each": new, "max_batched_tokens": sc["budget"],
+                       "layers": cfg.num_hidden_layers, "hidden": cfg.hidden_size, "ffn": cfg.ffn_dim,
+                       "steps": st["steps"], "preemptions": st["preemptions"]}}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -145,6 +207,8 @@ def main() -> int:
     ap.add_argument("--point-steps", type=int, default=32)
     ap.add_argument("--only-prefill", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiling) and print its record")
+    ap.add_argument("--scenario", choices=sorted(SCENARIOS),
+                    help="instead of the benchmark: a serving run through the scheduler on another shape")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -152,6 +216,10 @@ def main() -> int:
     if int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; start it without a multi-process launcher")
         return 2
+
+    if args.scenario:
+        print(json.dumps(run_scenario(args.scenario, "bfloat16" if args.dtype == "bf16" else "float32")))
+        return 0
 
     import torch
     from tuff_amd.engine.engine import Engine
