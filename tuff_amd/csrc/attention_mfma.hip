@@ -341,15 +341,27 @@ __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restr
     const float* o = ws_o + (row * n_parts + p_lo) * hd;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     float L = 0.f;
-#pragma unroll 4
-    for (int i = 0; i < np; ++i) {
-        const float w = wts[i];
-        L += wls[i];
+    // the partial outputs of sixteen partitions are asked for together; the sums run in ascending order
+    const int per = (hd + WAVE - 1) / WAVE;                // channels a lane
+    for (int i0 = 0; i0 < np; i0 += 16) {
+        float ov[16][4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int d = lane + j * WAVE;
-            if (d < hd) acc[j] = fmaf(w, o[(long long)i * hd + d], acc[j]);
-        }
+        for (int u = 0; u < 16; ++u)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int d = lane + j * WAVE;
+                ov[u][j] = (j < per && i0 + u < np && d < hd) ? o[(long long)(i0 + u) * hd + d] : 0.f;
+            }
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+            if (i0 + u < np) {
+                const float w = wts[i0 + u];
+                L += wls[i0 + u];
+                if (w > 0.f) {                             // a partition without weight may hold anything
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[j] = fmaf(w, ov[u][j], acc[j]);
+                }
+            }
     }
     const float inv = 1.0f / L;
 #pragma unroll
