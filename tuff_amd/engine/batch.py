@@ -93,16 +93,26 @@ def pack_step(entries: Sequence[StepEntry], manager, vocab_size: int,
     info = buf[offs[8 + 2 * n_groups]:offs[9 + 2 * n_groups]].reshape(R, 4)
     t = li = 0
     max_q = max_ctx = 1
+    slot_maps = [buf[offs[8 + 2 * g]:offs[9 + 2 * g]] for g in range(n_groups)]
+    block_tables = [buf[offs[9 + 2 * g]:offs[10 + 2 * g]].reshape(R, max_blocks) for g in range(n_groups)]
+    for bt in block_tables:
+        bt.fill(-1)
     for r, e in enumerate(entries):
         n = len(e.tokens)
         total = manager.length(e.req_id)
         past = total - n
-        toks = np.asarray(e.tokens, dtype=np.int64)
-        if n and (toks.min() < 0 or toks.max() >= vocab_size):
-            raise ValueError(f"request {e.req_id!r}: token id outside [0, {vocab_size})")
-        tokens[t:t + n] = toks
-        positions[t:t + n] = np.arange(past, total)
-        req_of[t:t + n] = r
+        if n == 1:                        # the common entry of a serving step, without array detours
+            tok = int(e.tokens[0])
+            if tok < 0 or tok >= vocab_size:
+                raise ValueError(f"request {e.req_id!r}: token id outside [0, {vocab_size})")
+            tokens[t], positions[t], req_of[t] = tok, past, r
+        else:
+            toks = np.asarray(e.tokens, dtype=np.int64)
+            if n and (toks.min() < 0 or toks.max() >= vocab_size):
+                raise ValueError(f"request {e.req_id!r}: token id outside [0, {vocab_size})")
+            tokens[t:t + n] = toks
+            positions[t:t + n] = np.arange(past, total)
+            req_of[t:t + n] = r
         q_start[r], q_len[r], ctx_len[r], slot[r] = t, n, total, manager.slot(e.req_id)
         info[r] = (t, n, past, total)
         for w in e.want:
@@ -112,21 +122,18 @@ def pack_step(entries: Sequence[StepEntry], manager, vocab_size: int,
             li += 1
         for g in range(n_groups):
             table = tables[r][g]
-            sm = buf[offs[8 + 2 * g]:offs[9 + 2 * g]]
-            bt = buf[offs[9 + 2 * g]:offs[10 + 2 * g]].reshape(R, max_blocks)
-            bt[r, :len(table)] = table
-            bt[r, len(table):] = -1
+            block_tables[g][r, :len(table)] = table
             if n == 1:
                 page = int(table[past // ps])
                 if page < 0:
                     raise RuntimeError(f"request {e.req_id!r}: a token would be written to a freed page")
-                sm[t] = page * ps + past % ps
+                slot_maps[g][t] = page * ps + past % ps
             elif n:
                 pos = np.arange(past, total)
                 pages = table[pos // ps].astype(np.int64)
                 if pages.min() < 0:
                     raise RuntimeError(f"request {e.req_id!r}: a token would be written to a freed page")
-                sm[t:t + n] = pages * ps + pos % ps
+                slot_maps[g][t:t + n] = pages * ps + pos % ps
         t += n
         max_q, max_ctx = max(max_q, n), max(max_ctx, total)
     identity = n_logits == T and bool((rows == np.arange(T)).all())
