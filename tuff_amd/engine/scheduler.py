@@ -29,7 +29,7 @@ from ..sampling.params import SamplerState, SamplingParams
 WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
 
 
-@dataclasses.dataclass
+@dataclasses.dataclass(eq=False)           # a request is itself: lists of requests are searched by identity
 class Request:
     id: Hashable
     prompt: list
