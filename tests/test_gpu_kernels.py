@@ -799,6 +799,21 @@ def test_shortconv_last_tap_is_the_current_token(gpu):
     assert torch.allclose(out.cpu(), want, atol=1e-6)
 
 
+def test_scatter_of_token_ids(gpu):
+    from tuff_amd.csrc import ops
+    dst = torch.arange(100, 137, dtype=torch.int32)
+    src = torch.arange(1000, 1011, dtype=torch.int32)
+    places, sources = [36, 0, 5, 17], [10, 3, 3, 0]
+    d = dst.to(gpu)
+    ops.scatter_i32(d, src.to(gpu), torch.tensor(places + sources, dtype=torch.int32, device=gpu))
+    want = dst.clone()
+    want[places] = src[sources]
+    assert torch.equal(d.cpu(), want)
+    for bad in ([37, 0], [0, 11], [-1, 0]):           # an index out of range writes nothing
+        ops.scatter_i32(d, src.to(gpu), torch.tensor(bad, dtype=torch.int32, device=gpu))
+        assert torch.equal(d.cpu(), want)
+
+
 # --------------------------------------------------------------------------- sampling
 def test_argmax_ties_go_to_the_lowest_index(gpu):
     from tuff_amd.csrc import ops

@@ -193,6 +193,45 @@ def test_recorded_decode_steps_equal_eager_steps(gpu, dtype):
     util.assert_close(dtype, got["y"][mask], full[mask], "y")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_token_ids_taken_from_the_device(gpu, dtype):
+    """A step may take some of its token ids from a vector on the device (the sampler's output of
+    the step before) instead of from its entries: a step of portions beside single tokens, and a
+    recorded step of single tokens, give exactly what they give with the ids in the entries."""
+    from tuff_amd.engine.batch import StepEntry
+    V = util.TINY_B["vocab_size"]
+    toks = {k: util.rand_tokens(40, V, 5 + i) for i, k in enumerate("abc")}
+    drawn = torch.tensor([toks["c"][20], 0, toks["a"][20], toks["b"][21], toks["a"][21]], dtype=torch.int32, device=gpu)
+
+    def steps(eng, from_device):
+        for k in toks:
+            eng.begin(k)
+        eng.step([StepEntry(k, toks[k][:20], []) for k in "ab"])
+        hide = (lambda t: 0) if from_device else (lambda t: t)
+        # c's portion between two single tokens, then single tokens in another order than `drawn`
+        first = [StepEntry("a", [hide(toks["a"][20])], [0]), StepEntry("c", toks["c"][:20], [19]),
+                 StepEntry("b", toks["b"][20:21], [0])]
+        second = [StepEntry("b", [hide(toks["b"][21])], [0]), StepEntry("c", [hide(toks["c"][20])], [0]),
+                  StepEntry("a", [hide(toks["a"][21])], [0])]
+        out = [eng.step(first, (drawn, [0], [2]) if from_device else None).float().cpu(),
+               eng.step(second, (drawn, [0, 1, 2], [3, 0, 4]) if from_device else None).float().cpu()]
+        for k in toks:
+            eng.end(k)
+        return out
+
+    for graphs in (False, True):
+        eng = make_engine("B", dtype, use_graphs=graphs)
+        want, got = steps(eng, False), steps(eng, True)
+        assert all(torch.equal(w, g) for w, g in zip(want, got))
+        assert not graphs or eng.graph_replays >= 1
+    util.assert_close(dtype, got[1][2:], util.plain_logits("B", toks["a"][:22], stored_for(dtype))[21:], "a")
+    with pytest.raises(ValueError, match="out of range"):
+        eng.begin("a")
+        eng.step([StepEntry("a", [1, 2], [])], (drawn, [2], [0]))
+    assert eng.length("a") == 0
+    eng.end("a")
+
+
 def test_layers_of_full_size_float32_against_the_plain_implementation(gpu):
     """Layers with the sizes of a 1.2B model, float32, against the plain implementation: whole, a
     head then single tokens, and two requests mixed in portions."""

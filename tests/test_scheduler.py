@@ -4,7 +4,7 @@ import hashlib
 import pytest
 
 from tuff_amd.cache.manager import CacheLayout, CacheManager
-from tuff_amd.engine.scheduler import Request, Scheduler
+from tuff_amd.engine.scheduler import PLACEHOLDER, Request, Scheduler
 from tuff_amd.parts.base import FixedState, PagedKV
 from tuff_amd.sampling.params import SamplingParams
 
@@ -246,10 +246,11 @@ def test_seeded_sampling_state_survives_preemption():
 
 
 # ---------------------------------------------------------------- deciding a step ahead
-def run_ahead(sched, ex, eos=None):
-    """The loop of LLM.run over the fake executor: where schedule_ahead() allows, the next step
-    is 'started' (the executor extends the cache and records a stand-in token) before the
-    current step's tokens are handed to update()."""
+def run_ahead(sched, ex, stats=None):
+    """The loop of LLM.run over the fake executor: the next step is decided between advance() and
+    commit() and 'started' (the executor extends the cache) before the current step's tokens are
+    handed over; the executor sees the real token where the scheduler has a placeholder, as the
+    GPU does."""
     steps, ahead = [], 0
     under_way = None
     while under_way is not None or sched.has_unfinished():
@@ -260,22 +261,28 @@ def run_ahead(sched, ex, eos=None):
         else:
             batch, sampled = under_way
             under_way = None
-        nxt = sched.schedule_ahead(batch)
-        if nxt is not None:
-            # the executor sees the real token of every request, as the GPU does
+        live = sched.advance(batch)
+        nxt = sched.schedule(ahead=True)
+        if nxt:
+            assert sum(len(s.tokens) for s in nxt) <= sched.max_batched_tokens
+            assert len({s.request.id for s in nxt}) == len(nxt)
             for s in nxt:
-                s.tokens = [sampled[s.request.id]]
-            under_way = (nxt, ex.step_stale_ok(nxt, sched))
+                if PLACEHOLDER in s.tokens:
+                    assert len(s.tokens) == 1 and s.samples
+                    s.tokens = [sampled[s.request.id]]
+            under_way = (nxt, ex.step(nxt))
             ahead += 1
-        sched.update(batch, sampled)
-        steps.append(batch)
+            if stats is not None and any(len(s.tokens) > 1 for s in nxt):
+                stats["mixed"] = stats.get("mixed", 0) + 1
+        sched.commit(batch, sampled)
+        for r in list(sched.running) + list(sched.waiting) + sched.finished:
+            assert PLACEHOLDER not in r.output
+        steps.append(live)
     return steps, ahead
 
 
 class AheadExecutor(FakeExecutor):
-    def step_stale_ok(self, batch, sched):
-        """Like step(); a request may end (and be released) while this step is under way."""
-        return self.step(batch)
+    """A request may end (and be released) while a step that holds it is under way."""
 
     def end(self, rid):
         self.manager.release(rid)
@@ -283,20 +290,22 @@ class AheadExecutor(FakeExecutor):
 
 
 def test_a_step_decided_ahead_feeds_the_same_tokens():
-    prompts = {"a": list(range(9)), "b": list(range(40, 47)), "c": list(range(100, 103))}
-    new = {"a": 12, "b": 7, "c": 20}
+    prompts = {"a": list(range(9)), "b": list(range(40, 47)), "c": list(range(100, 103)), "d": list(range(200, 231)),
+               "e": list(range(300, 305))}
+    new = {"a": 12, "b": 7, "c": 20, "d": 3, "e": 1}
     outs = {}
     for mode in ("plain", "ahead"):
         ex = AheadExecutor()
-        sched = make(ex, max_batched_tokens=8)
+        sched = make(ex, max_batched_tokens=8, max_num_seqs=3)
         reqs = {k: Request(k, prompts[k], SamplingParams(max_new_tokens=new[k])) for k in prompts}
         for r in reqs.values():
             sched.add(r)
         if mode == "plain":
             run(sched, ex)
         else:
-            _, ahead = run_ahead(sched, ex)
-            assert ahead >= 10
+            stats = {}
+            steps, ahead = run_ahead(sched, ex, stats)
+            assert ahead == len(steps) - 1 and stats["mixed"] >= 4      # portions of prompts too
         outs[mode] = {k: r.output for k, r in reqs.items()}
         assert all(r.finish_reason == "length" for r in reqs.values())
         assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == 64
@@ -304,33 +313,35 @@ def test_a_step_decided_ahead_feeds_the_same_tokens():
     assert outs["plain"]["a"] == expected_output(prompts["a"], 12)
 
 
-def test_no_step_is_decided_ahead_when_the_next_one_is_not_plain():
+def test_a_step_ahead_holds_placeholders_and_leaves_out_who_is_sure_to_end():
     ex = AheadExecutor()
     sched = make(ex, max_batched_tokens=8)
-    a = Request("a", list(range(7)), SamplingParams(max_new_tokens=3))
+    a = Request("a", list(range(7)), SamplingParams(max_new_tokens=2))
     b = Request("b", list(range(20, 26)), SamplingParams(max_new_tokens=30))
     sched.add(a)
     batch = sched.schedule()                      # a's prompt: 7 tokens, samples
-    sched.add(b)
-    assert sched.schedule_ahead(batch) is None    # someone waits for admission
-    sched.update(batch, ex.step(batch))
-    batch = sched.schedule()                      # a decodes, b's prompt
-    assert [len(s.tokens) for s in batch] == [1, 6]
     sampled = ex.step(batch)
-    nxt = sched.schedule_ahead(batch)             # a has 1 of 3, gets its second now: the third is still open
-    assert nxt is not None and [(s.request.id, s.start, s.samples) for s in nxt] == [("a", 8, True), ("b", 6, True)]
-    for s in nxt:
-        s.tokens = [sampled[s.request.id]]
+    sched.add(b)
+    assert sched.advance(batch) == batch and a.output == [PLACEHOLDER] and a.num_computed == 7
+    nxt = sched.schedule(ahead=True)              # a decodes the token nobody has seen, b is admitted beside it
+    assert [(s.request.id, s.start, s.tokens, s.samples) for s in nxt] == \
+        [("a", 7, [PLACEHOLDER], True), ("b", 0, list(range(20, 26)), True)]
+    nxt[0].tokens = [sampled["a"]]
     sampled2 = ex.step(nxt)
-    sched.update(batch, sampled)
-    assert sched.schedule_ahead(nxt) is None      # a gets its last token in nxt
-    sched.update(nxt, sampled2)
-    assert a.finish_reason == "length" and len(a.output) == 3
+    assert sched.commit(batch, sampled) == [] and a.output == [sampled["a"]]
+    sched.advance(nxt)                            # a's second token is its last: it gives back what it holds now
+    assert a.status == "finished" and a not in sched.running and ex.manager.live() == ["b"]
+    assert a not in sched.finished and a.output[1] == PLACEHOLDER
+    third = sched.schedule(ahead=True)
+    assert [(s.request.id, s.tokens) for s in third] == [("b", [PLACEHOLDER])]
+    assert sched.commit(nxt, sampled2) == [a] and a.finish_reason == "length" and sched.finished == [a]
+    assert a.output == expected_output(range(7), 2)
 
 
 def test_deciding_ahead_stops_where_pages_run_out():
     """Three pages of four tokens for two requests that need two each: when both want their second
-    page no step is decided ahead, schedule() preempts, and the output is what it would have been."""
+    page no step is decided ahead (and nothing is changed by the attempt), schedule() preempts,
+    and the output is what it would have been."""
     outs = {}
     for mode in ("plain", "ahead"):
         ex = AheadExecutor(num_pages=3)
@@ -341,7 +352,8 @@ def test_deciding_ahead_stops_where_pages_run_out():
         if mode == "plain":
             run(sched, ex)
         else:
-            run_ahead(sched, ex)
+            steps, ahead = run_ahead(sched, ex)
+            assert ahead < len(steps) - 1
         assert sched.num_preemptions >= 1
         outs[mode] = [r.output for r in reqs]
         assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == 3
@@ -363,5 +375,31 @@ def test_a_request_that_ends_while_the_next_step_is_under_way():
     assert len(b.output) <= 30 and b.finish_reason in ("length", "stop")
     want_b = expected_output(range(50, 58), 30)
     assert b.output == want_b[:len(b.output)]
+    assert all(s.request is not a for live in steps[cut + 1:] for s in live)   # the step under way did not count
     assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == 64
     ex.manager.check()
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_scenarios_ahead_equal_plain(seed):
+    """Requests of random lengths over a small pool, with a window group or without, with an
+    end-of-sequence token that some of them hit: the loop that starts steps early produces what the
+    plain loop produces, and gives everything back."""
+    import random
+    rng = random.Random(seed)
+    pages, window = rng.choice([6, 10, 24]), rng.choice([None, 8])
+    budget, seqs = rng.choice([4, 7, 16]), rng.choice([1, 2, 4])
+    spec = [(list(range(100 * i, 100 * i + rng.randrange(1, 14))), rng.randrange(1, 10)) for i in range(rng.randrange(2, 9))]
+    eos = next_token(spec[0][0]) if rng.random() < 0.5 else None
+    outs = {}
+    for mode in ("plain", "ahead"):
+        ex = AheadExecutor(num_pages=pages, window=window)
+        sched = make(ex, max_batched_tokens=budget, max_num_seqs=seqs, eos_token_id=eos)
+        reqs = [Request(i, p, SamplingParams(max_new_tokens=n)) for i, (p, n) in enumerate(spec)]
+        for r in reqs:
+            sched.add(r)
+        (run if mode == "plain" else run_ahead)(sched, ex)
+        outs[mode] = [(r.output, r.finish_reason) for r in reqs]
+        assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == pages and ex.manager.free_slots == 4
+        assert sorted(r.id for r in sched.finished) == list(range(len(spec)))
+    assert outs["plain"] == outs["ahead"]

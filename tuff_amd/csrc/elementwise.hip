@@ -136,3 +136,21 @@ TUFF_EXPORT int tuff_fill_u32(void* p, uint32_t value, long long n, hipStream_t 
     hipLaunchKernelGGL(fill_u32_kernel, grid, block, 0, stream, (uint32_t*)p, value, n);
     return launch_status();
 }
+
+// -------------------------------------------------------------------- scatter
+// dst[idx[i]] = src[idx[n + i]] for i < n, bounds checked (a bad index writes nothing): token ids that
+// a sampling kernel has left on the device go into the next step's token buffer without a trip
+// to the host.
+__global__ void scatter_i32_kernel(int* __restrict__ dst, int n_dst, const int* __restrict__ src, int n_src,
+                                   const int* __restrict__ idx, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int d = idx[i], s = idx[n + i];
+    if (d >= 0 && d < n_dst && s >= 0 && s < n_src) dst[d] = src[s];
+}
+
+TUFF_EXPORT int tuff_scatter_i32(int* dst, int n_dst, const int* src, int n_src, const int* idx, int n, hipStream_t stream) {
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(scatter_i32_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, stream, dst, n_dst, src, n_src, idx, n);
+    return launch_status();
+}

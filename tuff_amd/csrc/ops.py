@@ -31,6 +31,7 @@ _SIGNATURES = {
         "tuff_swiglu": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_cast": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_void_p],
         "tuff_fill_u32": [_c_void_p, ctypes.c_uint32, _c_ll, _c_void_p],
+        "tuff_scatter_i32": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p],
     },
     "gemm_f32": {
         "tuff_gemm_f32": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -196,6 +197,14 @@ def fill_u32(t: torch.Tensor, value: int = 0) -> None:
     if not t.is_cuda or not t.is_contiguous():
         raise KernelError("fill_u32: contiguous GPU tensor required")
     _check(load("elementwise").tuff_fill_u32(t.data_ptr(), value, t.numel(), _stream()), "fill_u32")
+
+
+def scatter_i32(dst: torch.Tensor, src: torch.Tensor, idx: torch.Tensor) -> None:
+    """dst[idx[i]] = src[idx[n + i]] for i < n = len(idx) / 2; all int32 on the GPU."""
+    n = idx.shape[0] // 2
+    _check(load("elementwise").tuff_scatter_i32(_gpu("dst", dst, torch.int32), dst.numel(), _gpu("src", src, torch.int32),
+                                                src.numel(), _gpu("idx", idx, torch.int32, (2 * n,)), n, _stream()),
+           "scatter_i32")
 
 
 # ------------------------------------------------------------------------------ GEMM

@@ -109,9 +109,10 @@ class Engine:
         """Runs one batch.  Returns float32 logits [wanted, vocab] on the device, in the order
         of the entries and of their `want` lists, or None if nothing is wanted.
         Raises OutOfPages (and leaves every request as it was) if the pool is too small.
-        device_tokens (int32 on the device, one per token of the step): the token ids are taken
-        from there, by a copy on the stream, instead of from the entries (whose ids then only
-        stand in); for a caller that starts a step before it has seen the last one's tokens."""
+        device_tokens: for a caller that starts a step before it has seen the last one's tokens.
+        Either an int32 tensor on the device with one id per token of the step, or a triple
+        (tensor, places, sources): token `places[i]` of the step is `tensor[sources[i]]`.  The ids
+        are put in place by a kernel on the stream; the entries' ids at those places only stand in."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         entries = [e for e in entries if len(e.tokens) > 0]
         if not entries:
@@ -141,17 +142,43 @@ class Engine:
             raise
         if device_tokens is not None:
             n = sum(len(e.tokens) for e in entries)
-            if device_tokens.dtype != torch.int32 or device_tokens.shape != (n,) or device_tokens.device != self.device:
+            try:
+                device_tokens = self._check_device_tokens(device_tokens, n)
+            except ValueError:
                 for e in done:
                     self.manager.truncate(e.req_id, self.manager.length(e.req_id) - len(e.tokens))
-                raise ValueError(f"device_tokens must be int32 [{n}] on {self.device}")
+                raise
         self.steps += 1
         if self.use_graphs and all(len(e.tokens) == 1 for e in entries):
             return self._decode_step(entries, device_tokens)
         ctx = build_context(entries, self.manager, self.device, self.model.vocab_size)
-        if device_tokens is not None:
-            ctx.tokens.copy_(device_tokens)
+        self._place_device_tokens(ctx.tokens, device_tokens)
         return self.model.forward(ctx, self.storage.views)
+
+    def _check_device_tokens(self, device_tokens, n: int):
+        """A tensor of all n ids stays; a triple becomes (tensor, index tensor [places | sources])."""
+        if isinstance(device_tokens, torch.Tensor):
+            if device_tokens.dtype != torch.int32 or device_tokens.shape != (n,) or device_tokens.device != self.device:
+                raise ValueError(f"device_tokens must be int32 [{n}] on {self.device}")
+            return device_tokens
+        src, places, sources = device_tokens
+        if src.dtype != torch.int32 or src.dim() != 1 or src.device != self.device or len(places) != len(sources):
+            raise ValueError(f"device_tokens: an int32 vector on {self.device} and as many places as sources are needed")
+        if any(not 0 <= p < n for p in places) or any(not 0 <= q < src.shape[0] for q in sources):
+            raise ValueError("device_tokens: a place or a source is out of range")
+        if not places:
+            return None
+        idx = torch.tensor(list(places) + list(sources), dtype=torch.int32).pin_memory().to(self.device, non_blocking=True)
+        return src, idx
+
+    @staticmethod
+    def _place_device_tokens(tokens: torch.Tensor, device_tokens) -> None:
+        if device_tokens is None:
+            return
+        if isinstance(device_tokens, torch.Tensor):
+            tokens.copy_(device_tokens)
+        else:
+            ops.scatter_i32(tokens, device_tokens[0], device_tokens[1])
 
     # --------------------------------------------------------------- recorded decode
     GRAPH_TABLE_BUCKET = 64          # block tables of recorded steps are padded to multiples of this
@@ -207,8 +234,7 @@ class _RecordedStep:
         self.pinned.numpy()[:] = p.buf
         self.dev.copy_(self.pinned, non_blocking=True)
         self.copied.record()
-        if device_tokens is not None:
-            self.ctx.tokens.copy_(device_tokens)
+        Engine._place_device_tokens(self.ctx.tokens, device_tokens)
 
     def record(self, forward) -> None:
         torch.cuda.synchronize()

@@ -18,7 +18,7 @@ from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .batch import StepEntry
 from .engine import Engine
-from .scheduler import Request, Scheduler
+from .scheduler import PLACEHOLDER, Request, Scheduler
 
 
 @dataclasses.dataclass
@@ -97,9 +97,11 @@ class LLM:
 class Loop:
     """The run loop, one step a call: scheduler -> step -> sampler -> scheduler.
 
-    While the requests only decode, the next step is started before the tokens of the
-    current one have reached the host: it takes them from the sampler's output on the device
-    (`run_ahead`).  The host then accounts for a step while the GPU runs the next one.
+    The next step is decided and started before the tokens of the current one have reached the
+    host (`run_ahead`): a request that decodes takes its token from the sampler's output on the
+    device.  The host then decides, packs and accounts while the GPU runs.  Not where the next
+    step would have to preempt somebody, and not while a sampler needs the tokens on the host
+    (a penalty over the request's history).
     Requests may be added to the scheduler between calls."""
 
     def __init__(self, llm: "LLM", sched: Scheduler):
@@ -107,9 +109,25 @@ class Loop:
         self.under_way = None                             # a step started ahead: (batch, sampling, pending)
         self.steps = self.tokens = self.ahead_steps = 0
 
-    def _start(self, batch, device_tokens=None):
-        entries = [StepEntry(s.request.id, s.tokens, [len(s.tokens) - 1] if s.samples else [])
-                   for s in batch]
+    def _start(self, batch, before=None):
+        """before: (requests that draw a token in the step before, its sampler launch)."""
+        entries, places, sources, at = [], [], [], 0
+        row = {id(r): i for i, r in enumerate(before[0])} if before is not None else {}
+        for s in batch:
+            toks = s.tokens
+            if PLACEHOLDER in toks:
+                if len(toks) != 1 or before is None:
+                    raise RuntimeError("a token that is not known yet can only be fed alone, and from the step before")
+                places.append(at)
+                sources.append(row[id(s.request)])
+                toks = [0]
+            entries.append(StepEntry(s.request.id, toks, [len(toks) - 1] if s.samples else []))
+            at += len(toks)
+        device_tokens = None
+        if places:
+            out = before[1].out
+            whole = len(places) == at == out.shape[0] and sources == places
+            device_tokens = out if whole else (out, places, sources)
         logits = self.llm.engine.step(entries, device_tokens)
         sampling = [s.request for s in batch if s.samples]
         pending = self.llm.sampler.launch(logits, [r.sampler for r in sampling]) if sampling else None
@@ -131,17 +149,16 @@ class Loop:
         else:
             batch, sampling, pending = self.under_way
             self.under_way = None
-        if self.llm.run_ahead and pending is not None and len(sampling) == len(batch) \
-                and not any(sampler.needs_history(r.sampler) for r in sampling):
-            nxt = sched.schedule_ahead(batch)
-            if nxt is not None:
-                self.under_way = (nxt,) + self._start(nxt, pending.out)
+        live = sched.advance(batch)
+        if self.llm.run_ahead and not any(sampler.needs_history(r.sampler) for r in sampling):
+            nxt = sched.schedule(ahead=True)
+            if nxt:
+                self.under_way = (nxt,) + self._start(nxt, (sampling, pending))
                 self.ahead_steps += 1
         sampled = {}
         if pending is not None:
             sampled = {r.id: t for r, t in zip(sampling, pending.tokens())}
-        live = [s for s in batch if s.request.status != "finished"]
-        sched.update(batch, sampled)
+        sched.commit(batch, sampled)
         self.steps += 1
         self.tokens += sum(len(s.tokens) for s in live)
         return live, {s.request.id: sampled[s.request.id] for s in live if s.samples}

@@ -3,7 +3,12 @@
 Every call to `schedule()` decides one step: requests that are decoding get their one token
 first, then prompts are continued and new requests admitted, in arrival order, while the
 token budget, the state slots and the pages last; the last prompt portion is cut to fit the
-budget.  `update()` takes the sampled tokens, finishes requests and frees what they held.
+budget.  `update()` takes the sampled tokens, finishes requests and frees what they held.  It has
+two halves for a caller that starts the next step before it has seen this one's tokens:
+`advance()` accounts for a step that has been started (positions move on, every request that draws
+a token gets a PLACEHOLDER at the end of its output, requests that end with this token whatever it
+is are finished), `commit()` puts the tokens where the placeholders are and finishes requests at
+an end-of-sequence token.  Between the two, `schedule(ahead=True)` decides the next step.
 
 When pages run out: a waiting request is simply not admitted yet.  If a running request
 cannot get the pages for its next tokens, the most recently admitted running request is
@@ -27,6 +32,7 @@ from ..cache.manager import CacheManager
 from ..sampling.params import SamplerState, SamplingParams
 
 WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
+PLACEHOLDER = -1                 # in Request.output: a token that has been drawn on the device and not yet seen
 
 
 @dataclasses.dataclass(eq=False)           # a request is itself: lists of requests are searched by identity
@@ -63,6 +69,9 @@ class Scheduled:
     start: int                       # first position fed in this step
     tokens: list
     samples: bool                    # the step reaches the request's last token: draw the next
+    counted: bool = True             # advance(): the request was live when the step was accounted
+    slot: int = -1                   # advance(): where in Request.output the drawn token goes
+    finishes: bool = False           # advance(): the request ends with this token, whatever it is
 
 
 class Scheduler:
@@ -154,7 +163,12 @@ class Scheduler:
     def _total_pages(self) -> list[int]:
         return [g.pool.num_pages for g in self.manager.groups]
 
-    def schedule(self) -> list[Scheduled]:
+    def schedule(self, ahead: bool = False) -> Optional[list[Scheduled]]:
+        """The next step.  ahead: the step before has been through advance() and not through
+        commit(); tokens not yet seen appear as PLACEHOLDER in Scheduled.tokens (always as the one
+        token of a decoding request).  Nobody can be preempted then, since a request's tokens must
+        be known to compute it again: where a running request lacks pages the answer is None, and
+        nothing has been changed."""
         budget = self.max_batched_tokens
         promised = [0] * len(self.manager.groups)
         out: list[Scheduled] = []
@@ -167,6 +181,8 @@ class Scheduler:
                 continue
             n = min(req.remaining(), budget)
             while not self._fits(req, n, promised):
+                if ahead:
+                    return None
                 victim = self.running[-1]
                 if victim is req and len(self.running) == 1:
                     # alone and still too large: shrink the portion, or give up
@@ -225,56 +241,60 @@ class Scheduler:
             budget -= n
         return out
 
-    def schedule_ahead(self, prev: list[Scheduled]) -> Optional[list[Scheduled]]:
-        """The step after `prev`, decided before prev's tokens are known: every request of prev
-        feeds the token it is about to get (Scheduled.tokens holds a stand-in).  Only in the
-        plain case: prev draws a token for every running request, none of them can finish by
-        length with it, nobody waits for admission, and the pages for one more token each are
-        free.  Otherwise None: decide with schedule() once prev has been accounted.
-        A request that does finish with prev's token (end of sequence) still runs in the step
-        returned here; update() ignores it."""
-        if self.waiting or not prev or len(prev) != len(self.running):
-            return None
-        promised = [0] * len(self.manager.groups)
-        out = []
-        for s in prev:
-            req = s.request
-            if not s.samples or req.status != RUNNING:
-                return None
-            n_out = len(req.output) + 1                      # with the token prev is drawing
-            if n_out >= req.params.max_new_tokens:
-                return None
-            if self.max_model_len is not None and len(req.prompt) + n_out >= self.max_model_len:
-                return None
-            if not self._fits(req, 1, promised):
-                return None
-            self._promise(req, 1, promised)
-            out.append(Scheduled(req, s.start + len(s.tokens), [0], True))
-        return out
-
     def update(self, scheduled: list[Scheduled], sampled: dict) -> list[Request]:
         """sampled: {request id: token} for every Scheduled with samples=True.
         Returns the requests that finished in this step."""
-        done = []
+        self.advance(scheduled)
+        return self.commit(scheduled, sampled)
+
+    def advance(self, scheduled: list[Scheduled]) -> list[Scheduled]:
+        """Accounts for a step that has been started and whose tokens are not known yet.
+        Returns the entries that count: those whose requests had not finished meanwhile (a step
+        that was started early may hold a request that ended with the token before)."""
+        live = []
         for s in scheduled:
             req = s.request
-            if req.status == FINISHED:                       # finished while this step was under way
+            s.counted = req.status != FINISHED
+            if not s.counted:
                 continue
+            live.append(s)
             req.num_computed += len(s.tokens)
             if not s.samples:
                 continue
-            tok = int(sampled[req.id])
-            req.output.append(tok)
+            s.slot = len(req.output)
+            req.output.append(PLACEHOLDER)
             reason = None
-            if self.eos_token_id is not None and tok == self.eos_token_id and not req.params.ignore_eos:
-                reason = "stop"
-            elif len(req.output) >= req.params.max_new_tokens:
+            if len(req.output) >= req.params.max_new_tokens:
                 reason = "length"
             elif self.max_model_len is not None and len(req.prompt) + len(req.output) >= self.max_model_len:
                 reason = "context"
             if reason:
+                # what it holds can go back now: whoever takes it runs after this step
+                s.finishes = True
                 self.running.remove(req)
                 self._end(req.id)
-                self._finish(req, reason)
+                req.status, req.finish_reason = FINISHED, reason
+        return live
+
+    def commit(self, scheduled: list[Scheduled], sampled: dict) -> list[Request]:
+        """The tokens of a step that advance() has accounted for.  Returns the requests that
+        finished in this step."""
+        done = []
+        for s in scheduled:
+            if not (s.counted and s.samples):
+                continue
+            req = s.request
+            tok = int(sampled[req.id])
+            req.output[s.slot] = tok
+            stop = self.eos_token_id is not None and tok == self.eos_token_id and not req.params.ignore_eos
+            if s.finishes:
+                if stop:
+                    req.finish_reason = "stop"
+                self.finished.append(req)
+                done.append(req)
+            elif stop and req.status == RUNNING:
+                self.running.remove(req)
+                self._end(req.id)
+                self._finish(req, "stop")
                 done.append(req)
         return done
