@@ -43,7 +43,9 @@ def test_gemm_f32(gpu, M, N, K):
                                    (33, 100, 2048), (64, 2048, 8192), (20, 64, 1024), (48, 200, 512), (16, 24, 4096),
                                    (8, 6144, 2048),
                                    # each shape of block of the tiled kernel, with ragged edges and a partial last step
-                                   (1100, 8200, 72), (1030, 8190, 136), (1100, 4001, 200), (257, 129, 520)])
+                                   (1100, 8200, 72), (1030, 8190, 136), (1100, 4001, 200), (257, 129, 520),
+                                   # the same with K a multiple of 64: operands go straight into LDS
+                                   (1100, 8200, 192), (1030, 8190, 128), (1100, 4001, 256), (257, 129, 512), (100, 40, 64)])
 def test_gemm_bf16(gpu, M, N, K):
     from tuff_amd.csrc import ops
     x, w = _r(M, K, seed=4, dtype=torch.bfloat16), _r(N, K, seed=5, dtype=torch.bfloat16)
@@ -73,7 +75,7 @@ def test_gemm_bf16(gpu, M, N, K):
 @pytest.mark.parametrize("M,N,K", [(1, 32, 64), (8, 512, 240), (16, 6144, 2048), (5, 200, 96), (64, 384, 256),
                                    (40, 2050, 2048), (300, 130, 136), (2048, 512, 128), (1100, 8200, 72),
                                    (200, 384, 1024), (72, 4100, 2048),
-                                   (1030, 8202, 136), (1100, 4002, 200)])
+                                   (1030, 8202, 136), (1100, 4002, 200), (1030, 8202, 128), (1100, 4002, 192)])
 def test_gemm_bf16_swiglu_epilogue(gpu, M, N, K):
     """Rows of w are gate and up rows interleaved; the output is silu(gate) * up."""
     from tuff_amd.csrc import ops

@@ -8,7 +8,8 @@
 // the shapes of a decode step, the run-wise reads are 17 % faster.
 //
 // Three kernels, chosen by M on the host:
-//  * tiled     M > 64: 128x128 or 256x256 block tiles staged through LDS (compute bound);
+//  * tiled     M > 64: 128x128 or 256x256 block tiles staged through LDS (compute bound), in two
+//    forms: operands loaded straight into LDS (K a multiple of 64) or through registers (other K);
 //  * skinny64  16 < M <= 64: a workgroup owns 64 rows of W, one MFMA column tile a wave; the
 //    activations of a K chunk are staged once in LDS for all four waves (bandwidth bound);
 //  * skinny16  M <= 16: a workgroup owns 16 rows of W; its four waves split K (bandwidth bound).
@@ -243,6 +244,162 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_tiled_kernel
             }
         });
     }
+
+    if (gridDim.z > 1) {
+        float* mine = ws + (long long)blockIdx.z * M * N;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                store_quad<OUT_F32>(mine, m0 + wm + i * 16 + r16, n0 + wn + j * 16 + g * 4, M, N, acc[i][j]);
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            store_quad<MODE>(Y, m0 + wm + i * 16 + r16, n0 + wn + j * 16 + g * 4, M, N, acc[i][j]);
+}
+
+// The same product with the operands going from memory straight into LDS (global_load_lds_dwordx4),
+// without a stop in registers; used where K is a multiple of 64.  A wave's load instruction fills
+// 1 KB of LDS, lane l the 16 bytes at 16 l.  X keeps the swizzled row-major layout above: an
+// instruction covers eight rows of 128 bytes, and the lane that fills chunk position p of row r
+// fetches chunk p ^ (r % 8) of that row.  W lies in LDS as in memory, one block of 1 KB per (row
+// tile, k 32): the fragment of lane l is at 16 l.  STAGES buffers of a step of 64 k each: the
+// operands of STAGES - 1 steps are on their way while one is multiplied.
+// Measured against the kernel above (M = 2048; N x K): 3072 x 2048 42.8 -> 32.9 us, 2048 x 2048
+// 35.1 -> 27.4, 2048 x 8192 102.7 -> 81.3, 16384 x 2048 157.6 -> 148.6, 6144 x 2048 69.0 -> 61.2.
+// With all CUs busy and random operands the clock, not the instruction stream, sets the pace: the
+// same loop over constant data runs a quarter faster.
+template <int VM>
+__device__ __forceinline__ void wait_loads_and_lds() {               // s_waitcnt vmcnt(VM) lgkmcnt(0)
+    static_assert(VM >= 0 && VM < 64, "vmcnt has six bits");
+    __builtin_amdgcn_s_waitcnt((VM & 15) | ((VM >> 4) << 14) | 0x0070);
+}
+
+template <int TM, int TN, int WAVES_M, int WAVES_N, int STAGES, int MODE>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_dma_kernel(
+        const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, int M, int N, int K,
+        int steps_per_slice, float* __restrict__ ws) {
+    constexpr int NW = WAVES_M * WAVES_N;
+    constexpr int BM = 16 * TM * WAVES_M, BN = 16 * TN * WAVES_N;
+    constexpr int IA = BM / 8 / NW, IB = BN / 8 / NW;                  // load instructions of X and of W a wave issues a step
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "whole instructions");
+    extern __shared__ __attribute__((aligned(16))) bf16_t tiles[];       // [STAGES][BM * TBK] of X then [STAGES][BN * TBK] of W
+    bf16_t* As = tiles;
+    bf16_t* Bs = tiles + STAGES * BM * TBK;
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const int wm = (wave / WAVES_N) * 16 * TM, wn = (wave % WAVES_N) * 16 * TN;
+    const int r16 = lane % 16, g = lane / 16;
+    const long long m0 = (long long)blockIdx.y * BM, n0 = (long long)blockIdx.x * BN;
+
+    f32x4 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int kb = K / 32;
+    const bf16_t* Xb = X + m0 * K;
+    const bf16_t* Wb = W + (n0 / 16) * (long long)kb * 512;
+    const int last_a = (int)min((long long)BM - 1, (long long)M - 1 - m0);
+    const int last_tile = (int)min((long long)BN / 16 - 1, (N - 1 - n0) / 16);
+    // instruction q of X (q = wave + NW i) fills rows 8 q .. 8 q + 7; instruction q of W fills block q % 2 of row tile q / 2
+    unsigned offa[IA], offb[IB];
+#pragma unroll
+    for (int i = 0; i < IA; ++i)
+        offa[i] = (unsigned)min((wave + NW * i) * 8 + lane / 8, last_a) * (unsigned)K + (((lane % 8) ^ (lane / 8)) * 8);
+#pragma unroll
+    for (int i = 0; i < IB; ++i) {
+        const int q = wave + NW * i;
+        offb[i] = ((unsigned)min(q / 2, last_tile) * (unsigned)kb + q % 2) * 512u + lane * 8;
+    }
+    const int nk = K / TBK;
+    const int kt_begin = blockIdx.z * steps_per_slice, kt_end = min(nk, kt_begin + steps_per_slice);
+
+    auto issue = [&](int buf, int kt) {
+        const bf16_t* xs = Xb + kt * TBK;
+        const bf16_t* wsrc = Wb + (unsigned)(kt * 2) * 512u;
+#pragma unroll
+        for (int i = 0; i < IA; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xs + offa[i]),
+                                             (__attribute__((address_space(3))) void*)(As + buf * BM * TBK + (wave + NW * i) * 512), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < IB; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wsrc + offb[i]),
+                                             (__attribute__((address_space(3))) void*)(Bs + buf * BN * TBK + (wave + NW * i) * 512), 16, 0, 0);
+    };
+    const int fa0 = swz(wm + r16, g), fa1 = swz(wm + r16, 4 + g);
+    const int fb = (wn / 16) * 1024 + lane * 8;                        // block h of MFMA tile j: + (2 j + h) * 512
+
+    // The fragments of half a step (k 0..31 or 32..63: TM of X, TN of W) are read at once into one of
+    // two register sets, half a step before the MFMAs that use them: while one set is multiplied the
+    // other is on its way from LDS, also across the barrier between two steps.
+    bf16x8 fx[2][TM], fw[2][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fx[1][i] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fw[1][j] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    auto read_half = [&](auto set_tag, int buf, auto half_tag) {
+        constexpr int set = decltype(set_tag)::value, h = decltype(half_tag)::value;
+        const bf16_t* Ab = As + buf * BM * TBK + (h ? fa1 : fa0);
+        const bf16_t* Bb = Bs + buf * BN * TBK + fb + h * 512;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fw[set][j] = *(const bf16x8*)(Bb + 2 * j * 512);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fx[set][i] = *(const bf16x8*)(Ab + i * 16 * TBK);
+    };
+    auto mult = [&](auto set_tag) {
+        constexpr int set = decltype(set_tag)::value;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = mfma16(fw[set][j], fx[set][i], acc[i][j]);
+    };
+    // asks the instruction scheduler to spread the LDS reads of a half step evenly among its MFMAs
+    auto spread = [&]() {
+        constexpr int R = TM + TN, Q = TM * TN;
+        static_for<R>([&](auto r) {
+            constexpr int n = Q / R + (decltype(r)::value < Q % R ? 1 : 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);         // one LDS read
+            __builtin_amdgcn_sched_group_barrier(0x008, n, 0);         // n MFMAs
+        });
+    };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+
+    // Step kt lives in buffer (kt - kt_begin) % STAGES.  Before step kt is multiplied the loads of
+    // steps kt .. kt + STAGES - 2 are under way; a wave waits until all but those of the later steps
+    // have landed, the barrier then says the same of everybody's and that nobody reads the buffer
+    // of step kt - 1 any more, which the loads of step kt + STAGES - 1 go into.
+    static_for<STAGES - 1>([&](auto s) {
+        constexpr int st = decltype(s)::value;
+        if (kt_begin + st < kt_end) issue(st, kt_begin + st);
+    });
+    for (int kt0 = kt_begin; kt0 < kt_end; kt0 += STAGES) {
+        static_for<STAGES>([&](auto u) {
+            constexpr int buf = decltype(u)::value;
+            const int kt = kt0 + buf;
+            if (kt < kt_end) {
+                const int later = min(STAGES - 2, kt_end - 1 - kt);      // steps after kt whose loads are under way
+                bool waited = false;
+                static_for<STAGES - 1>([&](auto l) {
+                    constexpr int n = decltype(l)::value;
+                    if (!waited && later == n) { wait_loads_and_lds<n * (IA + IB)>(); waited = true; }
+                });
+                __builtin_amdgcn_s_barrier();
+                if (kt + STAGES - 1 < kt_end) issue((buf + STAGES - 1) % STAGES, kt + STAGES - 1);
+                read_half(S0(), buf, S0());
+                mult(S1());                                            // the second half of the step before (zeros at first)
+                spread();
+                read_half(S1(), buf, S1());
+                mult(S0());
+                spread();
+            }
+        });
+    }
+    if (kt_begin < kt_end) mult(S1());
 
     if (gridDim.z > 1) {
         float* mine = ws + (long long)blockIdx.z * M * N;
@@ -819,9 +976,26 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
             hipLaunchKernelGGL(kern, dim3(ceil_div(N, bn), ceil_div(M, bm), t.slices), dim3(64 * WM * WN), lds, stream, \
                                X, W, Y, M, N, K, t.steps_per_slice, ws); \
         } while (0)
-        if (t.shape == 0) TILED(8, 4, 2, 4, 1);
+#define TILED_DMA(TM, TN, WM, WN, STAGES) do { \
+            auto kern = gemm_bf16_dma_kernel<TM, TN, WM, WN, STAGES, MODE>; \
+            constexpr int bm = 16 * TM * WM, bn = 16 * TN * WN, lds = STAGES * (bm + bn) * TBK * 2; \
+            static bool set = false; \
+            if (!set) { \
+                if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -1; \
+                set = true; \
+            } \
+            hipLaunchKernelGGL(kern, dim3(ceil_div(N, bn), ceil_div(M, bm), t.slices), dim3(64 * WM * WN), lds, stream, \
+                               X, W, Y, M, N, K, t.steps_per_slice, ws); \
+        } while (0)
+        if (K % TBK == 0) {
+            if (t.shape == 0) TILED_DMA(8, 4, 2, 4, 2);
+            else if (t.shape == 1) TILED_DMA(4, 2, 2, 4, 2);
+            else TILED_DMA(4, 2, 2, 4, 4);
+        }
+        else if (t.shape == 0) TILED(8, 4, 2, 4, 1);
         else if (t.shape == 1) TILED(4, 2, 2, 4, 1);
         else TILED(4, 2, 2, 4, 4);
+#undef TILED_DMA
 #undef TILED
         if (t.slices > 1) {
             int rc = launch_status();
