@@ -193,6 +193,59 @@ def test_recorded_decode_steps_equal_eager_steps(gpu, dtype):
     util.assert_close(dtype, got["y"][mask], full[mask], "y")
 
 
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("A", "bfloat16"), ("B", "bfloat16")])
+def test_steps_with_portions_recorded_in_sections_equal_eager_steps(gpu, name, dtype, monkeypatch):
+    """A number of tokens that keeps coming is recorded as graphs with the attention and the head run
+    eagerly in between.  Steps of that size with other requests, other portions, other wanted rows and
+    other places in the cache, with steps of other sizes and of single tokens in between, give exactly
+    what an engine that records nothing gives; so do the tokens decoded afterwards out of the cache
+    and the conv states those steps left."""
+    from tuff_amd.engine.engine import Engine
+    monkeypatch.setattr(Engine, "SECTIONS_MIN_TOKENS", 40)
+    V = util.CONFIGS[name][0]["vocab_size"]
+    reqs = {k: util.rand_tokens(n, V, 10 + i) for i, (k, n) in enumerate(
+        [("a", 300), ("b", 220), ("c", 130), ("d", 90), ("e", 75)])}
+    steps, fed = [], {k: 0 for k in reqs}
+    def portion(rid, n, want=True):
+        t = reqs[rid][fed[rid]:fed[rid] + n]
+        fed[rid] += n
+        return {"id": rid, "tokens": t, "want": ([len(t) - 1] if want else [])}
+    def add(entries, end=()):
+        assert all(e["tokens"] for e in entries)
+        steps.append({"step": len(steps), "entries": entries, "end": list(end)})
+    T = 70
+    add([portion("a", T)])                                                # T tokens: first
+    add([portion("a", 40), portion("b", 30, want=False)])                 # second
+    add([portion("b", 69), portion("c", 1)])                              # third: recorded and replayed
+    add([portion("c", 1), portion("a", 1), portion("b", 1)])              # single tokens in between
+    add([portion("a", 1), portion("c", 60), portion("b", 1), portion("d", 8, want=False)])   # replay, four requests
+    add([portion("d", 33)])                                               # another size
+    add([portion("e", 2, want=False), portion("a", 1), portion("b", 60), portion("c", 1), portion("d", 6)])
+    add([portion("e", 70)], end=["e"])                                    # e's pages and slot go back ...
+    reqs["f"] = util.rand_tokens(100, V, 99); fed["f"] = 0
+    add([portion("f", 66), portion("a", 1), portion("c", 3)])             # ... and are used again
+    for _ in range(4):
+        add([portion(k, 1) for k in "abcdf"])
+    add([portion("a", 64), portion("f", 6)], end=list("abcdf"))
+    counts = [sum(len(e["tokens"]) for e in s["entries"]) for s in steps]
+    assert counts.count(T) == 8
+    eager = make_engine(name, dtype, max_tokens=1024, use_graphs=False, max_requests=5)
+    want = util.run_plan(eager, steps)
+    eng = make_engine(name, dtype, max_tokens=1024, max_requests=5)
+    assert eng.record_portions
+    got = util.run_plan(eng, steps)
+    assert eng.section_replays == 6 and eager.section_replays == 0
+    eng.manager.check()
+    for rid in reqs:
+        a, b = got[rid], want[rid]
+        assert torch.equal(torch.isnan(a[:, 0]), torch.isnan(b[:, 0]))
+        mask = ~torch.isnan(b[:, 0])
+        assert torch.equal(a[mask], b[mask]), rid
+    full = util.plain_logits(name, reqs["b"][:fed["b"]], stored_for(dtype))
+    mask = ~torch.isnan(got["b"][:, 0])
+    util.assert_close(dtype, got["b"][mask], full[mask], "b")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_token_ids_taken_from_the_device(gpu, dtype):
     """A step may take some of its token ids from a vector on the device (the sampler's output of

@@ -110,6 +110,7 @@ __global__ void shortconv_state_kernel(const T* __restrict__ bcx, float* __restr
     const int c = blockIdx.y * blockDim.x + threadIdx.x;
     if (c >= d) return;
     const int t0 = q_start[r], n = q_len[r];
+    if (n <= 0) return;                          // an entry without tokens (padding of a recorded step) owns no state
     float* st = state + (long long)state_slot[r] * (K - 1) * d;
     float tmp[MAX_TAPS];
     for (int j = 0; j < K - 1; ++j) {

@@ -46,6 +46,15 @@ class StepContext:
     max_q_len: int = 1
     max_ctx_len: int = 1           # an upper bound of every position + 1 of the step
     host: dict = dataclasses.field(default_factory=dict)     # 'q_len', 'ctx_len' (numpy) and what parts cache
+    recorder: object = None        # set while a step is recorded in sections
+
+    def run_eagerly(self, fn) -> None:
+        """fn(ctx) now; where the step is being recorded in sections, fn is kept instead and runs at
+        every replay, between the graphs of what came before and after it, with that step's ctx."""
+        if self.recorder is None:
+            fn(self)
+        else:
+            self.recorder.eager(fn)
 
 
 @dataclasses.dataclass
@@ -151,7 +160,9 @@ def context_on(dev: torch.Tensor, p: PackedStep, max_ctx_len: Optional[int] = No
                        q_start=sl(3), q_len=sl(4), ctx_len=sl(5), state_slot=sl(6), logit_rows=sl(7),
                        req_info=sl(8 + 2 * p.n_groups).view(p.R, 4), groups=groups, max_q_len=p.max_q_len,
                        max_ctx_len=max_ctx_len if max_ctx_len is not None else p.max_ctx_len,
-                       host={"q_len": p.q_len, "ctx_len": p.ctx_len, "logit_rows_identity": p.logit_rows_identity})
+                       host={"q_len": p.q_len, "ctx_len": p.ctx_len, "logit_rows_identity": p.logit_rows_identity,
+                             "packed": {name: p.buf[int(offs[i]):int(offs[i + 1])] for i, name in
+                                        ((0, "tokens"), (2, "req_of_token"), (3, "q_start"), (4, "q_len"), (6, "state_slot"))}})
 
 
 def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int) -> StepContext:

@@ -68,6 +68,10 @@ class Engine:
         self.use_graphs = bool(use_graphs) and model.graph_safe()
         self._graphs: dict = {}
         self.graph_replays = 0
+        self.record_portions = self.use_graphs and model.records_portions()
+        self._sectioned: dict = {}
+        self._sectioned_seen: dict = {}
+        self.section_replays = 0
 
     # ---------------------------------------------------------------- construction
     @classmethod
@@ -152,6 +156,8 @@ class Engine:
         if self.use_graphs and all(len(e.tokens) == 1 for e in entries):
             return self._decode_step(entries, device_tokens)
         ctx = build_context(entries, self.manager, self.device, self.model.vocab_size)
+        if self.record_portions and ctx.T >= self.SECTIONS_MIN_TOKENS and ctx.R <= self.manager.num_slots:
+            return self._portion_step(ctx, device_tokens)
         self._place_device_tokens(ctx.tokens, device_tokens)
         return self.model.forward(ctx, self.storage.views)
 
@@ -179,6 +185,43 @@ class Engine:
             tokens.copy_(device_tokens)
         else:
             ops.scatter_i32(tokens, device_tokens[0], device_tokens[1])
+
+    # ------------------------------------------------------- steps recorded in sections
+    SECTIONS_MIN_TOKENS = 128        # below, the products choose their kernels by more than the number of rows
+    SECTIONS_RECORD_AT = 3           # a number of tokens is recorded when it comes for this time
+    MAX_SECTIONED = 4
+
+    def _portion_step(self, ctx, device_tokens=None) -> Optional[torch.Tensor]:
+        """A step with prompt portions.  What its kernels' launches depend on outside of the
+        sections that parts run eagerly (ctx.run_eagerly) is the number of tokens alone, so a
+        number of tokens that keeps coming (a scheduler fills its budget) is recorded once: graphs
+        of the stretches between those sections, replayed with the sections run in between."""
+        rec = self._sectioned.get(ctx.T)
+        if rec is None:
+            seen = self._sectioned_seen[ctx.T] = self._sectioned_seen.get(ctx.T, 0) + 1
+            if seen < self.SECTIONS_RECORD_AT:
+                self._place_device_tokens(ctx.tokens, device_tokens)
+                return self.model.forward(ctx, self.storage.views)
+            if len(self._sectioned) >= self.MAX_SECTIONED:
+                self._sectioned.pop(next(iter(self._sectioned)))
+            rec = _SectionedStep(ctx.T, self.manager.num_slots, self.device)
+            try:
+                rec.record(ctx, lambda c: self.model.forward(c, self.storage.views))
+            except Exception as e:                         # noqa: BLE001 - recording is an optimisation
+                import sys
+                print(f"[tuff_amd] recording a step of {ctx.T} tokens in sections failed "
+                      f"({type(e).__name__}: {e}); continuing without", file=sys.stderr)
+                self.record_portions = False
+                self._sectioned.clear()
+                self._place_device_tokens(ctx.tokens, device_tokens)
+                return self.model.forward(ctx, self.storage.views)
+            self._sectioned[ctx.T] = rec
+        else:
+            self._sectioned[ctx.T] = self._sectioned.pop(ctx.T)       # most recently used last
+        merged = rec.refresh(ctx)
+        self._place_device_tokens(merged.tokens, device_tokens)
+        self.section_replays += 1
+        return rec.replay(merged)
 
     # --------------------------------------------------------------- recorded decode
     GRAPH_TABLE_BUCKET = 64          # block tables of recorded steps are padded to multiples of this
@@ -216,6 +259,91 @@ class Engine:
         g.graph.replay()
         self.graph_replays += 1
         return g.logits
+
+
+class _SectionedStep:
+    """A step of T tokens recorded as graphs with eager sections between them.
+
+    What the graphs read of the step lies in one persistent buffer, [tokens T | req_of_token T |
+    q_start | q_len | state_slot], the three per-request arrays padded to the most requests a step
+    can hold (q_len 0 beyond the step's own); every other field of a step's context is the step's own.
+    """
+
+    def __init__(self, T: int, max_requests: int, device):
+        self.T, self.R = T, max_requests
+        n = 2 * T + 3 * max_requests
+        self.pinned = torch.empty(n, dtype=torch.int32, pin_memory=True)
+        self.dev = torch.empty(n, dtype=torch.int32, device=device)
+        self.copied = torch.cuda.Event()
+        self.pool = torch.cuda.graph_pool_handle()
+        self.program: list = []                # graphs and functions of a context, in order
+        self._graph = None
+        self._capture = None
+
+    def _views(self):
+        T, R, d = self.T, self.R, self.dev
+        return dict(tokens=d[:T], req_of_token=d[T:2 * T], q_start=d[2 * T:2 * T + R],
+                    q_len=d[2 * T + R:2 * T + 2 * R], state_slot=d[2 * T + 2 * R:2 * T + 3 * R])
+
+    def refresh(self, ctx):
+        """Brings the persistent buffer up to this step (one copy on the stream, out of what the
+        step's own context was packed from) and returns the step's context over it."""
+        import dataclasses
+        T, R, r = self.T, self.R, ctx.R
+        packed = ctx.host["packed"]
+        self.copied.synchronize()                           # the last copy out of `pinned` is done
+        buf = self.pinned.numpy()
+        buf[:T] = packed["tokens"]
+        buf[T:2 * T] = packed["req_of_token"]
+        buf[2 * T:] = 0
+        buf[2 * T:2 * T + r] = packed["q_start"]
+        buf[2 * T + R:2 * T + R + r] = packed["q_len"]
+        buf[2 * T + 2 * R:2 * T + 2 * R + r] = packed["state_slot"]
+        self.dev.copy_(self.pinned, non_blocking=True)
+        self.copied.record()
+        return dataclasses.replace(ctx, **self._views())
+
+    # -- recording: nothing runs; the eager sections are only noted
+    def _begin(self) -> None:
+        self._graph = torch.cuda.CUDAGraph()
+        self._capture = torch.cuda.graph(self._graph, pool=self.pool)
+        self._capture.__enter__()
+
+    def _end(self) -> None:
+        import warnings
+        with warnings.catch_warnings(record=True) as caught:
+            warnings.simplefilter("always")
+            self._capture.__exit__(None, None, None)
+        if not any("Graph is empty" in str(w.message) for w in caught):    # e.g. nothing after the last section
+            self.program.append(self._graph)
+        self._graph = self._capture = None
+
+    def eager(self, fn) -> None:
+        self._end()
+        self.program.append(fn)
+        self._begin()
+
+    def record(self, ctx, forward) -> None:
+        import dataclasses
+        merged = dataclasses.replace(ctx, recorder=self, host=dict(ctx.host), **self._views())
+        torch.cuda.synchronize()
+        self._begin()
+        try:
+            forward(merged)
+        except BaseException:
+            self._capture.__exit__(None, None, None)
+            self._graph = self._capture = None
+            raise
+        self._end()
+
+    def replay(self, ctx):
+        out = None
+        for piece in self.program:
+            if isinstance(piece, torch.cuda.CUDAGraph):
+                piece.replay()
+            else:
+                out = piece(ctx)
+        return out
 
 
 class _RecordedStep:

@@ -98,6 +98,9 @@ class DecoderModel:
     def graph_safe(self) -> bool:
         return all(b.graph_safe for b in self.blocks) and self.final_norm.graph_safe
 
+    def records_portions(self) -> bool:
+        return self.graph_safe() and all(getattr(b, "records_portions", False) for b in self.blocks)
+
     def num_parameters(self) -> int:
         n = 0
         for d in self.weight_decls():
@@ -132,13 +135,7 @@ class DecoderModel:
         rt = self.rt
         x = torch.empty(ctx.T, self.hidden_size, dtype=torch.float32, device=rt.device)
         ops.embed_rows(self.embedding, ctx.tokens, x)
-        all_rows = ctx.n_logits == ctx.T and bool(ctx.host.get("logit_rows_identity", False))
-        # the final norm inside the head's product (at most 16 rows), or, when every row is wanted,
-        # from the row scales the last block leaves (at most 64)
-        head_fused = (hasattr(self.final_norm, "pending") and self.head.dtype == torch.bfloat16
-                      and self.hidden_size % 8 == 0 and ctx.n_logits > 0
-                      and (ctx.n_logits <= ops.NORMED_MAX_ROWS and self.hidden_size <= ops.NORMED_MAX_K
-                           or all_rows and ctx.n_logits <= ops.EMIT_MAX_ROWS))
+        head_fused, all_rows = self._head_fused(ctx)
         for i, run in enumerate(self.schedule):
             block = self.blocks[run.block]
             if getattr(block, "takes_next_norm", False):
@@ -150,8 +147,32 @@ class DecoderModel:
                 block.forward(x, ctx, cache_views.get(run.cache), run.writes, next_norm=nxt)
             else:
                 block.forward(x, ctx, cache_views.get(run.cache), run.writes)
+        # which rows are wanted is a fact of the step, not of its shape: the head runs outside of what is recorded
+        # (a recorder keeps the function and hands back what it returns at each replay)
+        out: list = []
+
+        def head(c):
+            out[:] = [self._head(x, c)]
+            return out[0]
+
+        ctx.run_eagerly(head)
+        return out[0] if out else None
+
+    def _head_fused(self, ctx) -> tuple:
+        all_rows = ctx.n_logits == ctx.T and bool(ctx.host.get("logit_rows_identity", False))
+        # the final norm inside the head's product (at most 16 rows), or, when every row is wanted,
+        # from the row scales the last block leaves (at most 64)
+        fused = (hasattr(self.final_norm, "pending") and self.head.dtype == torch.bfloat16
+                 and self.hidden_size % 8 == 0 and ctx.n_logits > 0
+                 and (ctx.n_logits <= ops.NORMED_MAX_ROWS and self.hidden_size <= ops.NORMED_MAX_K
+                      or all_rows and ctx.n_logits <= ops.EMIT_MAX_ROWS))
+        return fused, all_rows
+
+    def _head(self, x, ctx) -> Optional[torch.Tensor]:
         if ctx.n_logits == 0:
             return None
+        rt = self.rt
+        head_fused, all_rows = self._head_fused(ctx)
         logits = torch.empty(ctx.n_logits, self.vocab_size, dtype=torch.float32, device=rt.device)
         if head_fused:
             fn = self.final_norm

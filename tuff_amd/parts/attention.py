@@ -51,6 +51,10 @@ class AttentionMixer(Mixer):
     def graph_safe(self):
         return self.position is None or self.position.graph_safe
 
+    @property
+    def records_portions(self):
+        return self.graph_safe
+
     def weight_decls(self):
         decls = self.qkv.weight_decls() + self.out.weight_decls()
         if self.eps is not None:
@@ -85,28 +89,34 @@ class AttentionMixer(Mixer):
     def forward(self, h, ctx, cache, residual, write_cache: bool = True) -> None:
         T = h.shape[0]
         H, Hkv, hd = self.H, self.Hkv, self.hd
-        g = ctx.groups[cache.group]
         qkv = self.qkv.forward(h)
         q = self.rt.empty(T, H * hd)
+        o = self.rt.empty(T, H * hd)
         norm = dict(eps=self.eps or 0.0, q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w)
         tables = self.position.rotary_tables() if self.position is not None else None
-        if self.position is None or tables is not None:
-            rot = {}
-            if tables is not None:
-                rot = dict(inv_freq=tables[0], rotary_dim=tables[1], interleaved=tables[2])
-            wr = dict(k_cache=cache.k, v_cache=cache.v, slot_mapping=g.slot_mapping) if write_cache else {}
-            ops.qkv_post(qkv, q, H=H, Hkv=Hkv, hd=hd, positions=ctx.positions, page_size=cache.page_size,
-                         **norm, **rot, **wr)
-        else:
-            # a position encoding of its own: norm, then its apply(), then the cache write
-            k = self.rt.empty(T, Hkv * hd)
-            ops.qkv_post(qkv, q, H=H, Hkv=Hkv, hd=hd, positions=ctx.positions, k_out=k, **norm)
-            self.position.apply(q, k, ctx.positions)
-            if write_cache:
-                v = qkv[:, (H + Hkv) * hd:].contiguous()
-                ops.kv_write(k, v, cache.k, cache.v, g.slot_mapping, Hkv=Hkv, hd=hd, page_size=cache.page_size)
-        o = self.rt.empty(T, H * hd)
-        self.attend(q, o, ctx, cache, g)
+        fused = self.position is None or tables is not None
+        # a position encoding of its own: norm, then its apply(), then the cache write
+        k = None if fused else self.rt.empty(T, Hkv * hd)
+
+        def over_the_cache(ctx):
+            """What depends on where the step's tokens lie: positions, cache slots, block tables."""
+            g = ctx.groups[cache.group]
+            if fused:
+                rot = {}
+                if tables is not None:
+                    rot = dict(inv_freq=tables[0], rotary_dim=tables[1], interleaved=tables[2])
+                wr = dict(k_cache=cache.k, v_cache=cache.v, slot_mapping=g.slot_mapping) if write_cache else {}
+                ops.qkv_post(qkv, q, H=H, Hkv=Hkv, hd=hd, positions=ctx.positions, page_size=cache.page_size,
+                             **norm, **rot, **wr)
+            else:
+                ops.qkv_post(qkv, q, H=H, Hkv=Hkv, hd=hd, positions=ctx.positions, k_out=k, **norm)
+                self.position.apply(q, k, ctx.positions)
+                if write_cache:
+                    v = qkv[:, (H + Hkv) * hd:].contiguous()
+                    ops.kv_write(k, v, cache.k, cache.v, g.slot_mapping, Hkv=Hkv, hd=hd, page_size=cache.page_size)
+            self.attend(q, o, ctx, cache, g)
+
+        ctx.run_eagerly(over_the_cache)
         self.out.forward(o, accumulate_into=residual)
 
     @staticmethod

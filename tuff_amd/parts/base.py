@@ -68,6 +68,14 @@ class Part:
     #: the host, so that a step through this part can be recorded into a graph and replayed.
     graph_safe = False
 
+    #: True if a step with prompt portions through this part can be recorded in sections: outside
+    #: of ctx.run_eagerly(fn) the part is graph_safe and reads of ctx only T, tokens, req_of_token,
+    #: q_start, q_len and state_slot (they stay in place between replays, with q_len 0 for requests
+    #: beyond the step's own); everything else of the step (positions, tables, wanted rows, host
+    #: facts) it reads inside fn(ctx), which runs again at every replay with that step's ctx, on
+    #: tensors it was given from outside (they keep their place too).
+    records_portions = False
+
     #: True if forward() may be handed a parts.norm.PendingNorm in place of the normed tensor h
     #: (the part passes it straight to a Linear, which can run the norm inside its kernel).
     accepts_pending_norm = False

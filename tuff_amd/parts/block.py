@@ -26,6 +26,10 @@ class PreNormBlock(Block):
     def graph_safe(self):
         return all(p.graph_safe for p in self._parts())
 
+    @property
+    def records_portions(self):
+        return all(p.records_portions for p in self._parts())
+
     def weight_decls(self):
         return [d for p in self._parts() for d in p.weight_decls()]
 

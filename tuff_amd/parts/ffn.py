@@ -15,6 +15,7 @@ from .linear import Linear
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
     graph_safe = True
+    records_portions = True
     accepts_pending_norm = True
     adds_once_through_linear = True
 

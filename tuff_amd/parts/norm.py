@@ -37,6 +37,7 @@ class PendingNorm:
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
     graph_safe = True
+    records_portions = True
 
     def __init__(self, dim: int, eps: float, name: str, aliases: tuple = ()):
         self.dim, self.eps, self.name, self.aliases = int(dim), float(eps), name, tuple(aliases)

@@ -15,6 +15,7 @@ from .base import POSITION_ENCODINGS, PositionEncoding, Runtime
 @POSITION_ENCODINGS.register("rotary")
 class Rotary(PositionEncoding):
     graph_safe = True
+    records_portions = True
 
     def __init__(self, head_dim: int, base: float, rotary_dim: Optional[int] = None,
                  interleaved: bool = False):

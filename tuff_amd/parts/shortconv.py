@@ -19,6 +19,7 @@ MAX_KERNEL = 17      # the state kernel keeps K-1 <= 16 rows in registers
 @MIXERS.register("shortconv")
 class ShortConvMixer(Mixer):
     graph_safe = True
+    records_portions = True
     accepts_pending_norm = True
     adds_once_through_linear = True
 
