@@ -45,7 +45,9 @@ def test_gemm_f32(gpu, M, N, K):
                                    # each shape of block of the tiled kernel, with ragged edges and a partial last step
                                    (1100, 8200, 72), (1030, 8190, 136), (1100, 4001, 200), (257, 129, 520),
                                    # the same with K a multiple of 64: operands go straight into LDS
-                                   (1100, 8200, 192), (1030, 8190, 128), (1100, 4001, 256), (257, 129, 512), (100, 40, 64)])
+                                   (1100, 8200, 192), (1030, 8190, 128), (1100, 4001, 256), (257, 129, 512), (100, 40, 64),
+                                   # few blocks and a short K: blocks of 64 x 64, ragged in M and N
+                                   (200, 1000, 1536), (65, 70, 3072), (500, 1536, 1536), (130, 2049, 320)])
 def test_gemm_bf16(gpu, M, N, K):
     from tuff_amd.csrc import ops
     x, w = _r(M, K, seed=4, dtype=torch.bfloat16), _r(N, K, seed=5, dtype=torch.bfloat16)
@@ -75,7 +77,7 @@ def test_gemm_bf16(gpu, M, N, K):
 @pytest.mark.parametrize("M,N,K", [(1, 32, 64), (8, 512, 240), (16, 6144, 2048), (5, 200, 96), (64, 384, 256),
                                    (40, 2050, 2048), (300, 130, 136), (2048, 512, 128), (1100, 8200, 72),
                                    (200, 384, 1024), (72, 4100, 2048),
-                                   (1030, 8202, 136), (1100, 4002, 200), (1030, 8202, 128), (1100, 4002, 192)])
+                                   (1030, 8202, 136), (1100, 4002, 200), (1030, 8202, 128), (1100, 4002, 192), (120, 13826, 1536)])
 def test_gemm_bf16_swiglu_epilogue(gpu, M, N, K):
     """Rows of w are gate and up rows interleaved; the output is silu(gate) * up."""
     from tuff_amd.csrc import ops

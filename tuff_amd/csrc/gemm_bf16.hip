@@ -859,7 +859,8 @@ SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16, bool emit = fals
 }
 
 // How a product of more than 64 rows is cut: shape 0: 256 x 256 blocks; 1: 128 x 128 blocks, two a CU;
-// 2: 128 x 128 blocks, one a CU, four register sets.  Depends on the sizes only.
+// 2: 128 x 128 blocks, one a CU, four steps of operands under way; 3: 64 x 64 blocks of four waves.
+// Depends on the sizes only.
 struct TiledPlan { int shape, slices, steps_per_slice; long long ws_floats; };
 
 TiledPlan plan_tiled(int M, int N, int K) {
@@ -869,6 +870,10 @@ TiledPlan plan_tiled(int M, int N, int K) {
     TiledPlan t;
     t.shape = large >= 160 ? 0 : small > 256 ? 1 : 2;
     t.slices = 1; t.steps_per_slice = nk; t.ws_floats = 0;
+    // few blocks and a short K: blocks of 64 x 64 give enough workgroups without slices of K, whose partial
+    // tiles cost a second kernel and as much traffic as the product's own (K = 1536 .. 2048, 96 to 512
+    // rows: 9 to 14 us instead of 11 to 19); beyond 48 steps the slices win
+    if (t.shape == 2 && small <= 128 && K % TBK == 0 && nk <= 48) { t.shape = 3; return t; }
     if (t.shape == 2 && small <= 128) {
         // as many slices as give every CU at most one block, at least eight steps a slice
         int s = max(1, min((int)(256 / small), nk / 8));
@@ -962,7 +967,8 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
         // Large blocks where they give most CUs one.  Of the small ones a CU holds two if there are
         // enough; if not, a block is alone on its CU and hides the memory's latency by itself, with
         // the operands of four steps under way.  Where even the small blocks are fewer than half the
-        // CUs (few rows, narrow output), K is cut into slices, a block a slice.
+        // CUs (few rows, narrow output), blocks of 64 x 64 take over if K is short, else K is cut into
+        // slices, a block a slice.
         const TiledPlan t = plan_tiled(M, N, K);
         if (t.slices > 1 && !ws) return -4;
 #define TILED(TM, TN, WM, WN, AHEAD) do { \
@@ -988,7 +994,8 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
                                X, W, Y, M, N, K, t.steps_per_slice, ws); \
         } while (0)
         if (K % TBK == 0) {
-            if (t.shape == 0) TILED_DMA(8, 4, 2, 4, 2);
+            if (t.shape == 3) TILED_DMA(2, 2, 2, 2, 4);
+            else if (t.shape == 0) TILED_DMA(8, 4, 2, 4, 2);
             else if (t.shape == 1) TILED_DMA(4, 2, 2, 4, 2);
             else TILED_DMA(4, 2, 2, 4, 4);
         }
