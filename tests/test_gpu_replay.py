@@ -246,6 +246,45 @@ def test_steps_with_portions_recorded_in_sections_equal_eager_steps(gpu, name, d
     util.assert_close(dtype, got["b"][mask], full[mask], "b")
 
 
+def test_recordings_are_dropped_and_made_again(gpu, monkeypatch):
+    """Room for one recording of each kind: sizes that take turns push each other out and are recorded
+    again, and every step still equals the eager one."""
+    from tuff_amd.engine.engine import Engine
+    monkeypatch.setattr(Engine, "SECTIONS_MIN_TOKENS", 40)
+    monkeypatch.setattr(Engine, "MAX_SECTIONED", 1)
+    monkeypatch.setattr(Engine, "MAX_GRAPHS", 1)
+    V = util.TINY_A["vocab_size"]
+    reqs = {k: util.rand_tokens(800, V, 30 + i) for i, k in enumerate("abc")}
+    steps, fed = [], {k: 0 for k in reqs}
+    def portion(rid, n):
+        t = reqs[rid][fed[rid]:fed[rid] + n]
+        fed[rid] += n
+        assert len(t) == n
+        return {"id": rid, "tokens": t, "want": [len(t) - 1]}
+    def add(entries, end=()):
+        steps.append({"step": len(steps), "entries": entries, "end": list(end)})
+    for rnd in range(3):
+        for _ in range(4):
+            add([portion("a", 40), portion("b", 10)])          # 50 tokens
+        for _ in range(2):
+            add([portion("a", 1), portion("b", 1)])            # two single tokens
+        for _ in range(4):
+            add([portion("b", 1), portion("c", 59)])           # 60 tokens
+        for _ in range(2):
+            add([portion(k, 1) for k in "abc"])                # three single tokens
+    add([portion("a", 1)], end=list("abc"))
+    eager = make_engine("A", "bfloat16", max_tokens=2560, use_graphs=False)
+    want = util.run_plan(eager, steps)
+    eng = make_engine("A", "bfloat16", max_tokens=2560)
+    got = util.run_plan(eng, steps)
+    # a size is recorded when it has come three times: in the first round its third and fourth step replay, later all four
+    assert eng.section_replays == 2 * 2 + 2 * 2 * 4 and len(eng._sectioned) == 1 and len(eng._graphs) == 1
+    assert eng.graph_replays == 3 * 2 * 1
+    for rid in reqs:
+        mask = ~torch.isnan(want[rid][:, 0])
+        assert torch.equal(got[rid][mask], want[rid][mask]), rid
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_token_ids_taken_from_the_device(gpu, dtype):
     """A step may take some of its token ids from a vector on the device (the sampler's output of

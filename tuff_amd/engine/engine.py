@@ -203,6 +203,7 @@ class Engine:
                 self._place_device_tokens(ctx.tokens, device_tokens)
                 return self.model.forward(ctx, self.storage.views)
             if len(self._sectioned) >= self.MAX_SECTIONED:
+                torch.cuda.synchronize()                    # its last replay may still be under way
                 self._sectioned.pop(next(iter(self._sectioned)))
             rec = _SectionedStep(ctx.T, self.manager.num_slots, self.device)
             try:
@@ -240,6 +241,7 @@ class Engine:
         g = self._graphs.get(key)
         if g is None:
             if len(self._graphs) >= self.MAX_GRAPHS:
+                torch.cuda.synchronize()                    # its last replay may still be under way
                 self._graphs.pop(next(iter(self._graphs)))
             g = _RecordedStep(p, self.device, width * self.page_size)
             self._graphs[key] = g
