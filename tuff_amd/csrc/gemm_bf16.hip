@@ -859,7 +859,8 @@ SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16, bool emit = fals
 }
 
 // How a product of more than 64 rows is cut: shape 0: 256 x 256 blocks; 1: 128 x 128 blocks, two a CU;
-// 2: 128 x 128 blocks, one a CU, four steps of operands under way; 3: 64 x 64 blocks of four waves.
+// 2: 128 x 128 blocks, one a CU, four steps of operands under way; 3: 64 x 64 blocks of four waves;
+// 4: 256 x 192 blocks.
 // Depends on the sizes only.
 struct TiledPlan { int shape, slices, steps_per_slice; long long ws_floats; };
 
@@ -870,6 +871,13 @@ TiledPlan plan_tiled(int M, int N, int K) {
     TiledPlan t;
     t.shape = large >= 160 ? 0 : small > 256 ? 1 : 2;
     t.slices = 1; t.steps_per_slice = nk; t.ws_floats = 0;
+    // blocks of 256 x 192 where they need fewer rounds of 256 workgroups times columns than 256 x 256
+    // (6144 columns and 2048 rows: 256 blocks, one round, instead of 192 blocks that leave a quarter of the CUs idle)
+    if (t.shape == 0 && K % TBK == 0) {
+        const long long wide = (long long)ceil_div(N, 192) * ceil_div(M, 256);
+        if (ceil_div(wide, 256) * 192 < ceil_div(large, 256) * 256) t.shape = 4;
+        return t;
+    }
     // few blocks and a short K: blocks of 64 x 64 give enough workgroups without slices of K, whose partial
     // tiles cost a second kernel and as much traffic as the product's own (K = 1536 .. 2048, 96 to 512
     // rows: 9 to 14 us instead of 11 to 19); beyond 48 steps the slices win
@@ -995,6 +1003,7 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
         } while (0)
         if (K % TBK == 0) {
             if (t.shape == 3) TILED_DMA(2, 2, 2, 2, 4);
+            else if (t.shape == 4) TILED_DMA(8, 3, 2, 4, 2);
             else if (t.shape == 0) TILED_DMA(8, 4, 2, 4, 2);
             else if (t.shape == 1) TILED_DMA(4, 2, 2, 4, 2);
             else TILED_DMA(4, 2, 2, 4, 4);
