@@ -575,7 +575,7 @@ def test_attention_prefill_key_segments(gpu, H, Hkv, hd, ps, window, monkeypatch
                               positions=case["positions"] if segments else None)
         outs[segments] = out.cpu().double().reshape(T, H, hd)
         _check_step(case, reqs, outs[segments], H, hd, window, f"segments {segments}")
-    assert blocks.shape[0] * Hkv < ops.PREFILL_MIN_WORKGROUPS and case["max_ctx_len"] >= 2 * ops.PREFILL_MIN_SEGMENT
+    assert 2 * blocks.shape[0] * Hkv <= ops.PREFILL_WORKGROUP_SLOTS and case["max_ctx_len"] >= 2 * ops.PREFILL_MIN_SEGMENT
     # the two ways differ in rounding only
     assert (outs[True] - outs[False]).abs().max() <= 2 ** -7 * float(outs[False].abs().max())
 

@@ -531,7 +531,8 @@ def attention_prefill_block_columns(hd: int) -> int:
     return 128 if hd <= 128 else 64
 
 
-PREFILL_MIN_WORKGROUPS = 192     # fewer than this: the keys are cut into segments, a workgroup a segment
+PREFILL_WORKGROUP_SLOTS = 512    # workgroups of attention_prefill the part runs side by side (two a CU); with at most
+                                 # half as many blocks the keys are cut into segments, a workgroup a segment
 PREFILL_MIN_SEGMENT = 1024       # keys; shorter segments are not worth their merge
 
 
@@ -575,8 +576,9 @@ def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info
         scale = 1.0 / math.sqrt(hd)
     n_segs, seg_keys, ws_o, ws_ml = 1, 0, None, None
     workgroups = nblk * Hkv
-    if positions is not None and 0 < workgroups < PREFILL_MIN_WORKGROUPS and int(max_ctx_len) >= 2 * PREFILL_MIN_SEGMENT:
-        want = min(-(-2 * PREFILL_MIN_WORKGROUPS // workgroups), int(max_ctx_len) // PREFILL_MIN_SEGMENT, 64)
+    if positions is not None and 0 < 2 * workgroups <= PREFILL_WORKGROUP_SLOTS and int(max_ctx_len) >= 2 * PREFILL_MIN_SEGMENT:
+        # as many segments as fill the slots once, not more: what does not fit waits for a second round
+        want = min(PREFILL_WORKGROUP_SLOTS // workgroups, int(max_ctx_len) // PREFILL_MIN_SEGMENT, 64)
         seg_keys = -(-(-(-int(max_ctx_len) // want)) // 64) * 64
         n_segs = -(-int(max_ctx_len) // seg_keys)
     if n_segs > 1:
