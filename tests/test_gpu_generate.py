@@ -277,3 +277,36 @@ def test_scheduler_scenarios_drawn_at_random(gpu, name, seed):
             continue
         want = alone.generate([p], sp)[0]
         assert (g.token_ids, g.finish_reason) == (want.token_ids, want.finish_reason), (seed, i, g.preemptions)
+
+
+@pytest.mark.parametrize("name,seed", [("A", 2), ("C", 11)])
+def test_scheduler_scenarios_with_steps_recorded_in_sections(gpu, name, seed):
+    """The same with long prompts and a budget that is filled step after step, so that steps with
+    portions are recorded and replayed (beside preemptions and steps started early): in float32
+    every request still generates what it generates alone."""
+    import random
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.engine.llm import LLM
+    from tuff_amd.sampling.params import SamplingParams
+    V = util.CONFIGS[name][0]["vocab_size"]
+    folder = util.model_folder(name, "float32")
+    alone = LLM(engine=Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=256, max_requests=2),
+                max_num_seqs=1, ctx_size=1000)
+    rng = random.Random(seed)
+    n = rng.randint(4, 9)
+    prompts = [util.rand_tokens(rng.randint(2, 700), V, seed * 100 + i) for i in range(n)]
+    params = [SamplingParams(max_new_tokens=rng.randint(1, 40), ignore_eos=rng.random() < 0.7,
+                             temp=rng.choice([0.0, 0.0, 0.8]), top_k=rng.choice([0, 20]), seed=rng.randint(1, 99))
+              for _ in range(n)]
+    pages = rng.randint(60, 120)
+    llm = LLM(engine=Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=pages, max_requests=4),
+              max_num_seqs=rng.randint(2, 4), max_batched_tokens=rng.choice([128, 130]), ctx_size=1000)
+    got = llm.generate(prompts, params)
+    llm.engine.manager.check()
+    assert not llm.engine.manager.live() and llm.engine.section_replays >= 3
+    for i, (p, sp, g) in enumerate(zip(prompts, params, got)):
+        if g.finish_reason == "capacity":
+            assert -(-(len(p) + sp.max_new_tokens) // 16) > pages
+            continue
+        want = alone.generate([p], sp)[0]
+        assert (g.token_ids, g.finish_reason) == (want.token_ids, want.finish_reason), (seed, i, g.preemptions)
