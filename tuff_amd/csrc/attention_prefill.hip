@@ -226,23 +226,28 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         for (int i = 0; i < VPT; ++i) *(bf16x8*)(Vs + buf * VBUF + v_lds[i]) = vreg[set][i];
     };
 
-    // ---- one half step (32 keys) of this wave out of LDS
-    auto half_step = [&](int buf, int sub, int key0, auto open_tag) {
-        constexpr bool open = decltype(open_tag)::value;
+    // ---- one half step (32 keys) of this wave out of LDS: the scores, then their weights and the sum
+    struct Scores { f32x4 v[2][NBW]; };
+    auto scores = [&](int buf, int sub) {
         const bf16_t* Kb = Ks + buf * KBUF + (sub * 32 + n16) * KROW + g * 8;
-        const bf16_t* Vb = Vs + buf * VBUF + n16 * VROW + sub * 32 + g * 8;
-        f32x4 s[2][NBW];
+        Scores sc;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-            for (int nb = 0; nb < NBW; ++nb) s[kb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int nb = 0; nb < NBW; ++nb) sc.v[kb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kc = 0; kc < KC; ++kc) {
                 const bf16x8 kf = *(const bf16x8*)(Kb + kb * 16 * KROW + kc * 32);
 #pragma unroll
-                for (int nb = 0; nb < NBW; ++nb) s[kb][nb] = mfma32(kf, qf[nb][kc], s[kb][nb]);
+                for (int nb = 0; nb < NBW; ++nb) sc.v[kb][nb] = mfma32(kf, qf[nb][kc], sc.v[kb][nb]);
             }
         }
+        return sc;
+    };
+    auto weigh_and_add = [&](int buf, int sub, int key0, const Scores& sc, auto open_tag) {
+        constexpr bool open = decltype(open_tag)::value;
+        const bf16_t* Vb = Vs + buf * VBUF + n16 * VROW + sub * 32 + g * 8;
+        const auto& s = sc.v;
         // open: every key of the half is visible to every column of the wave, no mask
         bf16x8 pf[NBW];
         float corr[NBW];
@@ -299,6 +304,11 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         }
     };
 
+    auto half_step = [&](int buf, int sub, int key0, auto open_tag) {
+        const Scores sc = scores(buf, sub);
+        weigh_and_add(buf, sub, key0, sc, open_tag);
+    };
+
     // set u holds step u, later step u + AHEAD, ...; step s + 1 goes into LDS while step s is computed.
     // (Loops over sets are unrolled, so a set's registers are named at compile time.)
 #pragma unroll
@@ -316,12 +326,20 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
             if (ls % 16 == 0) pages_cur = pages_next;
             if (ls % 16 == 1) pages_next = pages_of(ls / 16 + 1);
             load_step(u, ls, pages_cur);
+            if (key0 + 63 <= wave_pos_min && key0 >= wave_lo_max) {
+                // the whole step is visible to every column of the wave: the scores of both halves first,
+                // so that the products of one half run while the other's exponentials are computed
+                const Scores s0 = scores(buf, 0), s1 = scores(buf, 1);
+                weigh_and_add(buf, 0, key0, s0, std::true_type());
+                weigh_and_add(buf, 1, key0 + 32, s1, std::true_type());
+            } else {
 #pragma unroll
-            for (int sub = 0; sub < 2; ++sub) {
-                const int k0 = key0 + sub * 32;
-                if (k0 <= wave_pos_max && k0 + 31 >= (window > 0 ? max(0, wave_pos_min - window + 1) : 0)) {
-                    if (k0 + 31 <= wave_pos_min && k0 >= wave_lo_max) half_step(buf, sub, k0, std::true_type());
-                    else half_step(buf, sub, k0, std::false_type());
+                for (int sub = 0; sub < 2; ++sub) {
+                    const int k0 = key0 + sub * 32;
+                    if (k0 <= wave_pos_max && k0 + 31 >= (window > 0 ? max(0, wave_pos_min - window + 1) : 0)) {
+                        if (k0 + 31 <= wave_pos_min && k0 >= wave_lo_max) half_step(buf, sub, k0, std::true_type());
+                        else half_step(buf, sub, k0, std::false_type());
+                    }
                 }
             }
             store_step((u + 1) % AHEAD, buf ^ 1);
@@ -406,7 +424,7 @@ TUFF_EXPORT int tuff_attention_prefill(const void* q, const void* k_cache, const
 #define GO(HDP, NBW, AHEAD) return launch<HDP, NBW, AHEAD>(grid, stream, Q, K, V, (bf16_t*)out, block_table, max_blocks, (const int2*)blk, \
                                              (const int4*)req_info, H, Hkv, hd, page_size, window, sl, seg_keys, ws_o, ws_ml)
     if (hd <= 32) GO(32, 2, 3);
-    else if (hd <= 64) GO(64, 2, 3);
+    else if (hd <= 64) GO(64, 2, 2);
     else if (hd <= 96) GO(96, 2, 2);
     else if (hd <= 128) GO(128, 2, 2);
     else GO(256, 1, 1);
