@@ -26,7 +26,7 @@
 namespace {
 constexpr int STEP = 64;            // keys a step
 constexpr int NT = 256;             // threads a workgroup
-constexpr float SLACK = 8.f;        // see half_step
+constexpr float SLACK = 8.f;        // see whole_step
 constexpr int VROW = STEP + 8;      // bf16 a row of V^T in LDS: 64 keys and 16 bytes that keep rows off each other's banks
 
 __device__ __forceinline__ f32x4 mfma32(bf16x8 a, bf16x8 b, f32x4 c) {
@@ -226,7 +226,7 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         for (int i = 0; i < VPT; ++i) *(bf16x8*)(Vs + buf * VBUF + v_lds[i]) = vreg[set][i];
     };
 
-    // ---- one half step (32 keys) of this wave out of LDS: the scores, then their weights and the sum
+    // ---- the scores of one half step (32 keys) of this wave, out of LDS
     struct Scores { f32x4 v[2][NBW]; };
     auto scores = [&](int buf, int sub) {
         const bf16_t* Kb = Ks + buf * KBUF + (sub * 32 + n16) * KROW + g * 8;
@@ -244,12 +244,19 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         }
         return sc;
     };
-    auto weigh_and_add = [&](int buf, int sub, int key0, const Scores& sc, auto open_tag) {
+    // One step of 64 keys: the scores of both halves, then, per column, one reference point for the
+    // exponents of all 64 (so that the products of one half run while the other's exponentials are
+    // computed, and the bookkeeping is done once), then the weighted sums.  open: every key of the step
+    // is visible to every column of the wave, no mask.  Otherwise live0/live1 say which halves hold a
+    // key that some column sees; a column's masked keys weigh nothing, so what a column sums does not
+    // depend on which columns share its wave.
+    auto whole_step = [&](int buf, int key0, bool live0, bool live1, auto open_tag) {
         constexpr bool open = decltype(open_tag)::value;
-        const bf16_t* Vb = Vs + buf * VBUF + n16 * VROW + sub * 32 + g * 8;
-        const auto& s = sc.v;
-        // open: every key of the half is visible to every column of the wave, no mask
-        bf16x8 pf[NBW];
+        const bf16_t* Vb = Vs + buf * VBUF + n16 * VROW + g * 8;
+        Scores sc[2];
+        if (open || live0) sc[0] = scores(buf, 0);
+        if (open || live1) sc[1] = scores(buf, 1);
+        bf16x8 pf[2][NBW];
         float corr[NBW];
         bool same = true;
 #pragma unroll
@@ -258,15 +265,18 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
             // monotonic), so that score * scale - maximum is one fused operation: written as fmaf,
             // it is the same instruction with and without the mask.
             float mx = -INFINITY;
-            bool ok[8];
+            bool ok[2][8];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int key = key0 + 8 * g + 4 * kb + e;
-                    ok[kb * 4 + e] = open || (key <= pos_c[nb] && key >= lo_c[nb]);
-                    mx = fmaxf(mx, ok[kb * 4 + e] ? s[kb][nb][e] : -INFINITY);
-                }
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int key = key0 + 32 * sub + 8 * g + 4 * kb + e;
+                        const bool v = open || ((sub ? live1 : live0) && key <= pos_c[nb] && key >= lo_c[nb]);
+                        ok[sub][kb * 4 + e] = v;
+                        mx = fmaxf(mx, v ? sc[sub].v[kb][nb][e] : -INFINITY);
+                    }
             mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
             mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
             // The reference point of the exponents moves only when a score exceeds it by more than
@@ -279,11 +289,13 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
             same = same && (m_new == m_run[nb]);
             float sum = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float p = ok[i] ? __builtin_amdgcn_exp2f(fmaf(s[i / 4][nb][i % 4], scale_log2e, -m_safe)) : 0.f;
-                sum += p;
-                pf[nb][i] = (bf16_t)p;
-            }
+            for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float p = ok[sub][i] ? __builtin_amdgcn_exp2f(fmaf(sc[sub].v[i / 4][nb][i % 4], scale_log2e, -m_safe)) : 0.f;
+                    sum += p;
+                    pf[sub][nb][i] = (bf16_t)p;
+                }
             l_run[nb] = fmaf(l_run[nb], corr[nb], sum);
             m_run[nb] = m_new;
         }
@@ -297,16 +309,15 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
                     for (int e = 0; e < 4; ++e) o[db][nb][e] *= corr[nb];
         }
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-            const bf16x8 vf = *(const bf16x8*)(Vb + db * 16 * VROW);
+        for (int sub = 0; sub < 2; ++sub) {
+            if (!(open || (sub ? live1 : live0))) continue;
 #pragma unroll
-            for (int nb = 0; nb < NBW; ++nb) o[db][nb] = mfma32(vf, pf[nb], o[db][nb]);
+            for (int db = 0; db < DB; ++db) {
+                const bf16x8 vf = *(const bf16x8*)(Vb + db * 16 * VROW + sub * 32);
+#pragma unroll
+                for (int nb = 0; nb < NBW; ++nb) o[db][nb] = mfma32(vf, pf[sub][nb], o[db][nb]);
+            }
         }
-    };
-
-    auto half_step = [&](int buf, int sub, int key0, auto open_tag) {
-        const Scores sc = scores(buf, sub);
-        weigh_and_add(buf, sub, key0, sc, open_tag);
     };
 
     // set u holds step u, later step u + AHEAD, ...; step s + 1 goes into LDS while step s is computed.
@@ -326,22 +337,11 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
             if (ls % 16 == 0) pages_cur = pages_next;
             if (ls % 16 == 1) pages_next = pages_of(ls / 16 + 1);
             load_step(u, ls, pages_cur);
-            if (key0 + 63 <= wave_pos_min && key0 >= wave_lo_max) {
-                // the whole step is visible to every column of the wave: the scores of both halves first,
-                // so that the products of one half run while the other's exponentials are computed
-                const Scores s0 = scores(buf, 0), s1 = scores(buf, 1);
-                weigh_and_add(buf, 0, key0, s0, std::true_type());
-                weigh_and_add(buf, 1, key0 + 32, s1, std::true_type());
-            } else {
-#pragma unroll
-                for (int sub = 0; sub < 2; ++sub) {
-                    const int k0 = key0 + sub * 32;
-                    if (k0 <= wave_pos_max && k0 + 31 >= (window > 0 ? max(0, wave_pos_min - window + 1) : 0)) {
-                        if (k0 + 31 <= wave_pos_min && k0 >= wave_lo_max) half_step(buf, sub, k0, std::true_type());
-                        else half_step(buf, sub, k0, std::false_type());
-                    }
-                }
-            }
+            const int lo_any = window > 0 ? max(0, wave_pos_min - window + 1) : 0;
+            const bool live0 = key0 <= wave_pos_max && key0 + 31 >= lo_any;
+            const bool live1 = key0 + 32 <= wave_pos_max && key0 + 63 >= lo_any;
+            if (key0 + 63 <= wave_pos_min && key0 >= wave_lo_max) whole_step(buf, key0, true, true, std::true_type());
+            else if (live0 || live1) whole_step(buf, key0, live0, live1, std::false_type());
             store_step((u + 1) % AHEAD, buf ^ 1);
             __syncthreads();
         }
