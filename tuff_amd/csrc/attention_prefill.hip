@@ -16,7 +16,9 @@
 // Products (v_mfma_f32_16x16x32_bf16), per half step of 32 keys, as in the decode kernel:
 // S^T = K Q^T in two products of 16 keys whose rows are ordered so that lane group g ends up with
 // the scores of keys 8g..8g+7; after mask, maximum and exp these are, as they lie, the lane's
-// part of P^T for O^T += V^T P^T.
+// part of P^T for O^T += V^T P^T.  The scores of both halves of a step are taken first and the
+// reference point of the exponents is moved once a step of 64 keys, for every step alike, masked
+// or not.
 //
 // Cache layout: K [page][kv_head][offset][hd], V [page][kv_head][hd][offset]; page size a
 // multiple of 16, head size a multiple of 8.
