@@ -204,7 +204,7 @@ def main() -> int:
                     help="fewer layers than the shape has (sizes of a layer stay)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
-    ap.add_argument("--point-steps", type=int, default=32)
+    ap.add_argument("--point-steps", type=int, default=96)
     ap.add_argument("--only-prefill", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiling) and print its record")
     ap.add_argument("--scenario", choices=sorted(SCENARIOS),
