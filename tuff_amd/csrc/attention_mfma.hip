@@ -26,6 +26,7 @@
 // general kernel otherwise).
 #include "common.h"
 #include <math.h>
+#include <mutex>
 
 namespace {
 constexpr int PART = 256;
@@ -406,11 +407,11 @@ static int launch_merge(const float* ws_o, const float* ws_ml, bf16_t* out, cons
 // positions [n_tokens]: every token's position (read by the merge).
 // ws_o: float32 [n_tokens * H * n_parts * hd], ws_ml: float32 [n_tokens * H * n_parts * 2].
 // n_parts >= ceil((largest position + 1) / 256).  nb: 1, 2 or 4 column blocks a wave.
-TUFF_EXPORT int tuff_attention_mfma(const void* q, const void* k_cache, const void* v_cache, void* out,
-                                    float* ws_o, float* ws_ml, const int* block_table, int max_blocks,
-                                    const int* blk, int n_qblocks, int nb, const int* req_info, const int* positions,
-                                    int n_tokens, int H, int Hkv, int hd, int page_size, int window, float scale,
-                                    int n_parts, hipStream_t stream) {
+static int launch_attention(const void* q, const void* k_cache, const void* v_cache, void* out,
+                            float* ws_o, float* ws_ml, const int* block_table, int max_blocks,
+                            const int* blk, int n_qblocks, int nb, const int* req_info, const int* positions,
+                            int n_tokens, int H, int Hkv, int hd, int page_size, int window, float scale,
+                            int n_parts, hipStream_t stream) {
     if (n_tokens <= 0 || n_qblocks <= 0) return 0;
     if (hd > 256 || hd % 8 != 0 || page_size % 16 != 0 || Hkv <= 0 || H % Hkv != 0 || n_parts < 1) return -2;
     if (Hkv > 65535 || n_qblocks > 65535 || n_parts > COMBINE_MAX_PARTS) return -2;
@@ -434,6 +435,15 @@ TUFF_EXPORT int tuff_attention_mfma(const void* q, const void* k_cache, const vo
                         stream);
 }
 
+TUFF_EXPORT int tuff_attention_mfma(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                    float* ws_o, float* ws_ml, const int* block_table, int max_blocks,
+                                    const int* blk, int n_qblocks, int nb, const int* req_info, const int* positions,
+                                    int n_tokens, int H, int Hkv, int hd, int page_size, int window, float scale,
+                                    int n_parts, hipStream_t stream) {
+    return launch_attention(q, k_cache, v_cache, out, ws_o, ws_ml, block_table, max_blocks, blk, n_qblocks, nb, req_info,
+                            positions, n_tokens, H, Hkv, hd, page_size, window, scale, n_parts, stream);
+}
+
 // The merge alone, for partial results that another kernel left in the same layout (ws_o
 // [tokens * H * n_parts * hd], ws_ml [tokens * H * n_parts * 2] = (reference exponent, sum); partition
 // p of a row holds the keys p * part_keys .. (p + 1) * part_keys - 1).
@@ -442,4 +452,79 @@ TUFF_EXPORT int tuff_attention_merge(const float* ws_o, const float* ws_ml, void
     if (n_tokens <= 0) return 0;
     if (hd > 256 || n_parts < 1 || n_parts > COMBINE_MAX_PARTS || part_keys < 1) return -2;
     return launch_merge(ws_o, ws_ml, (bf16_t*)out, positions, n_tokens, H, hd, window, n_parts, part_keys, stream);
+}
+
+// ------------------------------------------------- the same attention without an allocation
+// tuff_attention_mfma_static: tuff_attention_mfma with the partitions' partial results kept in an
+// array of this library instead of a work space the caller brings, for callers that cannot
+// allocate (a HIP graph under capture, a serving loop that must not call the allocator).  It calls
+// no hipMalloc, hipFree or allocating library routine.
+//
+// The array is STATIC_SCRATCH_FLOATS floats (16 MiB) of device memory on every GPU the library is
+// loaded on, held until the process ends.  A call needs n_tokens * H * n_parts * (hd + 2) floats
+// (rounded up to 64 for the first of its two parts) and is refused with TUFF_STATIC_TOO_LARGE
+// beyond that.  All calls on one GPU share that GPU's array: it keeps the last call's contents
+// (nothing has to start at zero: a row of a partition that a token does not have is never used),
+// and two calls that overlap on one GPU, on different streams or from different threads, race.
+//
+// In host code the array's name stands for the symbol, not for device memory; the address on the
+// current device comes from hipGetSymbolAddress, once per device, and only that pointer is handed
+// to the kernels.
+constexpr long long STATIC_SCRATCH_FLOATS = 4ll << 20;
+constexpr int STATIC_MAX_DEVICES = 64;
+enum : int { TUFF_STATIC_TOO_LARGE = -7, TUFF_STATIC_NO_DEVICE = -8 };
+
+static __device__ __align__(256) float static_scratch[STATIC_SCRATCH_FLOATS];
+static float* static_scratch_ptr[STATIC_MAX_DEVICES];      // per device; written once, under the lock
+
+static std::mutex static_scratch_lock;
+
+// The array's address on the current device; looked up at the first call on that device.
+static int static_scratch_of_current_device(float** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES) return TUFF_STATIC_NO_DEVICE;
+    std::lock_guard<std::mutex> guard(static_scratch_lock);
+    if (!static_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(static_scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return TUFF_STATIC_NO_DEVICE;
+        static_scratch_ptr[dev] = (float*)p;
+    }
+    *ptr = static_scratch_ptr[dev];
+    return 0;
+}
+
+// Looks the array up on the current device, so that the first attention call there does nothing
+// but launch.  Returns 0, or a HIP error code.
+TUFF_EXPORT int tuff_attention_static_setup(void) {
+    float* p = nullptr;
+    return static_scratch_of_current_device(&p);
+}
+
+// Floats of the static array a call of these sizes needs, and (*capacity) how many there are.
+TUFF_EXPORT long long tuff_attention_static_floats(int n_tokens, int H, int hd, int n_parts, long long* capacity) {
+    if (capacity) *capacity = STATIC_SCRATCH_FLOATS;
+    const long long rows = (long long)n_tokens * H * n_parts;
+    return (rows * hd + 63) / 64 * 64 + rows * 2;
+}
+
+TUFF_EXPORT int tuff_attention_mfma_static(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                           const int* block_table, int max_blocks,
+                                           const int* blk, int n_qblocks, int nb, const int* req_info, const int* positions,
+                                           int n_tokens, int H, int Hkv, int hd, int page_size, int window, float scale,
+                                           int n_parts, hipStream_t stream) {
+    if (n_tokens <= 0 || n_qblocks <= 0) return 0;
+    if (H <= 0 || hd <= 0 || n_parts < 1) return -2;
+    if (tuff_attention_static_floats(n_tokens, H, hd, n_parts, nullptr) > STATIC_SCRATCH_FLOATS) return TUFF_STATIC_TOO_LARGE;
+    float* base = nullptr;
+    const int rc = static_scratch_of_current_device(&base);
+    if (rc) return rc;
+    const long long rows = (long long)n_tokens * H * n_parts;
+    float* ws_o = base;
+    float* ws_ml = base + (rows * hd + 63) / 64 * 64;
+    return launch_attention(q, k_cache, v_cache, out, ws_o, ws_ml, block_table, max_blocks, blk, n_qblocks, nb, req_info,
+                            positions, n_tokens, H, Hkv, hd, page_size, window, scale, n_parts, stream);
 }

@@ -66,6 +66,9 @@ _SIGNATURES = {
                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p],
         "tuff_attention_merge": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_void_p],
+        "tuff_attention_mfma_static": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                                       _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
+                                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p],
     },
     "attention_prefill": {
         "tuff_attention_prefill": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
@@ -154,6 +157,8 @@ def _check(code: int, what: str) -> None:
     if code != 0:
         if code == -2:
             raise KernelError(f"{what}: the kernel refuses these sizes")
+        if code == -7:
+            raise KernelError(f"{what}: the step needs more work space than the library's static array holds")
         raise KernelError(f"{what}: launch failed with HIP error {code}")
 
 
