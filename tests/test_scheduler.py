@@ -172,6 +172,75 @@ def test_pages_run_out_preempt_the_latest_and_recompute_with_unchanged_output():
     assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == 12
 
 
+def test_a_long_prompt_beside_decoding_requests_on_a_tight_pool_is_not_computed_over_and_over():
+    """Three requests decode; a fourth with a long prompt is admitted when its first portion fits and
+    then finds no pages for the next.  It must wait with what it holds (or take a shorter portion),
+    not be preempted and admitted again step after step: tokens computed twice and preemptions stay
+    small, and every output is the unconstrained one."""
+    prompts = {"a": list(range(6)), "b": list(range(50, 56)), "c": list(range(90, 96)), "long": list(range(200, 260))}
+    new = {"a": 22, "b": 18, "c": 14, "long": 4}
+    ex = FakeExecutor(num_pages=26, page_size=4)             # 3 x 7 pages at the end of a, b, c; long needs 16
+    sched = make(ex, max_batched_tokens=16)
+    reqs = {k: Request(k, prompts[k], SamplingParams(max_new_tokens=new[k])) for k in prompts}
+    for k in ("a", "b", "c", "long"):
+        sched.add(reqs[k])
+    steps = run(sched, ex)
+    for k in prompts:
+        assert reqs[k].output == expected_output(prompts[k], new[k]) and reqs[k].finish_reason == "length", k
+    fed = {k: sum(len(s.tokens) for b in steps for s in b if s.request.id == k) for k in prompts}
+    needed = {k: len(prompts[k]) + new[k] - 1 for k in prompts}
+    assert all(reqs[k].preemptions == 0 and fed[k] == needed[k] for k in ("a", "b", "c"))
+    assert sched.num_preemptions <= 2, sched.num_preemptions
+    assert reqs["long"].preemptions == sched.num_preemptions
+    assert fed["long"] <= needed["long"] * (1 + reqs["long"].preemptions), fed   # at most once over per preemption
+    # while it waited for pages it kept the ones it had: steps in which it was left out or got a shorter portion
+    waits = [b for b in steps if not any(s.request.id == "long" for s in b) and reqs["long"] in [s.request for bb in steps[:steps.index(b)] for s in bb]]
+    short = [s for b in steps for s in b if s.request.id == "long" and not s.samples and len(s.tokens) < 16 - (len(b) - 1)]
+    assert waits or short
+    assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == 26
+
+
+def test_prompts_that_hold_all_pages_between_them_do_not_stall():
+    """Two prompts admitted side by side whose rest fits only one at a time: nothing can move, so
+    the later one is preempted and the first goes on."""
+    ex = FakeExecutor(num_pages=10, page_size=4)
+    sched = make(ex, max_batched_tokens=16)
+    a = Request("a", list(range(30)), SamplingParams(max_new_tokens=3))       # 9 pages at the end
+    b = Request("b", list(range(100, 130)), SamplingParams(max_new_tokens=3))
+    sched.add(a)
+    first = sched.schedule()
+    sched.update(first, ex.step(first))                                       # a holds 4 pages
+    sched.add(b)
+    run(sched, ex)
+    assert a.output == expected_output(range(30), 3) and b.output == expected_output(range(100, 130), 3)
+    assert a.preemptions == 0 and b.preemptions <= 1
+    assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == 10
+
+
+def test_decoding_requests_take_turns_when_the_budget_is_smaller_than_their_number():
+    ex = FakeExecutor()
+    sched = make(ex, max_batched_tokens=4, max_num_seqs=4)
+    reqs = [Request(k, [i, i + 1], SamplingParams(max_new_tokens=9)) for i, k in enumerate("abcd")]
+    for r in reqs:
+        sched.add(r)
+    while any(r.remaining() != 1 or r.status != "running" for r in reqs):     # all four decoding
+        batch = sched.schedule()
+        sched.update(batch, ex.step(batch))
+    sched.max_batched_tokens = 3
+    seen = []
+    for _ in range(4):
+        batch = sched.schedule()
+        assert len(batch) == 3
+        seen.append({s.request.id for s in batch})
+        sched.update(batch, ex.step(batch))
+    counts = {k: sum(k in b for b in seen) for k in "abcd"}
+    assert set(counts.values()) == {3}, counts                               # 12 tokens, three each: nobody starves
+    sched.max_batched_tokens = 4
+    run(sched, ex)
+    for i, r in enumerate(reqs):
+        assert r.output == expected_output([i, i + 1], 9)
+
+
 def test_waiting_request_is_not_admitted_into_a_full_pool():
     ex = FakeExecutor(num_pages=6, page_size=4)
     sched = make(ex, max_batched_tokens=64)

@@ -10,13 +10,14 @@ a token gets a PLACEHOLDER at the end of its output, requests that end with this
 is are finished), `commit()` puts the tokens where the placeholders are and finishes requests at
 an end-of-sequence token.  Between the two, `schedule(ahead=True)` decides the next step.
 
-When pages run out: a waiting request is simply not admitted yet.  If a running request
-cannot get the pages for its next tokens, the most recently admitted running request is
-preempted: its pages and slot are given back, and it returns to the head of the waiting queue
-to be computed again from its first token, prompt and generated tokens together (a conv state
-cannot be rebuilt from the KV cache, so recomputation is the only exact way).  Its sampler state
-is kept, so its output does not change.  A request that does not fit the pool even alone is
-finished with reason "capacity".
+When pages run out: a waiting request is simply not admitted yet.  A running prompt whose next
+portion does not fit is cut to the pages there are, or sits a step out with what it holds.  If a
+decoding request cannot get the page for its next token, the most recently admitted running
+request is preempted: its pages and slot are given back, and it returns to the head of the
+waiting queue to be computed again from its first token, prompt and generated tokens together (a
+conv state cannot be rebuilt from the KV cache, so recomputation is the only exact way); it is not
+admitted again in the call that preempted it.  Its sampler state is kept, so its draws do not
+change.  A request that does not fit the pool even alone is finished with reason "capacity".
 
 The reference runs one request and has no scheduler; the loop shape follows its other
 backend's slot loop (src/qwen35/q35_server.c:869-1050): FIFO admission, prompt portions beside
@@ -90,6 +91,7 @@ class Scheduler:
         self.running: list[Request] = []          # in admission order
         self.finished: list[Request] = []
         self.num_preemptions = 0
+        self._decode_turn = 0                     # where the decoding requests' turns go on (budget < requests)
 
     # ------------------------------------------------------------------- requests
     def add(self, req: Request) -> None:
@@ -163,12 +165,47 @@ class Scheduler:
     def _total_pages(self) -> list[int]:
         return [g.pool.num_pages for g in self.manager.groups]
 
+    def _largest_fit(self, req: Request, n: int, promised: list[int]) -> int:
+        """The most tokens of `req`, at most n, whose pages are there (0: not even one)."""
+        if not self._fits(req, 1, promised):
+            return 0
+        lo, hi = 1, n                                         # lo fits; pages needed grow with the tokens
+        while lo < hi:
+            mid = (lo + hi + 1) // 2
+            if self._fits(req, mid, promised):
+                lo = mid
+            else:
+                hi = mid - 1
+        return lo
+
     def schedule(self, ahead: bool = False) -> Optional[list[Scheduled]]:
         """The next step.  ahead: the step before has been through advance() and not through
         commit(); tokens not yet seen appear as PLACEHOLDER in Scheduled.tokens (always as the one
         token of a decoding request).  Nobody can be preempted then, since a request's tokens must
         be known to compute it again: where a running request lacks pages the answer is None, and
-        nothing has been changed."""
+        nothing has been changed.
+
+        Who yields when pages are short: a prompt portion is cut to the pages there are, or waits a
+        step with what it holds; only a decoding request that cannot grow preempts, the most recently
+        admitted running request first.  If nothing at all can move (prompts holding all pages
+        between them), the most recently admitted one is preempted.  A request preempted in this call
+        is not admitted again in it."""
+        preempted_now: set[int] = set()
+        while True:
+            out = self._schedule_once(ahead, preempted_now)
+            if out is None or out or not self.running or ahead:
+                return out
+            # running requests and none can take a token: make room
+            victim = self.running[-1]
+            if len(self.running) == 1:
+                self.running.remove(victim)
+                self._end(victim.id)
+                self._finish(victim, "capacity")
+            else:
+                self._preempt(victim)
+                preempted_now.add(id(victim))
+
+    def _schedule_once(self, ahead: bool, preempted_now: set) -> Optional[list[Scheduled]]:
         budget = self.max_batched_tokens
         promised = [0] * len(self.manager.groups)
         out: list[Scheduled] = []
@@ -176,35 +213,27 @@ class Scheduler:
         # running requests, decoding ones first, then prompts in admission order
         rank = {id(r): i for i, r in enumerate(self.running)}
         order = sorted(self.running, key=lambda r: (r.remaining() != 1, rank[id(r)]))
+        n_decoding = sum(1 for r in order if r.remaining() == 1)
+        if n_decoding > budget:
+            # fewer tokens a step than decoding requests: they take turns, each step going on where
+            # the one before stopped
+            turn = self._decode_turn % n_decoding
+            order = order[turn:n_decoding] + order[:turn] + order[n_decoding:]
+            if not ahead:
+                self._decode_turn += budget
         for req in order:
             if req not in self.running or budget == 0:       # preempted meanwhile / nothing left
                 continue
             n = min(req.remaining(), budget)
-            while not self._fits(req, n, promised):
+            if not self._fits(req, n, promised):
                 if ahead:
                     return None
-                victim = self.running[-1]
-                if victim is req and len(self.running) == 1:
-                    # alone and still too large: shrink the portion, or give up
-                    while n > 1 and not self._fits(req, n, promised):
-                        n -= 1
-                    if not self._fits(req, n, promised):
-                        self.running.remove(req)
-                        self._end(req.id)
-                        self._finish(req, "capacity")
-                        n = 0
-                    break
-                scheduled_victim = next((s for s in out if s.request is victim), None)
-                if scheduled_victim is not None:
-                    out.remove(scheduled_victim)
-                    budget += len(scheduled_victim.tokens)
-                    promised = [0] * len(self.manager.groups)
-                    for s in out:
-                        self._promise(s.request, len(s.tokens), promised)
-                self._preempt(victim)
-                if victim is req:
-                    n = 0
-                    break
+                if req.remaining() > 1:
+                    # a prompt (or a request being computed again): what fits, or nothing this step
+                    n = self._largest_fit(req, n, promised)
+                else:
+                    n = self._make_room_for_a_decoding_request(req, out, promised, preempted_now)
+                    budget = self.max_batched_tokens - sum(len(s.tokens) for s in out)
             if n == 0:
                 continue
             self._promise(req, n, promised)
@@ -216,6 +245,8 @@ class Scheduler:
         while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs \
                 and self.manager.free_slots > 0:
             req = self.waiting[0]
+            if id(req) in preempted_now:
+                break
             total = len(req.prompt) + req.params.max_new_tokens
             need_alone = -(-total // self.manager.page_size)
             windows = [g.window for g in self.manager.groups]
@@ -226,10 +257,9 @@ class Scheduler:
             self._begin(req.id)
             n = min(req.remaining(), budget)
             if not self._fits(req, n, promised):
-                # try a shorter first portion; if not even one token fits, wait
-                while n > 1 and not self._fits(req, n, promised):
-                    n = n // 2
-                if not self._fits(req, n, promised) or self.running:
+                # a shorter first portion; if not even one token fits, wait
+                n = self._largest_fit(req, n, promised)
+                if n == 0 or self.running:
                     self._end(req.id)
                     break
             self.waiting.popleft()
@@ -240,6 +270,29 @@ class Scheduler:
             out.append(Scheduled(req, 0, toks, n == len(req.prompt) + len(req.output)))
             budget -= n
         return out
+
+    def _make_room_for_a_decoding_request(self, req: Request, out: list, promised: list[int], preempted_now: set) -> int:
+        """Preempts the most recently admitted running requests until req's one token has its page.
+        Returns the tokens req gets (1, or 0 if it went itself); `promised` is brought up to date
+        in place and entries of preempted requests leave `out`."""
+        while not self._fits(req, 1, promised):
+            victim = self.running[-1]
+            if victim is req and len(self.running) == 1:
+                self.running.remove(req)
+                self._end(req.id)
+                self._finish(req, "capacity")
+                return 0
+            scheduled_victim = next((s for s in out if s.request is victim), None)
+            if scheduled_victim is not None:
+                out.remove(scheduled_victim)
+                promised[:] = [0] * len(self.manager.groups)
+                for s in out:
+                    self._promise(s.request, len(s.tokens), promised)
+            self._preempt(victim)
+            preempted_now.add(id(victim))
+            if victim is req:
+                return 0
+        return 1
 
     def update(self, scheduled: list[Scheduled], sampled: dict) -> list[Request]:
         """sampled: {request id: token} for every Scheduled with samples=True.
