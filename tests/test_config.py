@@ -152,3 +152,40 @@ def test_run_order_is_data():
         DecoderModel(schedule=[LayerRun(0, cache=1), LayerRun(3, cache=1)], **kw)
     with pytest.raises(ValueError, match="cannot be shared"):
         DecoderModel(schedule=[LayerRun(1, cache=1), LayerRun(2, cache=1, writes=False)], **kw)
+
+
+def test_a_mixer_may_declare_several_cache_entries():
+    """cache_spec() returning a tuple: the run's entries are (cache, 0), (cache, 1), ...; sharing
+    such a run's paged entries works like sharing one, a fixed-size state among them forbids it."""
+    from tuff_amd.models.decoder import DecoderModel, LayerRun
+    from tuff_amd.parts.base import FixedState, Mixer, PagedKV
+    from tuff_amd.parts.block import PreNormBlock
+
+    class Keeps(Mixer):
+        def __init__(self, *specs):
+            self.specs = specs
+
+        def cache_spec(self):
+            return self.specs
+
+    base = registry.build_model(cfg_of(util.TINY_B))
+    n1 = base.blocks[0].norm1
+    kv_and_state = PreNormBlock(n1, Keeps(PagedKV(2, 8, 16), FixedState((5,), "bfloat16")))
+    two_kv = PreNormBlock(n1, Keeps(PagedKV(2, 8), PagedKV(1, 4, 16)))
+    nothing = PreNormBlock(n1, Keeps())
+    kw = dict(vocab_size=base.vocab_size, hidden_size=base.hidden_size, embedding=base.embedding_decl,
+              final_norm=base.final_norm, head=base.head_decl)
+    m = DecoderModel(blocks=[kv_and_state, base.blocks[1], two_kv, nothing], **kw)
+    assert m.cache_specs == {(0, 0): PagedKV(2, 8, 16), (0, 1): FixedState((5,), "bfloat16"), 1: FixedState((3, 96)),
+                             (2, 0): PagedKV(2, 8), (2, 1): PagedKV(1, 4, 16)}
+    views = {e: f"view of {e}" for e in m.cache_specs}
+    assert m._views_of(0, views) == ("view of (0, 0)", "view of (0, 1)") and m._views_of(1, views) == "view of 1"
+    assert m._views_of(3, views) == ()
+    from tuff_amd.cache.manager import CacheLayout
+    lay = CacheLayout.from_specs(m.cache_specs)
+    assert lay.group_windows == [16, None] and lay.group_of_entry == {(0, 0): 0, (2, 0): 1, (2, 1): 0}
+    assert lay.state_bytes_per_request() == 5 * 2 + 3 * 96 * 4
+    shared = DecoderModel(blocks=[two_kv], schedule=[LayerRun(0, cache=4), LayerRun(0, cache=4, writes=False)], **kw)
+    assert list(shared.cache_specs) == [(4, 0), (4, 1)]
+    with pytest.raises(ValueError, match="cannot be shared"):
+        DecoderModel(blocks=[kv_and_state], schedule=[LayerRun(0, cache=4), LayerRun(0, cache=4, writes=False)], **kw)

@@ -303,6 +303,116 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(gpu):
         registry.unregister_architecture("ToyLeakyForCausalLM")
 
 
+def test_toy_mixer_with_several_cache_entries(gpu):
+    """A mixer that keeps three things per request: the last input row (a convolution's tail), a
+    decaying matrix of outer products (a recurrent state) and a count of the tokens seen, in int32.
+    cache_spec() returns a tuple and forward() is handed a tuple of views.  Beside it in the same
+    model an attention layer with paged keys and values.  Whole, token by token and mixed, against a
+    plain loop; the counter must hold the request's length after every step."""
+    from tuff_amd.config.base import ModelConfig
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.models import registry
+    from tuff_amd.models.decoder import DecoderModel
+    from tuff_amd.parts.attention import AttentionMixer
+    from tuff_amd.parts.base import MIXERS, FixedState, Mixer, PagedKV, WeightDecl
+    from tuff_amd.parts.block import PreNormBlock
+    from tuff_amd.parts.ffn import SwiGLU
+    from tuff_amd.parts.norm import RMSNorm
+    from tuff_amd.weights.random_init import random_weights
+    d, dk, V, gamma, eps = 24, 8, 89, 0.8, 1e-5
+    seen_counts = {}
+
+    class TailAndMatrix(Mixer):
+        def __init__(self, d, dk, gamma, name):
+            self.d, self.dk, self.gamma, self.name = d, dk, gamma, name
+
+        def weight_decls(self):
+            return [WeightDecl(self.name, (self.d, self.d))]
+
+        def cache_spec(self):
+            return (FixedState((self.d,)), FixedState((self.dk, self.d)), FixedState((1,), "int32"))
+
+        def bind(self, weights, rt):
+            self.rt, self.w = rt, weights[self.name].float()
+
+        def forward(self, h, ctx, cache, residual, write_cache=True):
+            tail, matrix, count = cache                           # views in the order of the declarations
+            assert count.state.dtype == torch.int32 and matrix.state.shape[1:] == (self.dk, self.d)
+            hf = h.float()
+            slots = ctx.state_slot.tolist()
+            t = 0
+            for r, n in enumerate(ctx.host["q_len"].tolist()):
+                prev, S = tail.state[slots[r]].clone(), matrix.state[slots[r]].clone()
+                for i in range(n):
+                    x = hf[t + i]
+                    S = self.gamma * S + torch.outer(x[:self.dk], x + prev)
+                    residual[t + i] += (x[:self.dk] @ S) @ self.w.T
+                    prev = x
+                if write_cache:
+                    tail.state[slots[r]], matrix.state[slots[r]] = prev, S
+                    count.state[slots[r]] += n
+                    # zeroed when the slot was taken, then every token counted once, however the request was cut
+                    assert int(count.state[slots[r], 0]) == int(ctx.host["ctx_len"][r])
+                    seen_counts[slots[r]] = seen_counts.get(slots[r], 0) + 1
+                t += n
+
+    @dataclasses.dataclass
+    class Cfg(ModelConfig):
+        architecture: ClassVar[str] = "ToySeveralForCausalLM"
+        vocab_size: int
+
+    def build(cfg):
+        def ffn(i):
+            return SwiGLU(d, 40, names={"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"})
+        blocks = [PreNormBlock(RMSNorm(d, eps, "l0.n1"), MIXERS.get("tail_and_matrix")(d, dk, gamma, "l0.mix"),
+                               RMSNorm(d, eps, "l0.n2"), ffn(0)),
+                  PreNormBlock(RMSNorm(d, eps, "l1.n1"), AttentionMixer(d, 3, 1, 8, names={k: f"l1.{k}" for k in "qkvo"}),
+                               RMSNorm(d, eps, "l1.n2"), ffn(1))]
+        return DecoderModel(vocab_size=cfg.vocab_size, hidden_size=d, embedding=WeightDecl("emb", (cfg.vocab_size, d)),
+                            blocks=blocks, final_norm=RMSNorm(d, eps, "fn"))
+
+    MIXERS.register("tail_and_matrix", TailAndMatrix)
+    registry.register_architecture("ToySeveralForCausalLM", Cfg, build)
+    try:
+        model = registry.build_model(registry.config_from_dict({"architectures": ["ToySeveralForCausalLM"], "vocab_size": V}))
+        assert model.cache_specs == {(0, 0): FixedState((d,)), (0, 1): FixedState((dk, d)), (0, 2): FixedState((1,), "int32"),
+                                     1: PagedKV(1, 8, None)}
+        w32 = random_weights(model.weight_decls(), 5, torch.float32, "cpu")
+        eng = Engine(model, {k: v.to(gpu) for k, v in w32.items()}, dtype="float32", max_tokens=256, poison_cache=True)
+        assert len(eng.layout.states) == 3 and len(eng.layout.paged) == 1
+        assert eng.layout.state_bytes_per_request() == 4 * (d + dk * d + 1)
+        reqs = {"a": util.rand_tokens(21, V, 1), "b": util.rand_tokens(9, V, 2), "c": util.rand_tokens(14, V, 3)}
+        whole = util.run_plan(eng, util.plan_whole(reqs))
+        assert seen_counts
+        single = util.run_plan(eng, util.plan_tail(reqs, 100))
+        mixed = util.run_plan(eng, util.plan_mixed(reqs, seed=4, decode_tail=4))
+        w = {k: v.double() for k, v in w32.items()}
+        for rid, toks in reqs.items():
+            x = w["emb"][toks]
+            h = plain.rms_norm(x, w["l0.n1"], eps)
+            S, prev, rows = torch.zeros(dk, d, dtype=torch.float64), torch.zeros(d, dtype=torch.float64), []
+            for t in range(h.shape[0]):
+                S = gamma * S + torch.outer(h[t, :dk], h[t] + prev)
+                rows.append((h[t, :dk] @ S) @ w["l0.mix"].T)
+                prev = h[t]
+            x = x + torch.stack(rows)
+            x = x + plain.swiglu(plain.rms_norm(x, w["l0.n2"], eps), w["l0.g"], w["l0.u"], w["l0.d"])
+            h = plain.rms_norm(x, w["l1.n1"], eps)
+            q, k, v = (h @ w[f"l1.{n}"].T for n in "qkv")
+            o = torch.nn.functional.scaled_dot_product_attention(q.reshape(-1, 3, 8).transpose(0, 1)[None],
+                                                                 k.reshape(-1, 1, 8).transpose(0, 1)[None].expand(1, 3, -1, -1),
+                                                                 v.reshape(-1, 1, 8).transpose(0, 1)[None].expand(1, 3, -1, -1),
+                                                                 is_causal=True)[0].transpose(0, 1).reshape(-1, 24)
+            x = x + o @ w["l1.o"].T
+            x = x + plain.swiglu(plain.rms_norm(x, w["l1.n2"], eps), w["l1.g"], w["l1.u"], w["l1.d"])
+            want = plain.rms_norm(x, w["fn"], eps) @ w["emb"].T
+            for got in (whole, single, mixed):
+                util.assert_close_f32(got[rid], want, rid)
+    finally:
+        MIXERS.unregister("tail_and_matrix")
+        registry.unregister_architecture("ToySeveralForCausalLM")
+
+
 # ------------------------------------------------------- run order and cache groups as data
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_layer_run_twice_a_shared_cache_and_a_window_group(gpu, dtype):

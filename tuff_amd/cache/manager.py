@@ -75,7 +75,7 @@ class CacheGroup:
 @dataclasses.dataclass
 class CacheLayout:
     """Which cache entries exist and how they are grouped; derived from a model's run order."""
-    paged: dict[int, PagedKV]
+    paged: dict[int, PagedKV]                   # keyed by entry id: an int, or (int, j) for a mixer with several
     states: dict[int, FixedState]
     group_windows: list[Optional[int]]          # one per group
     group_of_entry: dict[int, int]
@@ -89,7 +89,7 @@ class CacheLayout:
             raise CacheError(f"unknown cache declaration {other[0]!r}")
         windows: list[Optional[int]] = []
         group_of = {}
-        for i in sorted(paged):
+        for i in sorted(paged, key=lambda e: e if isinstance(e, tuple) else (e, -1)):
             w = paged[i].window
             if w not in windows:
                 windows.append(w)
@@ -100,13 +100,7 @@ class CacheLayout:
         return sum(2 * s.num_kv_heads * s.head_dim * elem_size for s in self.paged.values())
 
     def state_bytes_per_request(self) -> int:
-        n = 0
-        for s in self.states.values():
-            k = 4
-            for d in s.shape:
-                k *= d
-            n += k
-        return n
+        return sum(s.nbytes() for s in self.states.values())
 
 
 @dataclasses.dataclass
@@ -130,6 +124,8 @@ class CacheManager:
                        for gi, (w, c) in enumerate(zip(layout.group_windows, counts))]
         self._free_slots = list(range(self.num_slots - 1, -1, -1))
         self._requests: dict[Hashable, _Request] = {}
+        #: debugging aid: called as on_free(group index, pages) whenever pages go back to a pool
+        self.on_free = None
 
     # ------------------------------------------------------------------ requests
     def __contains__(self, req_id) -> bool:
@@ -212,7 +208,7 @@ class CacheManager:
             gone = [p for p in r.tables[gi][:lo] if p != FREED]
             if gone:
                 r.arrays.pop(gi, None)
-                g.pool.free(gone)
+                self._give_back(gi, gone)
                 for b in range(min(lo, len(r.tables[gi]))):
                     r.tables[gi][b] = FREED
         need = self.pages_needed(req_id, n_new)
@@ -226,6 +222,11 @@ class CacheManager:
                 r.tables[gi].extend(g.pool.alloc(n))
         r.length += n_new
 
+    def _give_back(self, gi: int, pages: list) -> None:
+        self.groups[gi].pool.free(pages)
+        if pages and self.on_free is not None:
+            self.on_free(gi, pages)
+
     def truncate(self, req_id, length: int) -> None:
         """Takes back an extend(): the request holds `length` tokens again.  Pages beyond are
         returned; pages a window freed meanwhile stay freed."""
@@ -235,7 +236,7 @@ class CacheManager:
         keep = -(-length // self.page_size)
         for gi, g in enumerate(self.groups):
             extra = [p for p in r.tables[gi][keep:] if p != FREED]
-            g.pool.free(extra)
+            self._give_back(gi, extra)
             del r.tables[gi][keep:]
         r.arrays.clear()
         r.length = length
@@ -244,7 +245,7 @@ class CacheManager:
         """The request is over: all its pages and its slot are given back."""
         r = self._req(req_id)
         for gi, g in enumerate(self.groups):
-            g.pool.free([p for p in r.tables[gi] if p != FREED])
+            self._give_back(gi, [p for p in r.tables[gi] if p != FREED])
         self._free_slots.append(r.slot)
         del self._requests[req_id]
 

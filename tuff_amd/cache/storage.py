@@ -4,9 +4,10 @@ Per PagedKV entry: K as [num_pages, kv_heads, page_size, head_dim] and V transpo
 page, [num_pages, kv_heads, head_dim, page_size] (the matrix cores read both with the summed
 index contiguous), in the compute dtype
 (bfloat16 in serving, float32 in the 32-bit path; the reference keeps float32 rows
-[layer][kv_head][pos][hd], src/lfm25_gpu.cu:480-483).  Per FixedState entry: one float32
-tensor [num_slots, *shape].  Pages are not cleared when they are handed out again: nothing
-reads a position before it is written.  A state slot is zeroed when a request takes it
+[layer][kv_head][pos][hd], src/lfm25_gpu.cu:480-483).  Per FixedState entry: one
+tensor [num_slots, *shape] of the declared type (float32 unless the part says otherwise).  Pages are not cleared when they are handed out again: nothing
+reads a position before it is written (with poison=True the pool starts as NaN and pages are
+filled with NaN again when they are given back, which shows any such read).  A state slot is zeroed when a request takes it
 (the reference zeroes its conv state at start, src/lfm25_engine.c:46-51).
 """
 from __future__ import annotations
@@ -30,7 +31,18 @@ class PagedKVView:
 
 @dataclasses.dataclass
 class StateView:
-    state: torch.Tensor
+    state: torch.Tensor              # [num_slots, *shape] in the declared type
+    raw: torch.Tensor                # the same memory as int32 words [num_slots, words]
+
+
+_STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
+
+
+def _numel(shape) -> int:
+    n = 1
+    for d in shape:
+        n *= d
+    return n
 
 
 class CacheStorage:
@@ -53,13 +65,30 @@ class CacheStorage:
                 v = torch.empty(vshape, dtype=dtype, device=device)
             self.views[e] = PagedKVView(k, v, gi, ps, spec.window)
         for e, spec in layout.states.items():
-            st = torch.zeros((manager.num_slots,) + tuple(spec.shape), dtype=torch.float32, device=device)
-            self.views[e] = StateView(st)
+            # a slot is a whole number of 32-bit words, so that one fill kernel clears any type
+            words = -(-spec.nbytes() // 4)
+            raw = torch.zeros(manager.num_slots, words, dtype=torch.int32, device=device)
+            typed = raw.view(_STATE_DTYPES[spec.dtype])[:, :_numel(spec.shape)]
+            self.views[e] = StateView(typed.view((manager.num_slots,) + tuple(spec.shape)), raw)
+
+        if poison:
+            manager.on_free = self.poison_pages
+
+    def poison_pages(self, group: int, pages) -> None:
+        """Debugging aid (poison=True): pages that go back to the pool are filled with NaN, on the
+        stream, so that a later read of a position nobody has written since shows in the logits."""
+        idx = None
+        for v in self.views.values():
+            if isinstance(v, PagedKVView) and v.group == group:
+                if idx is None:
+                    idx = torch.tensor(list(pages), dtype=torch.long, device=v.k.device)
+                v.k[idx] = float("nan")
+                v.v[idx] = float("nan")
 
     def zero_slot(self, slot: int) -> None:
         for v in self.views.values():
             if isinstance(v, StateView):
-                ops.fill_u32(v.state[slot], 0)
+                ops.fill_u32(v.raw[slot], 0)
 
     def nbytes(self) -> int:
         n = 0
@@ -67,5 +96,5 @@ class CacheStorage:
             if isinstance(v, PagedKVView):
                 n += v.k.numel() * v.k.element_size() * 2
             else:
-                n += v.state.numel() * 4
+                n += v.raw.numel() * 4
         return n

@@ -10,7 +10,7 @@ from typing import Optional
 import torch
 
 from ..csrc import ops
-from ..parts.base import Block, FixedState, Norm, PagedKV, Runtime, WeightDecl
+from ..parts.base import Block, FixedState, Norm, PagedKV, Runtime, WeightDecl, cache_specs_of
 
 
 @dataclasses.dataclass(frozen=True)
@@ -53,22 +53,29 @@ class DecoderModel:
                 cache = next_id
                 used.add(cache)
             self.schedule.append(LayerRun(r.block, cache, r.writes))
-        # every cache entry has exactly one writer, which comes before its readers
-        self.cache_specs: dict[int, object] = {}
+        # Every cache entry has exactly one writer, which comes before its readers.  A run's entry is named
+        # by LayerRun.cache; a mixer that declares several things to keep has the entries (cache, 0),
+        # (cache, 1), ... in the order of its declarations.
+        self.cache_specs: dict = {}
+        self._run_entries: list = []             # per run: (the mixer declares a tuple, its entry ids)
+        written: dict = {}
         for r in self.schedule:
-            spec = self.blocks[r.block].mixer.cache_spec()
+            specs, several = cache_specs_of(self.blocks[r.block].mixer)
+            ids = tuple((r.cache, j) for j in range(len(specs))) if several else (r.cache,) * len(specs)
             if r.writes:
-                if r.cache in self.cache_specs:
+                if r.cache in written:
                     raise ValueError(f"cache entry {r.cache} has two writers")
-                self.cache_specs[r.cache] = spec
+                written[r.cache] = specs
+                self.cache_specs.update(zip(ids, specs))
             else:
-                if r.cache not in self.cache_specs:
+                if r.cache not in written:
                     raise ValueError(f"a run reads cache entry {r.cache} before any run writes it")
-                if self.cache_specs[r.cache] != spec:
+                if written[r.cache] != specs:
                     raise ValueError(f"a run reads cache entry {r.cache} of another shape: "
-                                     f"{self.cache_specs[r.cache]} vs {spec}")
-                if isinstance(spec, FixedState):
+                                     f"{written[r.cache]} vs {specs}")
+                if any(isinstance(s_, FixedState) for s_ in specs):
                     raise ValueError("a fixed-size state cannot be shared between runs")
+            self._run_entries.append((several, ids))
         self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
 
@@ -144,9 +151,9 @@ class DecoderModel:
                     nxt = nb.first_norm_consumer() if hasattr(nb, "first_norm_consumer") else None
                 else:
                     nxt = (self.final_norm, _HEAD) if head_fused and all_rows else None
-                block.forward(x, ctx, cache_views.get(run.cache), run.writes, next_norm=nxt)
+                block.forward(x, ctx, self._views_of(i, cache_views), run.writes, next_norm=nxt)
             else:
-                block.forward(x, ctx, cache_views.get(run.cache), run.writes)
+                block.forward(x, ctx, self._views_of(i, cache_views), run.writes)
         # which rows are wanted is a fact of the step, not of its shape: the head runs outside of what is recorded
         # (a recorder keeps the function and hands back what it returns at each replay)
         out: list = []
@@ -156,7 +163,23 @@ class DecoderModel:
             return out[0]
 
         ctx.run_eagerly(head)
+        for part in self.blocks + [self.final_norm]:
+            if hasattr(part, "forget"):                # what a product left for a norm that never asked for it
+                part.forget()
         return out[0] if out else None
+
+    def recording_key(self, ctx) -> tuple:
+        """What forward() reads of a step outside of ctx.run_eagerly and bakes into its launches: a
+        recording of a step in sections is valid for steps with the same key."""
+        head_fused, all_rows = self._head_fused(ctx)
+        return (ctx.T, bool(head_fused and all_rows))
+
+    def _views_of(self, i: int, cache_views: dict):
+        """What run i's mixer is handed as `cache`: None, a view, or a tuple of views."""
+        several, ids = self._run_entries[i]
+        if several:
+            return tuple(cache_views[e] for e in ids)
+        return cache_views[ids[0]] if ids else None
 
     def _head_fused(self, ctx) -> tuple:
         all_rows = ctx.n_logits == ctx.T and bool(ctx.host.get("logit_rows_identity", False))

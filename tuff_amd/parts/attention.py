@@ -86,7 +86,7 @@ class AttentionMixer(Mixer):
         if self.position is not None:
             self.position.bind(weights, rt)
 
-    def forward(self, h, ctx, cache, residual, write_cache: bool = True) -> None:
+    def forward(self, h, ctx, cache, residual, write_cache: bool = True, next_norm=None) -> None:
         T = h.shape[0]
         H, Hkv, hd = self.H, self.Hkv, self.hd
         qkv = self.qkv.forward(h)
@@ -117,7 +117,7 @@ class AttentionMixer(Mixer):
             self.attend(q, o, ctx, cache, g)
 
         ctx.run_eagerly(over_the_cache)
-        self.out.forward(o, accumulate_into=residual)
+        self.out.forward(o, accumulate_into=residual, next_norm=next_norm)
 
     @staticmethod
     def _upload(array, device):

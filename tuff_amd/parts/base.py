@@ -36,8 +36,27 @@ class PagedKV:
 
 @dataclasses.dataclass(frozen=True)
 class FixedState:
-    """Per-request state of fixed size, float32, zero for a new request."""
+    """Per-request state of fixed size, zero for a new request.  dtype: "float32", "bfloat16" or
+    "int32"."""
     shape: tuple
+    dtype: str = "float32"
+
+    def nbytes(self) -> int:
+        n = {"float32": 4, "bfloat16": 2, "int32": 4}[self.dtype]
+        for d in self.shape:
+            n *= d
+        return n
+
+
+def cache_specs_of(mixer) -> tuple:
+    """A mixer's cache declarations as a tuple (empty: it keeps nothing), and whether forward()
+    is handed a tuple of views (True) or one view / None (False)."""
+    spec = mixer.cache_spec()
+    if spec is None:
+        return (), False
+    if isinstance(spec, (tuple, list)):
+        return tuple(spec), True
+    return (spec,), False
 
 
 @dataclasses.dataclass
@@ -81,8 +100,9 @@ class Part:
     accepts_pending_norm = False
 
     #: True if forward() touches the residual stream exactly once, as its last operation, through
-    #: Linear.forward(accumulate_into=residual).  The block may then let that product prepare the
-    #: operand of the norm that follows (see Linear.forward).
+    #: Linear.forward(accumulate_into=residual, next_norm=next_norm), and takes a keyword next_norm
+    #: for it.  The block then tells it which norm reads the stream next, and that product may
+    #: leave the norm its operand (see Linear.forward).
     adds_once_through_linear = False
 
 
@@ -118,9 +138,16 @@ class Mixer(Part):
     """
 
     def cache_spec(self):
+        """None, one declaration (PagedKV or FixedState), or a tuple of declarations for a mixer
+        that keeps several things per request (keys and values beside a state, a convolution's
+        tail beside a recurrent matrix).  forward() gets None, one view, or a tuple of views in
+        the order of the declarations."""
         return None
 
     def forward(self, h, ctx, cache, residual, write_cache: bool = True) -> None:
+        """A mixer with adds_once_through_linear is also passed next_norm=<Norm or None>: the
+        norm that reads the residual stream right after this mixer, to be handed on to the
+        Linear that adds into it (Linear.forward(..., next_norm=...))."""
         raise NotImplementedError
 
 
@@ -128,6 +155,7 @@ class FeedForward(Part):
     """forward(h [T, d] compute dtype, ctx, residual float32 [T, d]) adds its output."""
 
     def forward(self, h, ctx, residual) -> None:
+        """As for mixers: with adds_once_through_linear the call carries next_norm=<Norm or None>."""
         raise NotImplementedError
 
 

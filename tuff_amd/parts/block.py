@@ -50,24 +50,29 @@ class PreNormBlock(Block):
     def forward(self, x, ctx, cache, write_cache: bool = True, next_norm=None) -> None:
         """next_norm: (norm, consumer) that will read x right after this block, or None."""
         h = self._normed(self.norm1, x, self.mixer)
-        self._announce(x, self.mixer, (self.norm2, self.ffn) if self.ffn is not None else next_norm)
-        self.mixer.forward(h, ctx, cache, x, write_cache)
+        after = self._hand_over(self.mixer, (self.norm2, self.ffn) if self.ffn is not None else next_norm)
+        self.mixer.forward(h, ctx, cache, x, write_cache, **after)
         if self.ffn is not None:
             h = self._normed(self.norm2, x, self.ffn)
-            self._announce(x, self.ffn, next_norm)
-            self.ffn.forward(h, ctx, x)
-        self._announce(x, None, None)
+            after = self._hand_over(self.ffn, next_norm)
+            self.ffn.forward(h, ctx, x, **after)
+
+    def forget(self) -> None:
+        """End of a step: drops what a product left for a norm that never asked for it."""
+        for n in (self.norm1, self.norm2):
+            if hasattr(n, "forget"):
+                n.forget()
 
     @staticmethod
-    def _announce(x, producer, nxt) -> None:
-        """Tells the producer's last projection (through an attribute of x) which norm reads x next,
-        if producer, norm and the norm's consumer all know the protocol."""
-        ok = (producer is not None and nxt is not None and producer.adds_once_through_linear
-              and hasattr(nxt[0], "announce_operand") and nxt[1] is not None and nxt[1].accepts_pending_norm)
-        if ok:
-            x._tuff_next_norm = nxt[0]
-        elif hasattr(x, "_tuff_next_norm"):
-            del x._tuff_next_norm
+    def _hand_over(producer, nxt) -> dict:
+        """The keyword that tells the producer's last projection which norm reads x next: only if
+        producer, norm and the norm's consumer all know how (else nothing is passed and the norm
+        runs as a kernel of its own)."""
+        if not producer.adds_once_through_linear:
+            return {}
+        ok = (nxt is not None and hasattr(nxt[0], "announce_operand") and nxt[1] is not None
+              and nxt[1].accepts_pending_norm)
+        return {"next_norm": nxt[0] if ok else None}
 
     @staticmethod
     def _normed(norm, x, consumer):

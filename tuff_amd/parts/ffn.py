@@ -57,11 +57,11 @@ class SwiGLU(FeedForward):
         self.gate_up.bind(weights, rt)
         self.down.bind(weights, rt)
 
-    def forward(self, h, ctx, residual) -> None:
+    def forward(self, h, ctx, residual, next_norm=None) -> None:
         if self.gate_up.interleaved:
             act = self.gate_up.forward(h, swiglu=True)          # silu(gate) * up in the product's epilogue
         else:
             gu = self.gate_up.forward(h)
             act = self.rt.empty(h.shape[0], self.width, dtype=gu.dtype)
             ops.swiglu(gu, act)
-        self.down.forward(act, accumulate_into=residual)
+        self.down.forward(act, accumulate_into=residual, next_norm=next_norm)

@@ -56,10 +56,13 @@ class Linear:
             self.weight = ops.tile_weight(self.weight)       # the order the kernels stream it in
 
     def forward(self, x, *, out_dtype: Optional[torch.dtype] = None,
-                accumulate_into: Optional[torch.Tensor] = None, swiglu: bool = False) -> Optional[torch.Tensor]:
+                accumulate_into: Optional[torch.Tensor] = None, swiglu: bool = False,
+                next_norm=None) -> Optional[torch.Tensor]:
         """x [T, in] in the compute dtype, or a PendingNorm.  Returns a new [T, out] tensor of
         `out_dtype` (default: the compute dtype), or adds into `accumulate_into` (float32) and
-        returns None.  swiglu (interleaved pairs only): returns silu(gate) * up, [T, out/2]."""
+        returns None.  swiglu (interleaved pairs only): returns silu(gate) * up, [T, out/2].
+        next_norm (with accumulate_into): the norm that reads the sum next; where the kernels can,
+        the product leaves it its operand and row sums (norm.announce_operand)."""
         from .norm import PendingNorm
         w = self.weight
         if swiglu and not self.interleaved:
@@ -95,7 +98,7 @@ class Linear:
 
         dev = w.device
         if accumulate_into is not None:
-            nxt = getattr(accumulate_into, "_tuff_next_norm", None)
+            nxt = next_norm
             if (nxt is not None and pending is None and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
                     and T <= ops.EMIT_MAX_ROWS):
                 # the norm that follows reads the sum just made: leave it its operand and row sums

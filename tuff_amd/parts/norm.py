@@ -68,6 +68,10 @@ class RMSNorm(Norm):
         xw = bf16(x * weight) and the per-tile sums of squares ss: the next pending(x) carries them."""
         self._ready = (x, xw, ss)
 
+    def forget(self) -> None:
+        """Drops what announce_operand() left, if nobody asked for it (end of a step)."""
+        self._ready = None
+
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         n = x.shape[0] if rows is None else rows.shape[0]
         out = self.rt.empty(n, self.dim)

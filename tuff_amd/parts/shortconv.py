@@ -53,18 +53,18 @@ class ShortConvMixer(Mixer):
         self.out_proj.bind(weights, rt)
         self.conv_w = weights[self.names["conv"]].reshape(self.d, self.K).contiguous()
 
-    def forward(self, h, ctx, cache, residual, write_cache: bool = True) -> None:
+    def forward(self, h, ctx, cache, residual, write_cache: bool = True, next_norm=None) -> None:
         T = h.shape[0]
         bcx = self.in_proj.forward(h)
         y = self.rt.empty(T, self.d)
         if write_cache and ctx.max_q_len == 1:
             # single tokens only: one kernel reads the state, writes the output and the new state
             ops.shortconv_decode(bcx, self.conv_w, cache.state, y, state_slot=ctx.state_slot, K=self.K)
-            self.out_proj.forward(y, accumulate_into=residual)
+            self.out_proj.forward(y, accumulate_into=residual, next_norm=next_norm)
             return
         ops.shortconv_fwd(bcx, self.conv_w, cache.state, y, req_of_token=ctx.req_of_token,
                           q_start=ctx.q_start, state_slot=ctx.state_slot, K=self.K)
         if write_cache:
             ops.shortconv_state(bcx, cache.state, q_start=ctx.q_start, q_len=ctx.q_len,
                                 state_slot=ctx.state_slot, K=self.K)
-        self.out_proj.forward(y, accumulate_into=residual)
+        self.out_proj.forward(y, accumulate_into=residual, next_norm=next_norm)
