@@ -5,7 +5,14 @@ weights (16 layers, 6 of them attention; hidden 2048), plus the 2,048-token pref
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
 
 A "step" is one decode step of the whole batch through the serving loop (step function, greedy
-pick on the GPU, the ids back on the host).  Prints one JSON line.
+pick on the GPU, the ids back on the host).  Every point is measured in RUNS runs of its own
+(requests made and brought to their context anew); the value is the mean over the runs and `spread`
+half the distance between the fastest and the slowest, as the reference reports its speeds
+(src/main.c:1891-1904).  Prints one JSON line.
+
+`probe` in that line is what this machine gives the product's own kernels where nothing but the memory
+or the matrix cores bounds them (a product of 8 rows with 268 MB of weights, a product of 8192^3): the
+denominators one may want beside the published peaks, which `roofline` and `frac` are priced against.
 """
 from __future__ import annotations
 
@@ -108,12 +115,14 @@ def run_decode(llm, cfg, batch: int, ctx_end: int, steps: int, warmup: int, seed
 
 
 def run_prefill(llm, cfg, tokens: int, repeats: int = 8):
+    """One prompt of `tokens` tokens in one step, to the first generated token on the host.  Returns
+    the seconds of `repeats` runs (one more, the first, warms up and is left out)."""
     import torch
     from tuff_amd.csrc import ops
     from tuff_amd.engine.batch import StepEntry
     eng = llm.engine
     g = torch.Generator().manual_seed(SEED + 1)
-    best = None
+    times = []
     picked = torch.empty(1, dtype=torch.int32, device=eng.device)
     for i in range(repeats + 1):
         prompt = torch.randint(0, cfg.vocab_size, (tokens,), generator=g).tolist()
@@ -126,9 +135,62 @@ def run_prefill(llm, cfg, tokens: int, repeats: int = 8):
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         eng.end(("prefill", i))
-        if i > 0:                                         # the first run warms up; the best of the rest counts
-            best = dt if best is None else min(best, dt)
-    return best
+        if i > 0:
+            times.append(dt)
+    return times
+
+
+def mean_spread(values):
+    return sum(values) / len(values), (max(values) - min(values)) / 2.0
+
+
+def prefill_record(times, flops: float, dtype: str) -> dict:
+    dt, spread = mean_spread(times)
+    return {"value": round(PREFILL_TOKENS / dt, 1), "tokens": PREFILL_TOKENS, "ms": round(dt * 1e3, 3),
+            "frac": round(flops / dt / (PEAK_TFLOPS[dtype] * 1e12), 4), "runs": len(times),
+            "spread_ms": round(spread * 1e3, 3)}
+
+
+def probe(device) -> dict:
+    """What the machine gives the product's own kernels at their best shapes."""
+    import torch
+    from tuff_amd.csrc import ops
+    g = torch.Generator(device=device).manual_seed(1)
+    out = {}
+    # read bandwidth: y = x W^T with 8 rows and 268 MB of weights, over four copies in turn (1 GB: more than any cache)
+    N, K = 65536, 2048
+    ws = [ops.tile_weight((torch.randn(N, K, generator=g, device=device) * 0.02).to(torch.bfloat16)) for _ in range(4)]
+    x = torch.randn(8, K, generator=g, device=device).to(torch.bfloat16)
+    y = torch.empty(8, N, dtype=torch.float32, device=device)
+    for reps, keep in ((4, False), (40, True)):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for i in range(reps):
+            ops.gemm(x, ws[i % 4], y)
+        end.record()
+        torch.cuda.synchronize()
+        if keep:
+            gbs = reps * N * K * 2 / (start.elapsed_time(end) * 1e-3) / 1e9
+            out["read_GBs"] = round(gbs, 1)
+            out["read_frac_of_published"] = round(gbs / HBM_PEAK_GBS, 4)
+    del ws
+    # matrix cores: a bfloat16 product of 8192^3
+    n = 8192
+    a = (torch.randn(n, n, generator=g, device=device) * 0.02).to(torch.bfloat16)
+    w = ops.tile_weight((torch.randn(n, n, generator=g, device=device) * 0.02).to(torch.bfloat16))
+    c = torch.empty(n, n, dtype=torch.bfloat16, device=device)
+    for reps, keep in ((2, False), (10, True)):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            ops.gemm(a, w, c)
+        end.record()
+        torch.cuda.synchronize()
+        if keep:
+            tf = reps * 2.0 * n ** 3 / (start.elapsed_time(end) * 1e-3) / 1e12
+            out["mfma_bf16_TFLOPs"] = round(tf, 1)
+            out["mfma_frac_of_published"] = round(tf / PEAK_TFLOPS["bf16"], 4)
+    return out
 
 
 # Two serving runs through the scheduler, on other shapes of the architecture: many requests of very
@@ -150,7 +212,7 @@ SCENARIOS = {
 }
 
 
-def run_scenario(name: str, dtype: str) -> dict:
+def run_scenario(name: str, dtype: str, runs: int = 3) -> dict:
     import math
     import random
     import torch
@@ -173,19 +235,23 @@ def run_scenario(name: str, dtype: str) -> dict:
               ctx_size=cfg.max_position_embeddings, ignore_eos=True)
     g = torch.Generator().manual_seed(SEED)
     prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=g).tolist() for n in lens]
-    best = None
-    for _ in range(2):                                     # the first run warms up
+    times = []
+    for run in range(runs + 1):                            # the first run warms up
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         outs = llm.generate(prompts, SamplingParams(max_new_tokens=new, ignore_eos=True))
         torch.cuda.synchronize()
-        best = time.perf_counter() - t0
+        if run:
+            times.append(time.perf_counter() - t0)
         if not all(len(o.token_ids) == new for o in outs):
             raise RuntimeError("a request of the scenario did not run to its end")
     total = sum(lens) + len(lens) * new
     st = llm.last_stats
-    return {"metric": f"tokens/s through the scheduler, prompts and generated ({name})", "value": round(total / best, 1),
-            "unit": "tokens/s", "n_gpus": 1, "seconds": round(best, 3), "generated_per_s": round(len(lens) * new / best, 1),
+    rate, spread = mean_spread([total / t for t in times])
+    best = sum(times) / len(times)
+    return {"metric": f"tokens/s through the scheduler, prompts and generated ({name})", "value": round(rate, 1),
+            "unit": "tokens/s", "n_gpus": 1, "runs": len(times), "spread": round(spread, 1),
+            "seconds": round(best, 3), "generated_per_s": round(len(lens) * new / best, 1),
             "dtype": dtype, "data": "synthetic: seeded random weights, uniform random token ids",
             "config": {"scenario": name, "requests": len(lens), "at_a_time": sc["at_a_time"], "prompt_tokens": sum(lens),
                        "longest_prompt": max(lens), "new_tokens_each": new, "max_batched_tokens": sc["budget"],
@@ -205,6 +271,9 @@ def main() -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--point-steps", type=int, default=96)
+    ap.add_argument("--runs", type=int, default=3, help="runs a point (mean and spread over them)")
+    ap.add_argument("--no-probe", dest="probe", action="store_false",
+                    help="skip the measurement of the machine's own read bandwidth and matrix rate")
     ap.add_argument("--only-prefill", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiling) and print its record")
     ap.add_argument("--scenario", choices=sorted(SCENARIOS),
@@ -218,7 +287,7 @@ def main() -> int:
         return 2
 
     if args.scenario:
-        print(json.dumps(run_scenario(args.scenario, "bfloat16" if args.dtype == "bf16" else "float32")))
+        print(json.dumps(run_scenario(args.scenario, "bfloat16" if args.dtype == "bf16" else "float32", args.runs)))
         return 0
 
     import torch
@@ -233,20 +302,27 @@ def main() -> int:
     llm = LLM(engine=eng, max_num_seqs=max_b, max_batched_tokens=2048, ctx_size=args.context, ignore_eos=True)
     model = eng.model
 
+    flops = prefill_flops(cfg, model, PREFILL_TOKENS)
     if args.only_prefill:
-        dt = run_prefill(llm, cfg, PREFILL_TOKENS)
-        flops = prefill_flops(cfg, model, PREFILL_TOKENS)
-        print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / dt, 1), "tokens": PREFILL_TOKENS,
-                                      "ms": round(dt * 1e3, 3),
-                                      "frac": round(flops / dt / (PEAK_TFLOPS[args.dtype] * 1e12), 4)}}))
+        print(json.dumps({"prefill": prefill_record(run_prefill(llm, cfg, PREFILL_TOKENS), flops, args.dtype)}))
         return 0
-    secs, ctx_mean = run_decode(llm, cfg, args.batch, args.context, args.steps, args.warmup, SEED)
-    tok_s = args.batch * args.steps / secs
-    ms_step = 1e3 * secs / args.steps
-    achieved = decode_bytes(cfg, model, eng, args.batch, ctx_mean) / (secs / args.steps) / 1e9
+
+    def decode_point(batch: int, steps: int, warmup: int, seed: int) -> dict:
+        secs, ctx_mean = [], 0.0
+        for run in range(args.runs):
+            s_, ctx_mean = run_decode(llm, cfg, batch, args.context, steps, warmup, seed + 1000 * run)
+            secs.append(s_)
+        rates = [batch * steps / s_ for s_ in secs]
+        rate, spread = mean_spread(rates)
+        step_s = sum(secs) / len(secs) / steps
+        gbs = decode_bytes(cfg, model, eng, batch, ctx_mean) / step_s / 1e9
+        return {"tok_s": rate, "spread": spread, "ms": 1e3 * step_s, "GBs": gbs}
+
+    head = decode_point(args.batch, args.steps, args.warmup, SEED)
     out = {
-        "metric": "decode tok/s at batch 8, context 8192 (LFM2.5-1.2B shape)", "value": round(tok_s, 1), "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
+        "metric": "decode tok/s at batch 8, context 8192 (LFM2.5-1.2B shape)", "value": round(head["tok_s"], 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(head["ms"], 4),
+        "runs": args.runs, "spread": round(head["spread"], 1),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
         "data": "synthetic: seeded random weights (seed 2), uniform random token ids",
         "config": {
@@ -259,19 +335,23 @@ def main() -> int:
             "prefill_tokens": PREFILL_TOKENS, "page_size": page, "parameters": model.num_parameters(),
             "norm_eps": cfg.norm_eps, "rope_theta": cfg.rope_theta,
             "parallelism": "single GPU"},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(head["GBs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(head["GBs"] / HBM_PEAK_GBS, 4)},
     }
     if not args.no_points:
-        dt = run_prefill(llm, cfg, PREFILL_TOKENS)
-        flops = prefill_flops(cfg, model, PREFILL_TOKENS)
-        out["prefill"] = {"value": round(PREFILL_TOKENS / dt, 1), "tokens": PREFILL_TOKENS, "ms": round(dt * 1e3, 3),
-                          "frac": round(flops / dt / (PEAK_TFLOPS[args.dtype] * 1e12), 4)}
+        out["prefill"] = prefill_record(run_prefill(llm, cfg, PREFILL_TOKENS), flops, args.dtype)
         points = {}
         for b in (1, 64):
-            s, _ = run_decode(llm, cfg, b, args.context, args.point_steps, 8, SEED + b)
-            points[f"decode_b{b}"] = round(b * args.point_steps / s, 1)
+            pt = decode_point(b, args.point_steps, 8, SEED + b)
+            points[f"decode_b{b}"] = round(pt["tok_s"], 1)
+            points[f"decode_b{b}_spread"] = round(pt["spread"], 1)
+            points[f"decode_b{b}_ms_per_step"] = round(pt["ms"], 4)
+            points[f"decode_b{b}_GBs"] = round(pt["GBs"], 1)
+            points[f"decode_b{b}_roofline_frac"] = round(pt["GBs"] / HBM_PEAK_GBS, 4)
         out["points"] = points
+    if args.probe and args.dtype == "bf16":
+        del llm
+        out["probe"] = probe(eng.device)
     print(json.dumps(out))
     return 0
 

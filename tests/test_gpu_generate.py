@@ -126,6 +126,46 @@ def test_preemption_does_not_change_the_output(gpu):
     assert not tight.engine.manager.live()
 
 
+def test_bfloat16_tokens_change_with_the_neighbours_only_at_near_ties(gpu, capsys):
+    """In bfloat16 the kernels a token goes through depend on the step it is in (products of up to 16,
+    up to 64 or more rows, single-token or portion attention), so its logits carry another rounding
+    with other neighbours.  Greedy tokens of six requests run together under a small budget, again
+    with so few pages that requests are preempted and computed again, and each alone: where a
+    request's tokens differ from its tokens alone, the plain model's top two logits at that step
+    (along the tokens it produced alone) are within the bound the logits' rounding allows."""
+    from tuff_amd.engine.llm import LLM
+    from tuff_amd.sampling.params import SamplingParams
+    name, n_new, tie = "B", 40, 2e-2
+    V = util.CONFIGS[name][0]["vocab_size"]
+    prompts = [util.rand_tokens(n, V, 300 + n) for n in (5, 37, 18, 70, 9, 52)]
+    p = SamplingParams(max_new_tokens=n_new)
+    folder = util.model_folder(name, "bfloat16")
+    alone_llm = LLM(folder, dtype="bfloat16", max_num_seqs=1, ctx_size=128)
+    alone = [alone_llm.generate([q], p)[0].token_ids for q in prompts]
+    cfg, w = util.plain_model(name, "bfloat16")
+    margins = []
+    for q, toks in zip(prompts, alone):
+        rows = plain.forward_logits(cfg, w, q + toks)[len(q) - 1:-1]
+        top = torch.topk(rows, 2, dim=-1).values
+        margins.append((top[:, 0] - top[:, 1]).tolist())
+    together = LLM(folder, dtype="bfloat16", max_num_seqs=6, max_batched_tokens=24, ctx_size=128)
+    tight = LLM(folder, dtype="bfloat16", max_num_seqs=6, max_batched_tokens=24, ctx_size=128, num_pages=20)
+    report = {}
+    for tag, llm in (("together", together), ("tight pool", tight)):
+        outs = [o.token_ids for o in llm.generate(prompts, p)]
+        diverged = 0
+        for i, (got, want) in enumerate(zip(outs, alone)):
+            assert len(got) == n_new
+            cut = agree_up_to_near_ties(got, want, margins[i], tie)
+            diverged += cut < n_new
+        report[tag] = diverged
+        llm.engine.manager.check()
+        assert not llm.engine.manager.live()
+    assert tight.last_stats["preemptions"] >= 1
+    with capsys.disabled():
+        print(f"\n[bf16 neighbours] requests whose greedy tokens left their tokens alone at a near-tie, of {len(prompts)}: {report}")
+
+
 def test_eos_stops_a_request(gpu):
     from tuff_amd.engine.llm import LLM
     from tuff_amd.sampling.params import SamplingParams
@@ -209,6 +249,16 @@ def test_command_line(gpu, tmp_path):
     # timed mode prints the speed line; usage errors give 2; a broken model gives 1
     p5 = _tuff("--model", folder, "--prompt-ids", ids, "-n", "8", "--warmup", "2", "--runs", "2")
     assert p5.returncode == 0 and "Pipeline Generation Speed" in p5.stdout, p5.stderr
+    assert "[Tuff timing]" not in p5.stderr
+    # TUFF_TIMING=1: a line per phase on standard error, seconds since the mark before and since the start
+    env = dict(os.environ, TUFF_TIMING="1")
+    p6 = subprocess.run([sys.executable, os.path.join(util.ROOT, "bin", "tuff"), "--model", folder, "--prompt-ids", ids,
+                         "-n", "4", "--warmup", "1", "--runs", "1"], capture_output=True, text=True, timeout=300, env=env)
+    marks = [l for l in p6.stderr.splitlines() if l.startswith("[Tuff timing] ")]
+    assert p6.returncode == 0 and [m.split(": ")[0][14:] for m in marks] == \
+        ["config", "model_load", "run 0: prefill", "run 0: warmup", "run 0: decode"], p6.stderr
+    ts = [float(m.split("(t=")[1].rstrip(")")) for m in marks]
+    assert ts == sorted(ts) and all(" s (t=" in m for m in marks)
     assert _tuff("--model", folder).returncode == 2
     assert _tuff("--model", folder, "--prompt-ids", ids, "-n", "5000").returncode == 2
     assert _tuff("--model", str(tmp_path), "--prompt-ids", ids).returncode == 1

@@ -14,7 +14,7 @@ LENGTHS = [45, 70, 100, 33, 129, 64]
 
 
 def requests_for(name):
-    V = util.CONFIGS[name][0]["vocab_size"]
+    V = util.CONFIGS[name.rstrip("+")][0]["vocab_size"]
     return {f"r{i}": util.rand_tokens(n, V, 100 * i + len(name)) for i, n in enumerate(LENGTHS)}
 
 
@@ -26,6 +26,7 @@ def make_engine(name, dtype, **kw):
     from tuff_amd.engine.engine import Engine
     kw.setdefault("page_size", 16)
     kw.setdefault("max_tokens", 1024)
+    kw.setdefault("poison_cache", True)          # NaN in every page that nobody has written since it was handed out
     return Engine.from_folder(util.model_folder(name, stored_for(dtype)), dtype=dtype, **kw)
 
 
@@ -45,6 +46,19 @@ def check_plan(name, dtype, plan, reqs, **kw):
 def test_whole(gpu, name, dtype):
     reqs = requests_for(name)
     check_plan(name, dtype, util.plan_whole(reqs), reqs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A+", "B+"])
+def test_loud_conv_mixers(gpu, name, dtype):
+    """The conv mixers' weights scaled up until they add more than the residual stream holds: a fault in
+    the conv state (a wrong slot, a wrong shift, a state that a portion's edge loses) then shows in
+    bfloat16 too, where random weights of the usual size would hide it under the rounding."""
+    reqs = requests_for(name)
+    check_plan(name, dtype, util.plan_tail(reqs, 32), reqs)
+    check_plan(name, dtype, util.plan_chunks(reqs, sizes=(2, 3, 2, 29, 5)), reqs)
+    plan = util.plan_mixed(reqs, seed=6)
+    check_plan(name, dtype, plan, reqs, max_tokens=util.live_tokens_peak(plan), max_requests=4)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -84,11 +98,10 @@ def test_mixed_with_page_reuse(gpu, name, dtype):
         assert pool.allocations > pool.num_pages, "the pool was so large that no page was used again"
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_splits_agree_with_each_other(gpu, dtype):
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("C", "float32"), ("B", "bfloat16")])
+def test_splits_agree_with_each_other(gpu, name, dtype):
     """The same logits whatever the cutting: bitwise in float32 where the kernels keep one order
     of summation per position, to rounding in bfloat16."""
-    name = "B"
     reqs = requests_for(name)
     eng = make_engine(name, dtype)
     whole = util.run_plan(eng, util.plan_whole(reqs))
@@ -334,11 +347,16 @@ def test_layers_of_full_size_float32_against_the_plain_implementation(gpu):
     folder = util.model_folder(name, "bfloat16")            # both paths read these bfloat16 weights
     eng = Engine.from_folder(folder, dtype="float32", page_size=16, max_tokens=256)
     want = {rid: util.plain_logits(name, toks, "bfloat16") for rid, toks in reqs.items()}
-    for plan in (util.plan_whole(reqs), util.plan_tail(reqs, 8), util.plan_mixed(reqs, seed=2, decode_tail=6)):
+    first = None
+    for plan in (util.plan_whole(reqs), util.plan_tail(reqs, 8), util.plan_mixed(reqs, seed=2, decode_tail=6),
+                 util.plan_chunks(reqs)):
         got = util.run_plan(eng, plan)
         eng.manager.check()
         for rid in reqs:
             util.assert_close_f32(got[rid], want[rid], f"full-size float32 {rid}")
+        first = first or got
+        for rid in reqs:                                    # and bitwise the same however the requests were cut
+            assert torch.equal(got[rid], first[rid]), f"full-size float32 {rid}: logits depend on the cutting"
     del eng
     eng16 = Engine.from_folder(folder, dtype="bfloat16", page_size=16, max_tokens=256)
     got16 = util.run_plan(eng16, util.plan_whole(reqs))

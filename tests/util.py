@@ -51,14 +51,31 @@ CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 5), "D": (TINY_D, 9
 _TMP = tempfile.TemporaryDirectory(prefix="tuff_amd_tests_")
 
 
+# With N(0, 0.02) weights a short-conv mixer adds about a thousandth of the residual stream's size (three
+# small projections and the taps multiply), which bfloat16 rounding hides: a wrong conv state would pass.
+# The "loud" variant of a configuration ("A+", "B+") scales the conv mixers' tensors so that they add about
+# the stream's own size and a fault in them shows in either precision.
+LOUD_CONV = {"conv.in_proj.weight": 3.0, "conv.conv.weight": 12.0, "conv.out_proj.weight": 2.0}
+
+
 @functools.lru_cache(maxsize=None)
 def model_folder(name: str, stored: str = "bfloat16") -> str:
-    """A model folder of configuration `name` with random weights, made once per session."""
+    """A model folder of configuration `name` with random weights, made once per session.
+    name + "+": the same with loud conv mixers."""
     from tuff_amd.models.registry import config_from_dict
     from tuff_amd.weights.random_init import write_random_model
-    raw, seed = CONFIGS[name]
-    out = os.path.join(_TMP.name, f"{name}_{stored}")
+    raw, seed = CONFIGS[name.rstrip("+")]
+    out = os.path.join(_TMP.name, f"{name.replace('+', '_loud')}_{stored}")
     write_random_model(config_from_dict(raw), out, seed, getattr(torch, stored))
+    if name.endswith("+"):
+        from safetensors.torch import load_file, save_file
+        path = os.path.join(out, "model.safetensors")
+        tensors = load_file(path)
+        for k in tensors:
+            for suffix, factor in LOUD_CONV.items():
+                if k.endswith(suffix):
+                    tensors[k] = (tensors[k].float() * factor).to(tensors[k].dtype)
+        save_file(tensors, path)
     return out
 
 

@@ -30,7 +30,9 @@ def _ids_from(text_or_path: str) -> list[int]:
 
 
 def build_parser() -> argparse.ArgumentParser:
-    ap = argparse.ArgumentParser(prog="tuff", description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap = argparse.ArgumentParser(prog="tuff", description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter,
+                                 epilog="Environment: TUFF_TIMING=1 prints one line per phase (configuration, model load, "
+                                        "prefill, warm-up, decode) with its seconds on standard error.")
     ap.add_argument("--model", help="model folder (config.json + model.safetensors)")
     ap.add_argument("--random", metavar="CONFIG_JSON", help="random weights for this config.json instead of --model")
     ap.add_argument("--prompt", "-p", help="prompt text (needs tokenizer.json in the model folder)")
@@ -166,8 +168,33 @@ def _run_jobs(argv: list) -> int:
     return overall
 
 
+class _Timing:
+    """TUFF_TIMING=1: one line per phase on stderr, "[Tuff timing] <phase>: <seconds since the mark
+    before> s (t=<seconds since the run began>)", as the reference prints them (src/main.c:204-225).
+    A mark waits for the GPU first, so a phase's time holds the work it started."""
+
+    def __init__(self):
+        self.on = os.environ.get("TUFF_TIMING", "")[:1] == "1"
+        self.start = self.last = time.monotonic()
+
+    def mark(self, what: str, sync: bool = True) -> None:
+        if not self.on:
+            return
+        if sync:
+            try:
+                import torch
+                if torch.cuda.is_available():
+                    torch.cuda.synchronize()
+            except Exception:                                # noqa: BLE001 - a mark never ends a run
+                pass
+        now = time.monotonic()
+        print(f"[Tuff timing] {what}: {now - self.last:.3f} s (t={now - self.start:.3f})", file=sys.stderr)
+        self.last = now
+
+
 def _run(argv: list, loaded: dict) -> int:
     """One run.  `loaded` keeps the engine from one run of a job file to the next."""
+    tm = _Timing()
     ap = build_parser()
     try:
         args = ap.parse_args(argv)
@@ -187,6 +214,7 @@ def _run(argv: list, loaded: dict) -> int:
     except (ConfigError, OSError, json.JSONDecodeError) as e:
         print(f"tuff: {e}", file=sys.stderr)
         return 1
+    tm.mark("config", sync=False)
     if args.inspect:
         _inspect(cfg, build_model(cfg))
         return 0
@@ -247,6 +275,7 @@ def _run(argv: list, loaded: dict) -> int:
                 eng = Engine.from_folder(args.model, **kw)
             loaded.update(key=key, engine=eng)
             print(f"tuff: model ready in {time.time() - t0:.2f} s", file=sys.stderr)
+        tm.mark("model_load")
     except Exception as e:                                   # noqa: BLE001 - reported, then exit code
         print(f"tuff: {type(e).__name__}: {e}", file=sys.stderr)
         return 1 if type(e).__name__ in ("WeightsError", "ConfigError") else 3
@@ -261,20 +290,23 @@ def _run(argv: list, loaded: dict) -> int:
 
     try:
         if args.teacher_force or args.dump_logits:
-            return _teacher_force(args, eng, ids, n_predict, chunk)
+            rc = _teacher_force(args, eng, ids, n_predict, chunk)
+            tm.mark("teacher_force")
+            return rc
         if args.dump_tokens:
             out = llm.generate([ids], params)[0]
+            tm.mark("generate")
             for t in out.token_ids:
                 print(t)
             print(f"tuff: {len(out.token_ids)} tokens, finish: {out.finish_reason}", file=sys.stderr)
             return 0
-        return _timed(args, llm, ids, params)
+        return _timed(args, llm, ids, params, tm)
     except Exception as e:                                   # noqa: BLE001
         print(f"tuff: {type(e).__name__}: {e}", file=sys.stderr)
         return 3
 
 
-def _timed(args, llm, ids, params) -> int:
+def _timed(args, llm, ids, params, tm) -> int:
     """Warm-up then timed decode, mean +- (max - min)/2 over runs (src/main.c:1720-1726, :1891-1904)."""
     import dataclasses
     import torch
@@ -287,19 +319,22 @@ def _timed(args, llm, ids, params) -> int:
         sched.add(req)
         marks = {}
 
-        def on_step(batch, sampled, req=req, marks=marks):
+        def on_step(batch, sampled, req=req, marks=marks, run=run):
             n = len(req.output)
             if n >= 1 and "prefill" not in marks:
                 torch.cuda.synchronize()
                 marks["prefill"] = time.perf_counter()
+                tm.mark(f"run {run}: prefill", sync=False)
             if n >= args.warmup + 1 and "t0" not in marks:
                 torch.cuda.synchronize()
                 marks["t0"] = time.perf_counter()
+                tm.mark(f"run {run}: warmup", sync=False)
         torch.cuda.synchronize()
         t_start = time.perf_counter()
         llm.run(sched, on_step)
         torch.cuda.synchronize()
         t1 = time.perf_counter()
+        tm.mark(f"run {run}: decode", sync=False)
         timed = len(req.output) - args.warmup - 1
         if timed > 0 and "t0" in marks:
             rates.append(timed / (t1 - marks["t0"]))
@@ -321,6 +356,7 @@ def _teacher_force(args, eng, ids, n_predict, chunk) -> int:
     The row after stream position q predicts reference step q - (n_prompt - 1) (:1379-1384).
     Without --teacher-force the model's own greedy tokens are fed and dumped."""
     import torch
+    from .csrc import ops
     from .engine.batch import StepEntry
     V = eng.model.vocab_size
     ref = _ids_from(args.teacher_force)[:n_predict] if args.teacher_force else None
@@ -344,7 +380,9 @@ def _teacher_force(args, eng, ids, n_predict, chunk) -> int:
         else:
             take, feed = 1, pending
         logits = eng.step([StepEntry("tf", feed, list(range(len(feed))))])
-        top = torch.argmax(logits, dim=-1).cpu().tolist()
+        picked = torch.empty(len(feed), dtype=torch.int32, device=logits.device)
+        ops.argmax(logits, picked)                         # ties go to the lowest id, as in generation
+        top = picked.cpu().tolist()
         if fout is not None:
             logits.cpu().numpy().astype("<f4").tofile(fout)
             rows_written += len(feed)

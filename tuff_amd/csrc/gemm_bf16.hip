@@ -842,7 +842,8 @@ SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16, bool emit = fals
         if (tiles16 <= 128) p.cols = 8;
         else if (tiles16 >= 4096) p.cols = 64;
         else if (tiles16 >= 512) p.cols = 32;
-        if (max_waves < 16 && p.cols > 16) p.cols = 16;                 // the norm inside keeps float32 rows in registers
+        if ((max_waves < 16 || emit) && p.cols > 16) p.cols = 16;       // the norm inside keeps float32 rows in registers;
+                                                                        // the emitting epilogue works on one tile
         p.tiles = ceil_div(N, p.cols);
         // enough waves in flight to cover the latency of HBM, at least one chunk a wave
         while (p.waves < max_waves && p.tiles * p.waves < 3072 && nchunks >= 2 * p.waves) p.waves *= 2;
@@ -901,7 +902,7 @@ struct Skinny16Extra {
 template <int MODE, int NORM, bool EMIT>
 int launch_skinny16(const void* X, const bf16_t* W, void* Y, int M, int N, int K, const Skinny16Extra& x, hipStream_t stream) {
     // the in-kernel norm needs more registers a wave: at most 8 waves a workgroup
-    const SkinnyPlan p = plan_skinny(M, N, K, NORM == NORM_INSIDE ? 8 : 16);
+    const SkinnyPlan p = plan_skinny(M, N, K, NORM == NORM_INSIDE ? 8 : 16, EMIT);
     dim3 grid(p.tiles);
     const size_t lds = NORM == NORM_INSIDE ? (size_t)K * sizeof(float) : 0;
 #define GO(NW, COLS) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<NW, MODE, NORM, EMIT, COLS>), grid, dim3(NW * WAVE), lds, stream, \
@@ -1028,7 +1029,7 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
 // *tiles tiles of columns, *rows rows each (16 for M <= 16, 64 for M <= 64).
 TUFF_EXPORT int tuff_gemm_bf16_emit_layout(int M, int N, int K, int* tiles, int* rows) {
     if (M > 64) return -2;
-    *tiles = plan_skinny(M, N, K).tiles;
+    *tiles = plan_skinny(M, N, K, 16, true).tiles;
     *rows = M <= 16 ? 16 : 64;
     return 0;
 }

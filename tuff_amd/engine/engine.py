@@ -153,10 +153,24 @@ class Engine:
                     self.manager.truncate(e.req_id, self.manager.length(e.req_id) - len(e.tokens))
                 raise
         self.steps += 1
+        try:
+            return self._run(entries, device_tokens)
+        except Exception:
+            # A launch that was refused.  The book-keeping goes back to before the step; paged entries are then
+            # as before (what was written lies beyond every request's length).  A fixed-size state of a layer
+            # that did run has moved on, so the caller should end the step's requests rather than go on with them.
+            for e in done:
+                self.manager.truncate(e.req_id, self.manager.length(e.req_id) - len(e.tokens))
+            raise
+
+    def _run(self, entries, device_tokens):
         if self.use_graphs and all(len(e.tokens) == 1 for e in entries):
             return self._decode_step(entries, device_tokens)
         ctx = build_context(entries, self.manager, self.device, self.model.vocab_size)
-        if self.record_portions and ctx.T >= self.SECTIONS_MIN_TOKENS and ctx.R <= self.manager.num_slots:
+        # Recorded in sections: steps with portions (a step of single tokens takes other kernels), keyed by
+        # everything their launches depend on outside of the sections that run eagerly.
+        if (self.record_portions and ctx.T >= self.SECTIONS_MIN_TOKENS and ctx.max_q_len > 1
+                and ctx.R <= self.manager.num_slots):
             return self._portion_step(ctx, device_tokens)
         self._place_device_tokens(ctx.tokens, device_tokens)
         return self.model.forward(ctx, self.storage.views)
@@ -193,12 +207,16 @@ class Engine:
 
     def _portion_step(self, ctx, device_tokens=None) -> Optional[torch.Tensor]:
         """A step with prompt portions.  What its kernels' launches depend on outside of the
-        sections that parts run eagerly (ctx.run_eagerly) is the number of tokens alone, so a
-        number of tokens that keeps coming (a scheduler fills its budget) is recorded once: graphs
+        sections that parts run eagerly (ctx.run_eagerly) is what the model's recording_key() names (the
+        number of tokens, and whether the last block prepares the head's norm), so a step shape that
+        keeps coming (a scheduler fills its budget) is recorded once: graphs
         of the stretches between those sections, replayed with the sections run in between."""
-        rec = self._sectioned.get(ctx.T)
+        key = self.model.recording_key(ctx)
+        rec = self._sectioned.get(key)
         if rec is None:
-            seen = self._sectioned_seen[ctx.T] = self._sectioned_seen.get(ctx.T, 0) + 1
+            if len(self._sectioned_seen) > 256 and key not in self._sectioned_seen:
+                self._sectioned_seen.clear()                # sizes that came once or twice and never again
+            seen = self._sectioned_seen[key] = self._sectioned_seen.get(key, 0) + 1
             if seen < self.SECTIONS_RECORD_AT:
                 self._place_device_tokens(ctx.tokens, device_tokens)
                 return self.model.forward(ctx, self.storage.views)
@@ -216,9 +234,9 @@ class Engine:
                 self._sectioned.clear()
                 self._place_device_tokens(ctx.tokens, device_tokens)
                 return self.model.forward(ctx, self.storage.views)
-            self._sectioned[ctx.T] = rec
+            self._sectioned[key] = rec
         else:
-            self._sectioned[ctx.T] = self._sectioned.pop(ctx.T)       # most recently used last
+            self._sectioned[key] = self._sectioned.pop(key)           # most recently used last
         merged = rec.refresh(ctx)
         self._place_device_tokens(merged.tokens, device_tokens)
         self.section_replays += 1
