@@ -403,6 +403,55 @@ def test_layers_of_full_size_bfloat16_against_float32(gpu):
     assert (outs["bfloat16"].argmax(-1) == outs["float32"].argmax(-1))[clear].all()
 
 
+def test_the_benchmarked_model(gpu):
+    """The model bench.py times (16 layers of the 1.2B shape, random weights of its seed): the float32
+    engine against the plain implementation in float64 on a prompt of 64 tokens, and the bfloat16 engine
+    against the float32 engine whole, with the last 32 tokens one by one, and mixed in portions beside
+    single tokens; the first choice agrees wherever float32 is not close to a tie."""
+    import bench
+    from plain.lfm2_plain import forward_logits
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.models.registry import build_model
+    from tuff_amd.weights.random_init import random_weights
+    cfg = bench.shape_config(bench.SHAPE["num_hidden_layers"])
+    assert cfg.num_hidden_layers == 16 and build_model(cfg).num_parameters() == 1170340608
+    V = cfg.vocab_size
+    reqs = {"a": util.rand_tokens(200, V, 61), "b": util.rand_tokens(64, V, 62), "c": util.rand_tokens(141, V, 63)}
+    plans = {"whole": util.plan_whole(reqs), "tail": util.plan_tail(reqs, 32),
+             "mixed": util.plan_mixed(reqs, seed=8, decode_tail=10)}
+    model = build_model(cfg)
+    weights = random_weights(model.weight_decls(), bench.SEED, torch.float32, gpu)
+    eng = Engine(model, weights, dtype="float32", page_size=16, max_tokens=1024, max_requests=4, poison_cache=True)
+    got32 = {k: util.run_plan(eng, p) for k, p in plans.items()}
+    for k in ("tail", "mixed"):
+        for rid in reqs:
+            assert torch.equal(got32[k][rid], got32["whole"][rid]), f"float32, {k}, {rid}: logits depend on the cutting"
+
+    class AsFloat64(dict):                      # one tensor at a time: the whole model in float64 would be 9 GB
+        def __getitem__(self, name):
+            return dict.__getitem__(self, name).double()
+
+        def __contains__(self, name):
+            return dict.__contains__(self, name)
+    raw = dict(cfg.to_dict(), layer_types=["conv" if cfg.is_conv(i) else "full_attention" for i in range(16)])
+    want = forward_logits(raw, AsFloat64({k: v.cpu() for k, v in weights.items()}), reqs["b"])
+    util.assert_close_f32_deep(got32["whole"]["b"], want, "benchmarked model, float32 against plain")
+    del eng, weights, model
+    torch.cuda.empty_cache()
+
+    eng16 = Engine.from_config(cfg, bench.SEED, dtype="bfloat16", page_size=16, max_tokens=1024, max_requests=4,
+                               poison_cache=True)
+    for k, plan in plans.items():
+        got16 = util.run_plan(eng16, plan)
+        for rid in reqs:
+            ref = got32["whole"][rid]
+            util.assert_close_bf16(got16[rid], ref, f"benchmarked model, bfloat16 {k} {rid}")
+            top = torch.topk(ref, 2, dim=-1).values
+            clear = (top[:, 0] - top[:, 1]) > 0.05 * float(ref.std())
+            assert clear.sum() > 0.5 * len(clear)
+            assert (got16[rid].argmax(-1) == ref.argmax(-1))[clear].all(), (k, rid)
+
+
 def random_configuration(seed: int) -> dict:
     """A small configuration whose every size and option is drawn from the seed."""
     import random

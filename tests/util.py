@@ -266,6 +266,19 @@ def assert_close_f32(got: torch.Tensor, want: torch.Tensor, what: str = ""):
                              f"(got {got[tuple(first)]:.7f}, want {want[tuple(first)]:.7f}), max err {err.max():.3e}")
 
 
+def assert_close_f32_deep(got: torch.Tensor, want: torch.Tensor, what: str = "", rel: float = 2e-4):
+    """float32 against float64 for models far larger than the tiny ones: every product adds K = 2048 to 8192
+    terms in float32, one after the other (relative error about 2^-24 sqrt(K) = 5e-6 of the terms' size), and a
+    token passes ~7 such products in each of 16 layers, which adds up like a random walk to ~5e-5 of the logits'
+    spread.  The bound is four times that, on every element, relative to the spread (RMS) of the logits."""
+    got, want = got.double(), want.double()
+    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
+    assert torch.isfinite(got).all(), f"{what}: non-finite logits"
+    spread = float(want.pow(2).mean().sqrt())
+    err = float((got - want).abs().max()) / spread
+    assert err <= rel, f"{what}: largest error {err:.3e} of the logits' spread {spread:.3f} > {rel}"
+
+
 def rel_rms(got: torch.Tensor, want: torch.Tensor) -> float:
     got, want = got.double(), want.double()
     return float(((got - want).pow(2).mean() / want.pow(2).mean().clamp_min(1e-30)).sqrt())
