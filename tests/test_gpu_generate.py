@@ -255,8 +255,10 @@ def test_command_line(gpu, tmp_path):
     p6 = subprocess.run([sys.executable, os.path.join(util.ROOT, "bin", "tuff"), "--model", folder, "--prompt-ids", ids,
                          "-n", "4", "--warmup", "1", "--runs", "1"], capture_output=True, text=True, timeout=300, env=env)
     marks = [l for l in p6.stderr.splitlines() if l.startswith("[Tuff timing] ")]
-    assert p6.returncode == 0 and [m.split(": ")[0][14:] for m in marks] == \
-        ["config", "model_load", "run 0: prefill", "run 0: warmup", "run 0: decode"], p6.stderr
+    import re
+    phases = [re.fullmatch(r"\[Tuff timing\] (.*): [0-9.]+ s \(t=[0-9.]+\)", m).group(1) for m in marks]
+    assert p6.returncode == 0 and phases == ["config", "model_load", "run 0: prefill", "run 0: warmup", "run 0: decode"], \
+        p6.stderr
     ts = [float(m.split("(t=")[1].rstrip(")")) for m in marks]
     assert ts == sorted(ts) and all(" s (t=" in m for m in marks)
     assert _tuff("--model", folder).returncode == 2

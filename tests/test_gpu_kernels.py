@@ -484,6 +484,106 @@ def test_attention_mfma(gpu, H, Hkv, hd, ps, window):
         _check_step(case, reqs, got, H, hd, window, nb)
 
 
+def _decode_case(gpu, R, H, Hkv, ps, lens, seed=0, nan_pool=True):
+    """R requests with lens[r] tokens in the cache after this step; the step brings each one's last
+    token as a projected row [q heads | k heads | v heads] of heads of 64.  Pages shuffled."""
+    hd, dt = 64, torch.bfloat16
+    g = torch.Generator().manual_seed(seed)
+    n_blocks = [-(-n // ps) for n in lens]
+    n_pages = sum(n_blocks) + 2
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    fill = float("nan") if nan_pool else 0.0
+    kc = torch.full((n_pages, Hkv, ps, hd), fill, dtype=dt)
+    vc = torch.full((n_pages, Hkv, hd, ps), fill, dtype=dt)
+    table = torch.full((R, max(n_blocks) + 1), -1, dtype=torch.int32)
+    slots = []
+    for r, (n, nb_) in enumerate(zip(lens, n_blocks)):
+        pages = torch.tensor([perm.pop() for _ in range(nb_)])
+        table[r, :nb_] = pages.to(torch.int32)
+        t = torch.arange(n - 1)                                           # everything but the step's own token
+        kc[pages[t // ps], :, t % ps, :] = _r(n - 1, Hkv, hd, seed=seed + 10 + r, dtype=dt)
+        vc[pages[t // ps], :, :, t % ps] = _r(n - 1, Hkv, hd, seed=seed + 40 + r, dtype=dt)
+        slots.append(int(pages[(n - 1) // ps]) * ps + (n - 1) % ps)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
+    return dict(kc=kc.to(gpu), vc=vc.to(gpu), table=table.to(gpu), qkv=_r(R, (H + 2 * Hkv) * hd, seed=seed + 3, dtype=dt).to(gpu),
+                positions=i32([n - 1 for n in lens]), slots=i32(slots),
+                req_info=i32([[r, 1, n - 1, n] for r, n in enumerate(lens)]), max_ctx_len=max(lens))
+
+
+@pytest.mark.parametrize("H,Hkv,ps", [(32, 8, 16), (6, 3, 64), (16, 1, 32)])
+@pytest.mark.parametrize("window", [0, 300])
+@pytest.mark.parametrize("norm_dt", [torch.float32, torch.bfloat16, None])
+def test_attention_decode_fused_equals_the_separate_kernels(gpu, H, Hkv, ps, window, norm_dt):
+    """A step of single tokens from the projected rows in one kernel (norm, rotation, cache write,
+    attention) against the kernel that prepares q and writes the cache followed by the attention
+    kernel: the same cache and the same output, bit for bit; stale pages hold NaN."""
+    from tuff_amd.csrc import ops
+    hd, eps, base = 64, 1e-6, 1e6
+    lens = [700, 1, 257, 256, 33, 1025, 64]
+    R = len(lens)
+    qw = kw = None
+    if norm_dt is not None:
+        qw, kw = (1 + _r(hd, seed=5, scale=0.1)).to(norm_dt).to(gpu), (1 + _r(hd, seed=6, scale=0.1)).to(norm_dt).to(gpu)
+    inv_freq = (base ** (-2 * torch.arange(hd // 2, dtype=torch.float64) / hd)).float().to(gpu)
+    outs = []
+    angles = ops.rope_table(inv_freq, 600)                  # reaches some of the positions, not all
+    for fused in (False, True, "with a table of angles"):
+        c = _decode_case(gpu, R, H, Hkv, ps, lens)
+        out = torch.full((R, H * hd), float("nan"), dtype=torch.bfloat16, device=gpu)
+        common = dict(block_table=c["table"], req_info=c["req_info"], positions=c["positions"], H=H, Hkv=Hkv,
+                      page_size=ps, max_ctx_len=c["max_ctx_len"], window=window)
+        if fused:
+            ops.attention_decode_fused(c["qkv"], c["kc"], c["vc"], out, inv_freq=inv_freq, slot_mapping=c["slots"],
+                                       q_norm_w=qw, k_norm_w=kw, eps=eps, angles=angles if fused is not True else None,
+                                       **common)
+        else:
+            q = torch.empty(R, H * hd, dtype=torch.bfloat16, device=gpu)
+            ops.qkv_post(c["qkv"], q, H=H, Hkv=Hkv, hd=hd, positions=c["positions"], eps=eps, q_norm_w=qw, k_norm_w=kw,
+                         inv_freq=inv_freq, rotary_dim=hd, k_cache=c["kc"], v_cache=c["vc"], slot_mapping=c["slots"],
+                         page_size=ps)
+            ops.attention_mfma(q, c["kc"], c["vc"], out, blocks=None, nb=1, hd=hd, **common)
+        outs.append((out.float().cpu(), c["kc"].float().cpu(), c["vc"].float().cpu()))
+    (o0, k0, v0) = outs[0]
+    same = lambda a, b: torch.equal(torch.nan_to_num(a, nan=12345.0), torch.nan_to_num(b, nan=12345.0))
+    for (o1, k1, v1) in outs[1:]:
+        assert torch.isfinite(o1).all()
+        assert same(k0, k1) and same(v0, v1), "the two ways write different keys or values"
+        assert torch.equal(o0, o1)
+    # reading only: nothing is written, the token's own key is then not in the cache (NaN there would show)
+    c = _decode_case(gpu, R, H, Hkv, ps, [n + 1 for n in lens], nan_pool=False)
+    before = (c["kc"].clone(), c["vc"].clone())
+    out = torch.empty((R, H * hd), dtype=torch.bfloat16, device=gpu)
+    ops.attention_decode_fused(c["qkv"], c["kc"], c["vc"], out, inv_freq=inv_freq, slot_mapping=None, q_norm_w=qw, k_norm_w=kw,
+                               eps=eps, block_table=c["table"], req_info=c["req_info"], positions=c["positions"], H=H, Hkv=Hkv,
+                               page_size=ps, max_ctx_len=c["max_ctx_len"], window=window)
+    assert torch.equal(before[0], c["kc"]) and torch.equal(before[1], c["vc"])
+
+
+def test_attention_of_single_tokens_is_the_same_with_one_wave_or_four_a_partition(gpu):
+    """Few requests: four waves share a partition of 256 keys; many: one wave walks it.  A request's
+    result is the same bit for bit in either company."""
+    from tuff_amd.csrc import ops
+    H, Hkv, hd, ps = 32, 8, 64, 16
+    lens = [2100, 37, 513] + [1800 + 7 * i for i in range(29)]           # 32 requests, 9 partitions: 2304 workgroups
+    inv_freq = (1e6 ** (-2 * torch.arange(hd // 2, dtype=torch.float64) / hd)).float().to(gpu)
+    qw = (1 + _r(hd, seed=5, scale=0.1)).to(gpu)
+
+    def run(n_req, fused):
+        c = _decode_case(gpu, len(lens), H, Hkv, ps, lens, nan_pool=False)
+        sub = dict(block_table=c["table"][:n_req].contiguous(), req_info=c["req_info"][:n_req].contiguous(),
+                   positions=c["positions"][:n_req].contiguous(), H=H, Hkv=Hkv, page_size=ps, max_ctx_len=c["max_ctx_len"])
+        out = torch.empty((n_req, H * hd), dtype=torch.bfloat16, device=gpu)
+        if fused:
+            ops.attention_decode_fused(c["qkv"][:n_req].contiguous(), c["kc"], c["vc"], out, inv_freq=inv_freq,
+                                       slot_mapping=c["slots"][:n_req].contiguous(), q_norm_w=qw, k_norm_w=qw, eps=1e-5, **sub)
+        else:
+            ops.attention_mfma(c["qkv"][:n_req, :H * hd].contiguous(), c["kc"], c["vc"], out, blocks=None, nb=1, hd=hd, **sub)
+        return out.float().cpu()
+    for fused in (False, True):
+        few, many = run(3, fused), run(len(lens), fused)
+        assert torch.isfinite(many).all() and torch.equal(few, many[:3]), f"fused={fused}"
+
+
 @pytest.mark.parametrize("H,Hkv,hd,ps", [(4, 2, 16, 16), (4, 1, 24, 16), (3, 3, 80, 16), (2, 1, 256, 32),
                                           (32, 8, 64, 16), (8, 2, 128, 64), (32, 1, 64, 16), (5, 5, 40, 48),
                                           (6, 2, 96, 80)])

@@ -2,11 +2,13 @@
 // tokens alike.
 //
 // Work is cut the same way whatever the batch: the keys of a request are split into partitions
-// of 256 positions (0..255, 256..511, ...).  One wave takes one partition, one kv head and one
-// block of query columns (a column = one query head of one token; all columns of a block share
-// the request and the kv head).  It produces, per column, the running maximum m, the sum l and
-// the unnormalised output o of that partition, in float32.  A second kernel merges a token's
-// partitions in ascending order.  Since the columns of a matrix product do not influence each
+// of 256 positions (0..255, 256..511, ...), each of four units of 64.  A workgroup takes one
+// partition, one kv head and one block of query columns (a column = one query head of one token;
+// all columns of a block share the request and the kv head): one wave that walks the four units, or,
+// where that would leave the chip idle, four waves with a unit each.  Either way a unit starts from
+// a fresh state and the units' results (running maximum m, sum l, unnormalised output o, float32)
+// are merged in ascending order through one chain of operations, so both give the same bits.  A
+// second kernel merges a token's partitions in ascending order.  Since the columns of a matrix product do not influence each
 // other, a token's result does not depend on how the sequence was cut into steps or on what
 // else was in the batch.
 //
@@ -35,17 +37,71 @@ __device__ __forceinline__ f32x4 mfma32(bf16x8 a, bf16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
-template <int HDP, int NB>
-__global__ __launch_bounds__(WAVE) void attn_partition_kernel(
-    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+// What the kernel does itself, for heads of 64 channels, when it is handed the projected rows
+// [q heads | k heads | v heads] of a step of single tokens instead of finished queries: the per-head
+// RMSNorm of q and k, the half-split rotation, and the write of the token's key and value into the
+// cache (by the workgroup whose partition holds the token's position, before it reads its keys).
+// The arithmetic is that of the kernel that does this for prompt portions (qkv_post64_kernel), sum
+// for sum, so a key in the cache does not tell which of the two wrote it.
+struct FusedQKV {
+    const void* q_norm_w = nullptr;        // [64] each, float32 or bfloat16 (norm_dt); null: no norm
+    const void* k_norm_w = nullptr;
+    int norm_dt = DT_F32;
+    float eps = 0.f;
+    const float* inv_freq = nullptr;       // [32]
+    const float* angles = nullptr;         // [n_angles][2][32]: cosines and sines of pos * inv_freq, or null
+    int n_angles = 0;
+    const int* slot_mapping = nullptr;     // [tokens]; null: the cache is only read
+};
+
+// cosine and sine of pos * inv_freq[j]: from the table where it reaches, else computed (the same bits)
+__device__ __forceinline__ void angle(const FusedQKV& fq, int pos, int j, float& rc, float& rs) {
+    if (pos < fq.n_angles) {
+        rc = fq.angles[((long long)pos * 2) * 32 + j];
+        rs = fq.angles[((long long)pos * 2 + 1) * 32 + j];
+    } else {
+        const float a = (float)pos * fq.inv_freq[j];
+        rc = cosf(a);
+        rs = sinf(a);
+    }
+}
+
+__device__ __forceinline__ float norm_weight(const void* w, int dt, int i) {
+    return dt == DT_F32 ? ((const float*)w)[i] : (float)((const bf16_t*)w)[i];
+}
+
+// One partial result (m, l, o) merged into a running one, element by element:
+//   m' = max(m, mu);  l' = l e^(m - m') + lu e^(mu - m');  o' likewise.
+// Both forms of the kernel (one wave or four a partition) merge a partition's four units of 64 keys
+// through this, in ascending order, so they give the same bits.
+__device__ __forceinline__ void merge_weights(float m, float mu, float& m_new, float& ca, float& cb) {
+    m_new = fmaxf(m, mu);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    ca = __expf(m - m_safe);               // 0 while nothing was seen
+    cb = __expf(mu - m_safe);
+}
+
+// a ca + b cb as one product and one fused multiply-add, spelled out: left to the compiler, two
+// instantiations of the kernel may fuse the other product and differ in the last bit
+__device__ __forceinline__ float merged(float a, float ca, float b, float cb) { return fmaf(b, cb, a * ca); }
+
+constexpr int UNIT = 64;                   // keys a unit: two steps of 32
+constexpr int UNITS = PART / UNIT;
+
+// NW: waves a workgroup (1: the wave walks the partition's four units; 4: a unit a wave, merged through LDS).
+template <int HDP, int NB, int NW, bool FUSED>
+__global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
     float* __restrict__ ws_o, float* __restrict__ ws_ml,
     const int* __restrict__ block_table, int max_blocks,
     const int2* __restrict__ blk, const int4* __restrict__ req_info,
-    int H, int Hkv, int hd, int page_size, int window, float scale, int n_parts) {
+    int H, int Hkv, int hd, int page_size, int window, float scale, int n_parts, FusedQKV fq) {
+    static_assert(NW == 1 || NW == UNITS, "one wave a partition or one a unit");
+    static_assert(!FUSED || (HDP == 64 && NB == 1), "the fused form is for heads of 64 and one column block");
     constexpr int KC = HDP / 32;          // 32-wide chunks of the head dimension
     constexpr int DB = HDP / 16;          // 16-wide blocks of output channels
     const int part = blockIdx.x, qb = blockIdx.y, kvh = blockIdx.z;
-    const int lane = threadIdx.x, n16 = lane % 16, g = lane / 16;
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n16 = lane % 16, g = lane / 16;
     const int G = H / Hkv;
     // Every load that depends on another costs a trip to memory, so the chain is kept short:
     // block -> request record (start, length, first position: a portion's positions are
@@ -67,35 +123,62 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
     if (key_begin > pos_max || key_begin + PART <= lo_min) return;
     const int key_end = min(key_begin + PART, pos_max + 1);
 
-    // this lane's columns
-    int pos_c[NB], lo_c[NB];
-    long long qrow[NB];                    // row of the column in q / in the work space; -1: no column
-    bf16x8 qf[NB][KC];
+    if constexpr (FUSED) {
+        // the token's key and value go into the cache before anybody reads the partition that holds them
+        if (fq.slot_mapping != nullptr && pos0 / PART == part) {
+            if (wave == 0) {
+                const long long slot = fq.slot_mapping[t0];
+                if (slot >= 0) {
+                    const long long page = slot / page_size, off = slot % page_size;
+                    const int row_width = (H + 2 * Hkv) * 64;
+                    const bf16_t* row = q + (long long)t0 * row_width;
+                    // value: lane = channel, as projected
+                    v_cache[((page * Hkv + kvh) * 64 + lane) * page_size + off] = row[(H + Hkv + kvh) * 64 + lane];
+                    // key: sixteen lanes hold four channels each (the other lanes do the same work again)
+                    const int l = lane % 16;
+                    const bf16x4 raw = *(const bf16x4*)(row + (H + kvh) * 64 + 4 * l);
+                    float v[4] = {(float)raw[0], (float)raw[1], (float)raw[2], (float)raw[3]};
+                    float ss = v[0] * v[0];
+                    ss = fmaf(v[1], v[1], ss);
+                    ss = fmaf(v[2], v[2], ss);
+                    ss = fmaf(v[3], v[3], ss);
+                    ss += __shfl_xor(ss, 8, WAVE);
+                    ss += __shfl_xor(ss, 4, WAVE);
+                    ss += __shfl_xor(ss, 2, WAVE);
+                    ss += __shfl_xor(ss, 1, WAVE);
+                    if (fq.k_norm_w != nullptr) {
+                        const float inv = 1.0f / sqrtf(ss / 64.0f + fq.eps);
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        const int c = col0 + nb * 16 + n16;
-        const bool valid = c < ncols;
-        const int tok = t0 + (valid ? c / G : 0);
-        const int head = kvh * G + (valid ? c % G : 0);
-        pos_c[nb] = valid ? pos0 + c / G : -1;
-        lo_c[nb] = (valid && window > 0) ? max(0, pos_c[nb] - window + 1) : 0;
-        qrow[nb] = valid ? (long long)tok * H + head : -1;
+                        for (int e = 0; e < 4; ++e) v[e] = v[e] * inv * norm_weight(fq.k_norm_w, fq.norm_dt, 4 * l + e);
+                    }
+                    const bool first = l < 8;
+                    bf16x4 o4;
 #pragma unroll
-        for (int kc = 0; kc < KC; ++kc) {
-            const int k = kc * 32 + g * 8;
-            bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-            qf[nb][kc] = (valid && k < hd) ? *(const bf16x8*)(q + qrow[nb] * hd + k) : z;
+                    for (int e = 0; e < 4; ++e) {
+                        float rc, rs;
+                        angle(fq, pos0, (4 * l + e) & 31, rc, rs);
+                        const float other = __shfl_xor(v[e], 8, WAVE);
+                        const float x0 = first ? v[e] : other, x1 = first ? other : v[e];
+                        o4[e] = (bf16_t)(first ? (x0 * rc - x1 * rs) : (x0 * rs + x1 * rc));
+                    }
+                    if (lane < 16) *(bf16x4*)(k_cache + ((page * Hkv + kvh) * page_size + off) * 64 + 4 * l) = o4;
+                }
+            }
+            __syncthreads();               // the stores have landed before a wave of this workgroup loads the keys
         }
     }
 
+    // the unit under way, and the partition's result so far
     float m_run[NB], l_run[NB];
     f32x4 o[DB][NB];
+    float m_acc[NB], l_acc[NB];
+    f32x4 o_acc[DB][NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-        m_run[nb] = -INFINITY;
-        l_run[nb] = 0.f;
+        m_acc[nb] = -INFINITY;
+        l_acc[nb] = 0.f;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) o[db][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int db = 0; db < DB; ++db) o_acc[db][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
     // One step covers 32 keys, two halves of 16 that each lie in one page.  The two S^T products
@@ -151,6 +234,77 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
             for (int db = 0; db < DB; ++db) t.vx[db] = v_frag(t, db);
         }
     };
+    // The first keys and values are asked for before the queries are prepared: they depend on the page
+    // numbers alone, and the queries' loads (and, in the fused form, their norm and rotation) then run
+    // while the keys are on their way.
+    Tile ta, tb;
+    const int key_first = NW == 1 ? key_begin : key_begin + wave * UNIT;
+    if constexpr (AHEAD) {
+        if (key_first < key_end) load_tile(key_first, ta);
+        if (NW > 1 && key_first + 32 < key_end) load_tile(key_first + 32, tb);
+    }
+
+    // this lane's columns
+    int pos_c[NB], lo_c[NB];
+    long long qrow[NB];                    // row of the column in the work space; -1: no column
+    bf16x8 qf[NB][KC];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int c = col0 + nb * 16 + n16;
+        const bool valid = c < ncols;
+        const int tok = t0 + (valid ? c / G : 0);
+        const int head = kvh * G + (valid ? c % G : 0);
+        pos_c[nb] = valid ? pos0 + c / G : -1;
+        lo_c[nb] = (valid && window > 0) ? max(0, pos_c[nb] - window + 1) : 0;
+        qrow[nb] = valid ? (long long)tok * H + head : -1;
+        if constexpr (FUSED) {
+            // channels 8g .. 8g+7 and 32 + 8g .. 32 + 8g+7 of the head: partners of the rotation sit in one lane
+            const bf16_t* src = q + (long long)tok * ((H + 2 * Hkv) * 64) + head * 64 + g * 8;
+            bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+            const bf16x8 r0 = valid ? *(const bf16x8*)src : z, r1 = valid ? *(const bf16x8*)(src + 32) : z;
+            float v0[8], v1[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { v0[e] = (float)r0[e]; v1[e] = (float)r1[e]; }
+            // sums of squares of four channels each, then the butterfly of sixteen such sums in the order
+            // of the kernel for portions (partners 32, 16, 8 and 4 channels away)
+            float p[2][2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                float a = v0[4 * h] * v0[4 * h], b = v1[4 * h] * v1[4 * h];
+#pragma unroll
+                for (int e = 1; e < 4; ++e) { a = fmaf(v0[4 * h + e], v0[4 * h + e], a); b = fmaf(v1[4 * h + e], v1[4 * h + e], b); }
+                p[0][h] = a; p[1][h] = b;
+            }
+            float s0 = p[0][0] + p[1][0], s1 = p[0][1] + p[1][1];
+            s0 += __shfl_xor(s0, 32, WAVE); s1 += __shfl_xor(s1, 32, WAVE);
+            s0 += __shfl_xor(s0, 16, WAVE); s1 += __shfl_xor(s1, 16, WAVE);
+            const float ss = s0 + s1;
+            if (fq.q_norm_w != nullptr) {
+                const float inv = 1.0f / sqrtf(ss / 64.0f + fq.eps);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    v0[e] = v0[e] * inv * norm_weight(fq.q_norm_w, fq.norm_dt, g * 8 + e);
+                    v1[e] = v1[e] * inv * norm_weight(fq.q_norm_w, fq.norm_dt, 32 + g * 8 + e);
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float rc, rs;
+                angle(fq, max(pos_c[nb], 0), g * 8 + e, rc, rs);
+                const float x0 = v0[e], x1 = v1[e];
+                qf[nb][0][e] = (bf16_t)(x0 * rc - x1 * rs);
+                qf[nb][1][e] = (bf16_t)(x0 * rs + x1 * rc);
+            }
+        } else {
+#pragma unroll
+            for (int kc = 0; kc < KC; ++kc) {
+                const int k = kc * 32 + g * 8;
+                bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+                qf[nb][kc] = (valid && k < hd) ? *(const bf16x8*)(q + qrow[nb] * hd + k) : z;
+            }
+        }
+    }
+
     auto compute = [&](int key0, const Tile& t) {
         // ---- S^T = K Q^T, twice 16 keys
         f32x4 s[2][NB];
@@ -196,7 +350,7 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
                 sum += p;
                 pf[nb][i] = (bf16_t)p;
             }
-            l_run[nb] = l_run[nb] * corr[nb] + sum;
+            l_run[nb] = fmaf(l_run[nb], corr[nb], sum);
             m_run[nb] = m_new;
         }
         // ---- O^T = O^T * corr + V^T P^T
@@ -219,40 +373,113 @@ __global__ __launch_bounds__(WAVE) void attn_partition_kernel(
             }
         }
     };
+    auto begin_unit = [&]() {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            m_run[nb] = -INFINITY;
+            l_run[nb] = 0.f;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) o[db][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    // the unit's sum of a column is spread over the four lane groups until here
+    auto unit_sums = [&]() {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            l_run[nb] += __shfl_xor(l_run[nb], 16, WAVE);
+            l_run[nb] += __shfl_xor(l_run[nb], 32, WAVE);
+        }
+    };
 
-    if constexpr (AHEAD) {
-        Tile t0, t1;
-        load_tile(key_begin, t0);
-        for (int key0 = key_begin; key0 < key_end; key0 += 64) {
-            const bool more = key0 + 32 < key_end;
-            if (more) load_tile(key0 + 32, t1);
-            compute(key0, t0);
-            if (more) {
-                if (key0 + 64 < key_end) load_tile(key0 + 64, t0);
-                compute(key0 + 32, t1);
+    if constexpr (NW == 1) {
+        // units in ascending order, each from a fresh state, merged into the partition's result as they end
+        for (int key0 = key_begin; key0 < key_end; key0 += UNIT) {
+            begin_unit();
+            if constexpr (AHEAD) {
+                const bool more = key0 + 32 < key_end;
+                if (more) load_tile(key0 + 32, tb);
+                compute(key0, ta);
+                if (more) {
+                    if (key0 + UNIT < key_end) load_tile(key0 + UNIT, ta);
+                    compute(key0 + 32, tb);
+                }
+            } else {
+                for (int k2 = key0; k2 < min(key0 + UNIT, key_end); k2 += 32) {
+                    load_tile(k2, ta);
+                    compute(k2, ta);
+                }
+            }
+            unit_sums();
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                float m_new, ca, cb;
+                merge_weights(m_acc[nb], m_run[nb], m_new, ca, cb);
+                l_acc[nb] = merged(l_acc[nb], ca, l_run[nb], cb);
+                m_acc[nb] = m_new;
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o_acc[db][nb][e] = merged(o_acc[db][nb][e], ca, o[db][nb][e], cb);
             }
         }
     } else {
-        Tile t0;
-        for (int key0 = key_begin; key0 < key_end; key0 += 32) {
-            load_tile(key0, t0);
-            compute(key0, t0);
+        // a unit a wave; the waves' results go through LDS and every wave merges a share of the elements,
+        // each element through the same chain as above
+        __shared__ float u_ml[UNITS][NB][16][2];
+        __shared__ __attribute__((aligned(16))) float u_o[UNITS][NB][DB][WAVE][4];
+        const int key0 = key_begin + wave * UNIT;
+        begin_unit();
+        if (key0 < key_end) {
+            if constexpr (AHEAD) {
+                compute(key0, ta);
+                if (key0 + 32 < key_end) compute(key0 + 32, tb);
+            } else {
+                for (int k2 = key0; k2 < min(key0 + UNIT, key_end); k2 += 32) {
+                    load_tile(k2, ta);
+                    compute(k2, ta);
+                }
+            }
+        }
+        unit_sums();
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            if (g == 0) { u_ml[wave][nb][n16][0] = m_run[nb]; u_ml[wave][nb][n16][1] = l_run[nb]; }
+#pragma unroll
+            for (int db = 0; db < DB; ++db) *(f32x4*)u_o[wave][nb][db][lane] = o[db][nb];
+        }
+        __syncthreads();
+        // wave w finishes the channel blocks db = w, w + 4, ... of every column block
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+            for (int u = 0; u < UNITS; ++u) {
+                const float mu = u_ml[u][nb][n16][0], lu = u_ml[u][nb][n16][1];
+                float m_new, ca, cb;
+                merge_weights(m_acc[nb], mu, m_new, ca, cb);
+                l_acc[nb] = merged(l_acc[nb], ca, lu, cb);
+                m_acc[nb] = m_new;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    if (db % NW != wave) continue;
+                    const f32x4 ou = *(const f32x4*)u_o[u][nb][db][lane];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o_acc[db][nb][e] = merged(o_acc[db][nb][e], ca, ou[e], cb);
+                }
+            }
         }
     }
 
     // ---- the partition's result per column
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-        float l = l_run[nb];
-        l += __shfl_xor(l, 16, WAVE);
-        l += __shfl_xor(l, 32, WAVE);
         if (qrow[nb] < 0) continue;
         const long long slot = qrow[nb] * n_parts + part;
-        if (g == 0) { ws_ml[slot * 2] = m_run[nb]; ws_ml[slot * 2 + 1] = l; }
+        if (g == 0 && wave == 0) { ws_ml[slot * 2] = m_acc[nb]; ws_ml[slot * 2 + 1] = l_acc[nb]; }
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
+            if (NW > 1 && db % NW != wave) continue;
             const int dim = db * 16 + 4 * g;
-            if (dim < hd) *(f32x4*)(ws_o + slot * hd + dim) = o[db][nb];
+            if (dim < hd) *(f32x4*)(ws_o + slot * hd + dim) = o_acc[db][nb];
         }
     }
 }
@@ -372,12 +599,25 @@ __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restr
     }
 }
 
-template <int HDP, int NB>
-void launch_partition(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, float* ws_o,
+// Workgroups of four waves where one wave a partition would leave most of the chip idle (a step of a
+// few single tokens); the result is the same bit for bit.
+int few_waves = 2048;
+
+template <int HDP, int NB, bool FUSED>
+void launch_partition(dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* kc, bf16_t* vc, float* ws_o,
                       float* ws_ml, const int* bt, int max_blocks, const int2* blk, const int4* req_info,
-                      int H, int Hkv, int hd, int ps, int window, float scale, int n_parts) {
-    hipLaunchKernelGGL((attn_partition_kernel<HDP, NB>), grid, dim3(WAVE), 0, stream, q, kc, vc, ws_o, ws_ml, bt, max_blocks,
-                       blk, req_info, H, Hkv, hd, ps, window, scale, n_parts);
+                      int H, int Hkv, int hd, int ps, int window, float scale, int n_parts, const FusedQKV& fq) {
+    const long long waves = (long long)grid.x * grid.y * grid.z;
+    if constexpr (HDP * NB <= 128) {
+        // the fused form prepares its queries in every wave: four waves pay for that four times
+        if (waves < (FUSED ? few_waves / 2 : few_waves)) {
+            hipLaunchKernelGGL((attn_partition_kernel<HDP, NB, UNITS, FUSED>), grid, dim3(UNITS * WAVE), 0, stream, q, kc, vc, ws_o,
+                               ws_ml, bt, max_blocks, blk, req_info, H, Hkv, hd, ps, window, scale, n_parts, fq);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((attn_partition_kernel<HDP, NB, 1, FUSED>), grid, dim3(WAVE), 0, stream, q, kc, vc, ws_o, ws_ml, bt,
+                       max_blocks, blk, req_info, H, Hkv, hd, ps, window, scale, n_parts, fq);
 }
 }  // namespace
 
@@ -416,11 +656,11 @@ static int launch_attention(const void* q, const void* k_cache, const void* v_ca
     if (hd > 256 || hd % 8 != 0 || page_size % 16 != 0 || Hkv <= 0 || H % Hkv != 0 || n_parts < 1) return -2;
     if (Hkv > 65535 || n_qblocks > 65535 || n_parts > COMBINE_MAX_PARTS) return -2;
     const bf16_t* Q = (const bf16_t*)q;
-    const bf16_t* K = (const bf16_t*)k_cache;
-    const bf16_t* V = (const bf16_t*)v_cache;
+    bf16_t* K = (bf16_t*)k_cache;                                        // read only without the fused form
+    bf16_t* V = (bf16_t*)v_cache;
     dim3 grid(n_parts, n_qblocks, Hkv);
-#define GO(HDP, NB) launch_partition<HDP, NB>(grid, stream, Q, K, V, ws_o, ws_ml, block_table, max_blocks, (const int2*)blk, \
-                                              (const int4*)req_info, H, Hkv, hd, page_size, window, scale, n_parts)
+#define GO(HDP, NB) launch_partition<HDP, NB, false>(grid, stream, Q, K, V, ws_o, ws_ml, block_table, max_blocks, (const int2*)blk, \
+                                                     (const int4*)req_info, H, Hkv, hd, page_size, window, scale, n_parts, FusedQKV())
 #define BY_NB(HDP) do { if (nb == 1) GO(HDP, 1); else if (nb == 2) GO(HDP, 2); else if (nb == 4) GO(HDP, 4); else return -2; } while (0)
     if (hd <= 32) BY_NB(32);
     else if (hd <= 64) BY_NB(64);
@@ -435,6 +675,14 @@ static int launch_attention(const void* q, const void* k_cache, const void* v_ca
                         stream);
 }
 
+// Below how many workgroups a step's partitions get four waves each (0: never).  For measurements and
+// tests; the result of the attention does not depend on it.  Returns the value before.
+TUFF_EXPORT int tuff_attention_few_waves(int n) {
+    const int old = few_waves;
+    if (n >= 0) few_waves = n;
+    return old;
+}
+
 TUFF_EXPORT int tuff_attention_mfma(const void* q, const void* k_cache, const void* v_cache, void* out,
                                     float* ws_o, float* ws_ml, const int* block_table, int max_blocks,
                                     const int* blk, int n_qblocks, int nb, const int* req_info, const int* positions,
@@ -442,6 +690,36 @@ TUFF_EXPORT int tuff_attention_mfma(const void* q, const void* k_cache, const vo
                                     int n_parts, hipStream_t stream) {
     return launch_attention(q, k_cache, v_cache, out, ws_o, ws_ml, block_table, max_blocks, blk, n_qblocks, nb, req_info,
                             positions, n_tokens, H, Hkv, hd, page_size, window, scale, n_parts, stream);
+}
+
+// A step of single tokens (request r's token is row r) over heads of 64 channels, from the projected
+// rows qkv [n_tokens, (H + 2 Hkv) * 64]: per-head RMSNorm of q and k (weights [64] of type norm_dt, or
+// null), half-split rotation over the whole head by inv_freq [32] (angles [n_angles][2][32]: the
+// cosines and sines of the first n_angles positions as tuff_rope_table makes them, or null), the token's key and value written
+// to the cache at slot_mapping[r] (null: the cache is only read), attention, merge.  The query heads
+// of a kv head must fit one block of sixteen columns (H / Hkv <= 16).
+TUFF_EXPORT int tuff_attention_decode_fused(const void* qkv, void* k_cache, void* v_cache, void* out,
+                                            float* ws_o, float* ws_ml, const int* block_table, int max_blocks,
+                                            const int* req_info, const int* positions, const int* slot_mapping,
+                                            const void* q_norm_w, const void* k_norm_w, int norm_dt, float eps,
+                                            const float* inv_freq, const float* angles, int n_angles,
+                                            int n_tokens, int H, int Hkv, int page_size,
+                                            int window, float scale, int n_parts, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (page_size % 16 != 0 || Hkv <= 0 || H % Hkv != 0 || H / Hkv > 16 || n_parts < 1 || !inv_freq) return -2;
+    if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) return -2;
+    if (Hkv > 65535 || n_tokens > 65535 || n_parts > COMBINE_MAX_PARTS) return -2;
+    FusedQKV fq;
+    fq.q_norm_w = q_norm_w; fq.k_norm_w = k_norm_w; fq.norm_dt = norm_dt; fq.eps = eps;
+    fq.inv_freq = inv_freq; fq.slot_mapping = slot_mapping;
+    fq.angles = angles; fq.n_angles = angles ? n_angles : 0;
+    launch_partition<64, 1, true>(dim3(n_parts, n_tokens, Hkv), stream, (const bf16_t*)qkv, (bf16_t*)k_cache, (bf16_t*)v_cache,
+                                  ws_o, ws_ml, block_table, max_blocks, nullptr, (const int4*)req_info, H, Hkv, 64, page_size,
+                                  window, scale, n_parts, fq);
+    int rc = launch_status();
+    if (rc) return rc;
+    return launch_merge((const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, n_tokens, H, 64, window, n_parts, PART,
+                        stream);
 }
 
 // The merge alone, for partial results that another kernel left in the same layout (ws_o

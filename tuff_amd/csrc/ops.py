@@ -52,6 +52,7 @@ _SIGNATURES = {
                           _c_void_p, _c_void_p, _c_int, _c_float,
                           _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_rope_table": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p],
         "tuff_kv_write": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                           _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
@@ -66,6 +67,10 @@ _SIGNATURES = {
                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p],
         "tuff_attention_merge": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_void_p],
+        "tuff_attention_decode_fused": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                                        _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_float,
+                                        _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
+                                        _c_void_p],
         "tuff_attention_mfma_static": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                                        _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
                                        _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p],
@@ -440,6 +445,16 @@ def qkv_post(qkv, q_out, *, H, Hkv, hd, positions, eps=0.0, q_norm_w=None, k_nor
         positions.data_ptr(), p(slot_mapping), T, H, Hkv, hd, page_size, _stream()), "qkv_post")
 
 
+def rope_table(inv_freq: torch.Tensor, n_pos: int) -> torch.Tensor:
+    """float32 [n_pos, 2, len(inv_freq)]: cosines and sines of pos * inv_freq, bit for bit what the
+    rotation kernels compute for themselves."""
+    n_freq = inv_freq.shape[0]
+    _gpu("inv_freq", inv_freq, torch.float32, (n_freq,))
+    out = torch.empty(int(n_pos), 2, n_freq, dtype=torch.float32, device=inv_freq.device)
+    _check(load("rope_kv").tuff_rope_table(inv_freq.data_ptr(), n_freq, int(n_pos), out.data_ptr(), _stream()), "rope_table")
+    return out
+
+
 def kv_write(k, v, k_cache, v_cache, slot_mapping, *, Hkv, hd, page_size) -> None:
     T = k.shape[0]
     dt = k.dtype
@@ -529,6 +544,62 @@ def attention_mfma(q, k_cache, v_cache, out, *, block_table, blocks, nb, req_inf
         block_table.data_ptr(), block_table.shape[1], None if blocks is None else blocks.data_ptr(), nblk, nb,
         req_info.data_ptr(), positions.data_ptr(), T, H, Hkv, hd, page_size,
         int(window or 0), float(scale), n_parts, _stream()), "attention_mfma")
+
+
+def attention_decode_fused_supported(dtype, H: int, Hkv: int, hd: int, page_size: int, rotary_dim: int, interleaved: bool) -> bool:
+    """A step of single tokens can go from the projected q/k/v rows to the attention output in one
+    kernel and its merge: bfloat16, heads of 64 rotated whole in half-split pairs, at most sixteen
+    query heads a kv head."""
+    return (dtype == torch.bfloat16 and hd == 64 and rotary_dim == 64 and not interleaved and page_size % 16 == 0
+            and H % Hkv == 0 and H // Hkv <= 16)
+
+
+def attention_decode_fused(qkv, k_cache, v_cache, out, *, block_table, req_info, positions, inv_freq, H, Hkv, page_size,
+                           max_ctx_len, slot_mapping=None, q_norm_w=None, k_norm_w=None, eps=0.0, window=0, scale=None,
+                           angles=None) -> None:
+    """Attention of a step in which every request has one token (row r of qkv is request r's), from the
+    projected rows qkv [R, (H + 2 Hkv) * 64]: QK-norm, rotation, the write of the new key and value
+    into the cache (slot_mapping; None: the cache is only read), attention over the cache, merge.
+    angles: rope_table(inv_freq, n) or None; positions below n take their cosines and sines from it
+    (computing them costs the kernel more than everything else it does for a short context)."""
+    R = qkv.shape[0]
+    hd = 64
+    _gpu("qkv", qkv, torch.bfloat16, (R, (H + 2 * Hkv) * hd))
+    _gpu("out", out, torch.bfloat16, (R, H * hd))
+    P = k_cache.shape[0]
+    _gpu("k_cache", k_cache, torch.bfloat16, (P, Hkv, page_size, hd))
+    _gpu("v_cache", v_cache, torch.bfloat16, (P, Hkv, hd, page_size))
+    _gpu("block_table", block_table, torch.int32)
+    _gpu("req_info", req_info, torch.int32, (R, 4))
+    _gpu("positions", positions, torch.int32, (R,))
+    _opt("slot_mapping", slot_mapping, torch.int32, (R,))
+    _gpu("inv_freq", inv_freq, torch.float32, (hd // 2,))
+    _opt("angles", angles, torch.float32, (None, 2, hd // 2))
+    if block_table.dim() != 2 or block_table.shape[0] != R:
+        raise KernelError("attention_decode_fused: block_table must be [requests, blocks]")
+    if block_table.shape[1] * page_size < int(max_ctx_len):
+        raise KernelError("attention_decode_fused: block_table is narrower than the longest context")
+    if not attention_decode_fused_supported(qkv.dtype, H, Hkv, hd, page_size, hd, False):
+        raise KernelError(f"attention_decode_fused: heads {H}:{Hkv} / page size {page_size} not supported")
+    norm_dt = DT_F32
+    if q_norm_w is not None or k_norm_w is not None:
+        if q_norm_w is None or k_norm_w is None or q_norm_w.dtype != k_norm_w.dtype:
+            raise KernelError("attention_decode_fused: q and k norm weights go together and share a dtype")
+        _gpu("q_norm_w", q_norm_w, shape=(hd,))
+        _gpu("k_norm_w", k_norm_w, shape=(hd,))
+        norm_dt = _dt(q_norm_w)
+    n_parts = max(1, -(-int(max_ctx_len) // ATTN_PARTITION))
+    if scale is None:
+        scale = 1.0 / math.sqrt(hd)
+    ws_o = torch.empty(R * H * n_parts * hd, dtype=torch.float32, device=qkv.device)
+    ws_ml = torch.empty(R * H * n_parts * 2, dtype=torch.float32, device=qkv.device)
+    p = lambda t: None if t is None else t.data_ptr()
+    _check(load("attention_mfma").tuff_attention_decode_fused(
+        qkv.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), ws_o.data_ptr(), ws_ml.data_ptr(),
+        block_table.data_ptr(), block_table.shape[1], req_info.data_ptr(), positions.data_ptr(), p(slot_mapping),
+        p(q_norm_w), p(k_norm_w), norm_dt, float(eps), inv_freq.data_ptr(), p(angles),
+        0 if angles is None else angles.shape[0], R, H, Hkv, page_size,
+        int(window or 0), float(scale), n_parts, _stream()), "attention_decode_fused")
 
 
 def attention_prefill_block_columns(hd: int) -> int:

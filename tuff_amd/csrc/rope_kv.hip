@@ -259,6 +259,19 @@ __global__ __launch_bounds__(256) void qkv_post64_kernel(
     }
 }
 
+// Cosines and sines of pos * inv_freq[j] for pos = 0 .. n_pos - 1, as the kernels above compute them
+// (the same float32 product and the same cosf and sinf): out [n_pos][2][n_freq], cosines then sines.
+// A kernel that takes its angles from this table gives the bits of one that computes them.
+__global__ void rope_table_kernel(const float* __restrict__ inv_freq, int n_freq, int n_pos, float* __restrict__ out) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (long long)n_pos * n_freq) return;
+    const int p = (int)(i / n_freq), j = (int)(i % n_freq);
+    const float pos = (float)p;
+    const float a = pos * inv_freq[j];
+    out[((long long)p * 2) * n_freq + j] = cosf(a);
+    out[((long long)p * 2 + 1) * n_freq + j] = sinf(a);
+}
+
 // Copies already encoded k and v rows [T, Hkv, hd] into the paged cache.
 template <typename T>
 __global__ __launch_bounds__(WAVE) void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v,
@@ -329,5 +342,12 @@ TUFF_EXPORT int tuff_kv_write(const void* k, const void* v, void* k_cache, void*
     dim3 grid(n_tokens, Hkv), block(WAVE);
     if (dt == DT_F32) hipLaunchKernelGGL(kv_write_kernel<float>, grid, block, 0, stream, (const float*)k, (const float*)v, (float*)k_cache, (float*)v_cache, slot_mapping, Hkv, hd, page_size);
     else hipLaunchKernelGGL(kv_write_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)k, (const bf16_t*)v, (bf16_t*)k_cache, (bf16_t*)v_cache, slot_mapping, Hkv, hd, page_size);
+    return launch_status();
+}
+
+TUFF_EXPORT int tuff_rope_table(const float* inv_freq, int n_freq, int n_pos, float* out, hipStream_t stream) {
+    if (n_pos <= 0 || n_freq <= 0) return 0;
+    const long long n = (long long)n_pos * n_freq;
+    hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, stream, inv_freq, n_freq, n_pos, out);
     return launch_status();
 }

@@ -46,7 +46,8 @@ def build_lfm2(cfg: Lfm2Config) -> DecoderModel:
                 aliases={"q": (g + "attn_q.weight",), "k": (g + "attn_k.weight",),
                          "v": (g + "attn_v.weight",), "o": (g + "attn_output.weight",),
                          "q_norm": (g + "attn_q_norm.weight",), "k_norm": (g + "attn_k_norm.weight",)},
-                qk_norm_eps=eps, position=Rotary(cfg.head_dim, cfg.rope_theta))
+                qk_norm_eps=eps,
+                position=Rotary(cfg.head_dim, cfg.rope_theta, table_positions=min(cfg.max_position_embeddings, 1 << 18)))
         norm2 = RMSNorm(d, eps, p + "ffn_norm.weight", aliases=(g + "ffn_norm.weight",))
         ffn = SwiGLU(d, cfg.ffn_dim,
                      names={"gate": p + "feed_forward.w1.weight", "up": p + "feed_forward.w3.weight",

@@ -98,9 +98,22 @@ class AttentionMixer(Mixer):
         # a position encoding of its own: norm, then its apply(), then the cache write
         k = None if fused else self.rt.empty(T, Hkv * hd)
 
+        one_kernel = (fused and tables is not None and ctx.max_q_len == 1 and ops.attention_decode_fused_supported(
+            qkv.dtype, H, Hkv, hd, cache.page_size, tables[1], tables[2]))
+
         def over_the_cache(ctx):
             """What depends on where the step's tokens lie: positions, cache slots, block tables."""
             g = ctx.groups[cache.group]
+            if one_kernel:
+                # single tokens, heads of 64: norm, rotation, cache write and attention in one kernel
+                ops.attention_decode_fused(qkv, cache.k, cache.v, o, block_table=g.block_table, req_info=ctx.req_info,
+                                           positions=ctx.positions, inv_freq=tables[0], H=H, Hkv=Hkv,
+                                           page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len,
+                                           slot_mapping=g.slot_mapping if write_cache else None,
+                                           q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w, eps=self.eps or 0.0,
+                                           window=self.window or 0, scale=self.scale,
+                                           angles=getattr(self.position, "angle_table", lambda: None)())
+                return
             if fused:
                 rot = {}
                 if tables is not None:
