@@ -171,20 +171,28 @@ def run_checks(scratch: str, checks: list[str], control: dict | None, timeout: i
     return out
 
 
-def prebuild(quiet: bool = False) -> None:
-    """Compiles every mutant's kernels (on any machine with hipcc; no GPU needed)."""
+def prebuild(quiet: bool = False, jobs: int = 6) -> None:
+    """Compiles every mutant's kernels (on any machine with hipcc; no GPU needed), several at a time,
+    each worker in a scratch copy of its own."""
+    import threading
+    from concurrent.futures import ThreadPoolExecutor
+    todo = [c for c in read_table() if module_of(c) is not None]
     with tempfile.TemporaryDirectory(prefix="tuff_amd_negctl_") as tmp:
-        scratch = make_scratch(os.path.join(tmp, "tree"))
-        for c in read_table():
-            if module_of(c) is None:
-                continue
-            apply(c, scratch)
+        local = threading.local()
+
+        def build_one(c):
+            if not hasattr(local, "tree"):
+                local.tree = make_scratch(os.path.join(tmp, f"tree_{threading.get_ident()}"))
+            apply(c, local.tree)
             try:
-                compile_mutant(c, scratch)
+                compile_mutant(c, local.tree)
             finally:
-                revert(c, scratch)
+                revert(c, local.tree)
             if not quiet:
                 print(f"[negative controls] {c['id']}: built", file=sys.stderr, flush=True)
+
+        with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo)))) as ex:
+            list(ex.map(build_one, todo))
 
 
 def main(argv) -> int:

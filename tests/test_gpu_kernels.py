@@ -889,6 +889,60 @@ def test_shortconv_long_portions_equal_single_tokens(gpu, d, K):
     assert torch.equal(s1, s2)
 
 
+@pytest.mark.parametrize("M,d,K,taps", [(1, 64, 64, 3), (8, 2048, 2048, 3), (16, 240, 328, 4), (5, 48, 96, 2), (3, 96, 8192, 7)])
+@pytest.mark.parametrize("norm", ["none", "inside", "scaled"])
+def test_gemm_with_the_convolution_in_its_epilogue(gpu, M, d, K, taps, norm):
+    """Input projection and gated short convolution of single tokens in one kernel, against the plain
+    formulas on the same bfloat16 inputs: out = C * conv(B * X) over each row's state, and the state
+    shifted by u = B * X.  With the norm inside the product and with the row scales another product left."""
+    from tuff_amd.csrc import ops
+    eps = 1e-5
+    w_in = _r(3 * d, K, seed=1, scale=K ** -0.5, dtype=torch.bfloat16)
+    conv_w = _r(d, taps, seed=2, scale=0.5, dtype=torch.bfloat16)
+    slots = torch.randperm(M + 3, generator=torch.Generator().manual_seed(3))[:M].to(torch.int32)
+    state0 = _r(M + 3, taps - 1, d, seed=4)
+    x32 = _r(M, K, seed=5)
+    nw = 1 + _r(K, seed=6, scale=0.1)
+    w = ops.tile_weight(ops.conv_group_rows(w_in.to(gpu)))
+    state = state0.clone().to(gpu)
+    out = torch.full((M, d), float("nan"), dtype=torch.bfloat16, device=gpu)
+    kw = dict(conv_w=conv_w.to(gpu), state=state, state_slot=slots.to(gpu))
+    if norm == "none":
+        h = x32.to(torch.bfloat16)
+        ops.gemm_conv(h.to(gpu), w, out, **kw)
+        h = h.double()
+    elif norm == "inside":
+        ops.gemm_conv(x32.to(gpu), w, out, norm_w=nw.to(gpu), eps=eps, **kw)
+        h = (x32 * nw).to(torch.bfloat16).double() / torch.sqrt((x32.double() ** 2).mean(-1, keepdim=True) + eps)
+    else:
+        xw = (x32 * nw).to(torch.bfloat16)
+        tiles = 5
+        ss = torch.zeros(tiles, 16)
+        cut = [K * t // tiles for t in range(tiles + 1)]
+        for t in range(tiles):
+            ss[t, :M] = (x32[:, cut[t]:cut[t + 1]] ** 2).sum(-1)
+        ops.gemm_conv(xw.to(gpu), w, out, ss=ss.to(gpu), eps=eps, **kw)
+        h = xw.double() / torch.sqrt((x32.double() ** 2).mean(-1, keepdim=True) + eps)
+    bcx = (h @ w_in.double().T).to(torch.bfloat16).double()
+    B, C, X = bcx[:, :d], bcx[:, d:2 * d], bcx[:, 2 * d:]
+    u = B * X
+    st = state0[slots.long()].double()                                   # [M, taps - 1, d]
+    y = (st * conv_w.double().T[:taps - 1][None]).sum(1) + u * conv_w.double()[:, taps - 1]
+    want = C * y
+    got = out.cpu().double()
+    assert torch.isfinite(got).all()
+    assert (got - want).abs().max() <= 2 ** -6 * float(want.abs().max()), (got - want).abs().max()
+    new_state = state.cpu().double()
+    want_state = torch.cat([st[:, 1:], u[:, None]], dim=1)
+    assert (new_state[slots.long()] - want_state).abs().max() <= 2 ** -6 * float(want_state.abs().max())
+    others = torch.ones(M + 3, dtype=torch.bool)
+    others[slots.long()] = False
+    assert torch.equal(new_state[others], state0[others].double())      # nobody else's state was touched
+    with pytest.raises(ops.KernelError, match="at most 16 rows"):
+        ops.gemm_conv(torch.zeros(17, K, dtype=torch.bfloat16, device=gpu), w, torch.empty(17, d, dtype=torch.bfloat16, device=gpu),
+                      conv_w=conv_w.to(gpu), state=state, state_slot=torch.zeros(17, dtype=torch.int32, device=gpu))
+
+
 def test_shortconv_last_tap_is_the_current_token(gpu):
     from tuff_amd.csrc import ops
     d, K = 32, 3

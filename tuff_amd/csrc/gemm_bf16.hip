@@ -27,7 +27,11 @@
 
 // OUT_SWIGLU: the rows of W are gate and up rows interleaved (2f: gate f, 2f+1: up f); the
 // output is bfloat16 [M, N/2] with y[m, f] = silu(g) * u, silu(g) = g / (1 + exp(-g)).
-enum : int { OUT_BF16 = 0, OUT_F32 = 1, OUT_F32_ACCUM = 2, OUT_SWIGLU = 3 };
+// OUT_CONV (at most 16 rows, one token a row): W is the input projection of a gated short convolution
+// with its rows regrouped, sixteen channels a group, as [B of the group | C of the group | X of the
+// group]; the epilogue forms u = B * X, runs the convolution over the row's state, writes
+// bfloat16 C * y [M, N/3] and shifts u into the state.  No projected row ever reaches memory.
+enum : int { OUT_BF16 = 0, OUT_F32 = 1, OUT_F32_ACCUM = 2, OUT_SWIGLU = 3, OUT_CONV = 4 };
 
 namespace {
 
@@ -441,6 +445,18 @@ constexpr int SK_CHUNK = 128;
 // NORM_SCALED product that follows.
 enum : int { NORM_NONE = 0, NORM_INSIDE = 1, NORM_SCALED = 2 };
 
+// What the OUT_CONV epilogue needs beside the product: the taps [d][taps] (float32 or bfloat16), the
+// float32 state [slots][taps - 1][d] and each row's slot.
+constexpr int CONV_MAX_TAPS = 16;
+struct ConvTail {
+    const void* taps_w = nullptr; int taps_dt = DT_F32; int taps = 0;
+    float* state = nullptr; const int* state_slot = nullptr;
+    __device__ __forceinline__ float tap(int ch, int k) const {
+        const long long i = (long long)ch * taps + k;
+        return taps_dt == DT_F32 ? ((const float*)taps_w)[i] : (float)((const bf16_t*)taps_w)[i];
+    }
+};
+
 template <int NW, int MODE, int NORM, bool EMIT, int COLS>
 __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const void* __restrict__ Xv, const bf16_t* __restrict__ W,
                                                                        void* __restrict__ Y, int M, int N, int K,
@@ -448,15 +464,19 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
                                                                        const int* __restrict__ rows,
                                                                        const float* __restrict__ ss_in, int n_ss,
                                                                        const float* __restrict__ emit_nw,
-                                                                       bf16_t* __restrict__ emit_xw, float* __restrict__ emit_ss) {
-    constexpr int TN = COLS > 16 ? COLS / 16 : 1;                        // MFMA tiles side by side: they share the rows of X
+                                                                       bf16_t* __restrict__ emit_xw, float* __restrict__ emit_ss,
+                                                                       ConvTail cv) {
+    constexpr bool CONV = MODE == OUT_CONV;
+    static_assert(!CONV || COLS == 8, "the convolution's epilogue takes eight channels a workgroup");
+    constexpr int TN = CONV ? 3 : (COLS > 16 ? COLS / 16 : 1);           // MFMA tiles side by side: they share the rows of X
     static_assert(!EMIT || TN == 1, "the emitting epilogue works on one tile");
     __shared__ float red[TN][NW][WAVE][4];
     __shared__ float ssq[16][16];                                        // [wave or part][row]
     extern __shared__ __attribute__((aligned(16))) float nw_lds[];       // NORM_INSIDE: the norm weight, K floats
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
     const int r16 = lane % 16, g = lane / 16;
-    const long long n0 = (long long)blockIdx.x * COLS;
+    // OUT_CONV: workgroup b takes the channels 8 b .. 8 b + 7: half (b % 2) of the three row tiles of group b / 2
+    const long long n0 = CONV ? (long long)(blockIdx.x / 2) * 48 + (blockIdx.x % 2) * 8 : (long long)blockIdx.x * COLS;
     const int nchunks = (K + SK_CHUNK - 1) / SK_CHUNK;
     const bf16_t* X = (const bf16_t*)Xv;
     const long long w_rows = min((long long)N, n0 + COLS);               // this tile's rows of W end here
@@ -591,6 +611,43 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
 #pragma unroll
             for (int w = 1; w < PARTS; ++w) total += ssq[w][row];
             scale = 1.0f / sqrtf(total / (float)K + eps);
+        }
+        if constexpr (CONV) {
+            // (row, channel): the three tiles hold B, C and X of the channel; the convolution as the kernel
+            // for single tokens does it, on the values rounded to bfloat16 as a projected row would hold them
+            float bcx[3];
+#pragma unroll
+            for (int tn = 0; tn < 3; ++tn) {
+                float v = red[tn][0][l][e];
+#pragma unroll
+                for (int w = 1; w < NW; ++w) v += red[tn][w][l][e];
+                if (NORM != NORM_NONE) v *= scale;
+                bcx[tn] = (float)(bf16_t)v;
+            }
+            const int row = (l / 16) * 4 + e, d = N / 3, Kc = cv.taps;
+            const int ch = (int)(blockIdx.x) * 8 + (l % 16);
+            if ((l % 16) < 8 && row < M && ch < d) {
+                float* st = cv.state + (long long)cv.state_slot[row] * (Kc - 1) * d;
+                float sv[CONV_MAX_TAPS], wv[CONV_MAX_TAPS];
+#pragma unroll
+                for (int k = 0; k < CONV_MAX_TAPS; ++k) {
+                    sv[k] = k < Kc - 1 ? st[(long long)k * d + ch] : 0.f;
+                    wv[k] = k < Kc - 1 ? cv.tap(ch, k) : 0.f;
+                }
+                const float w_last = cv.tap(ch, Kc - 1);
+                const float u = bcx[0] * bcx[2];
+                float y = 0.f;
+#pragma unroll
+                for (int k = 0; k < CONV_MAX_TAPS; ++k)
+                    if (k < Kc - 1) y = (k == 0) ? sv[k] * wv[k] : fmaf(sv[k], wv[k], y);
+                y = fmaf(u, w_last, y);
+#pragma unroll
+                for (int k = 1; k < CONV_MAX_TAPS; ++k)
+                    if (k < Kc - 1) st[(long long)(k - 1) * d + ch] = sv[k];
+                st[(long long)(Kc - 2) * d + ch] = u;
+                ((bf16_t*)Y)[(long long)row * d + ch] = (bf16_t)(bcx[1] * y);
+            }
+            return;
         }
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
@@ -897,23 +954,35 @@ struct Skinny16Extra {
     const float* norm_w = nullptr; float eps = 0.f; const int* rows = nullptr;       // NORM_INSIDE
     const float* ss_in = nullptr; int n_ss = 0;                                      // NORM_SCALED (+ eps)
     const float* emit_nw = nullptr; bf16_t* emit_xw = nullptr; float* emit_ss = nullptr;   // EMIT
+    ConvTail conv;                                                                   // OUT_CONV
 };
 
 template <int MODE, int NORM, bool EMIT>
 int launch_skinny16(const void* X, const bf16_t* W, void* Y, int M, int N, int K, const Skinny16Extra& x, hipStream_t stream) {
     // the in-kernel norm needs more registers a wave: at most 8 waves a workgroup
-    const SkinnyPlan p = plan_skinny(M, N, K, NORM == NORM_INSIDE ? 8 : 16, EMIT);
-    dim3 grid(p.tiles);
+    SkinnyPlan p = plan_skinny(M, N, K, NORM == NORM_INSIDE ? 8 : 16, EMIT);
     const size_t lds = NORM == NORM_INSIDE ? (size_t)K * sizeof(float) : 0;
 #define GO(NW, COLS) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<NW, MODE, NORM, EMIT, COLS>), grid, dim3(NW * WAVE), lds, stream, \
-                                        X, W, Y, M, N, K, x.norm_w, x.eps, x.rows, x.ss_in, x.n_ss, x.emit_nw, x.emit_xw, x.emit_ss)
-    if (p.cols == 16) { if (p.waves == 4) GO(4, 16); else if (p.waves == 8) GO(8, 16); else GO(16, 16); }
-    else if (p.cols == 8) { if (p.waves == 4) GO(4, 8); else if (p.waves == 8) GO(8, 8); else GO(16, 8); }
-    else if constexpr (!EMIT && NORM != NORM_INSIDE) {
-        if (p.cols == 32) { if (p.waves == 4) GO(4, 32); else if (p.waves == 8) GO(8, 32); else GO(16, 32); }
-        else if (p.cols == 64) { if (p.waves == 4) GO(4, 64); else if (p.waves == 8) GO(8, 64); else GO(16, 64); }
-        else return -3;
-    } else return -3;
+                                        X, W, Y, M, N, K, x.norm_w, x.eps, x.rows, x.ss_in, x.n_ss, x.emit_nw, x.emit_xw, x.emit_ss, \
+                                        x.conv)
+    if constexpr (MODE == OUT_CONV) {
+        // eight channels a workgroup (three half tiles); the waves split K as always, at most eight of them:
+        // sixteen would leave a wave 128 registers, too few for three tiles' operands of two chunks
+        const int nchunks = ceil_div(K, SK_CHUNK), groups = N / 3 / 8;
+        int waves = 4;
+        while (waves < 8 && groups * waves < 3072 && nchunks >= 2 * waves) waves *= 2;
+        dim3 grid(groups);
+        if (waves == 4) GO(4, 8); else GO(8, 8);
+    } else {
+        dim3 grid(p.tiles);
+        if (p.cols == 16) { if (p.waves == 4) GO(4, 16); else if (p.waves == 8) GO(8, 16); else GO(16, 16); }
+        else if (p.cols == 8) { if (p.waves == 4) GO(4, 8); else if (p.waves == 8) GO(8, 8); else GO(16, 8); }
+        else if constexpr (!EMIT && NORM != NORM_INSIDE) {
+            if (p.cols == 32) { if (p.waves == 4) GO(4, 32); else if (p.waves == 8) GO(8, 32); else GO(16, 32); }
+            else if (p.cols == 64) { if (p.waves == 4) GO(4, 64); else if (p.waves == 8) GO(8, 64); else GO(16, 64); }
+            else return -3;
+        } else return -3;
+    }
 #undef GO
     return launch_status();
 }
@@ -1105,4 +1174,34 @@ TUFF_EXPORT int tuff_gemm_bf16_scaled(const void* XW, const float* ss, int n_ss,
     FinishExtra x;
     x.ss_in = ss; x.n_ss = n_ss; x.eps = eps; x.K = K;
     return launch_skinny64_mode<NORM_SCALED>((const bf16_t*)XW, (const bf16_t*)W, Y, M, N, K, mode, ws, x, stream);
+}
+
+// For M <= 16 rows, one token a row: the input projection of a gated short convolution and the
+// convolution itself in one kernel.  W: the projection [3 d, K] with its rows regrouped (sixteen
+// channels a group: B, C, X of the group), tile-major; d must be a multiple of 16.  Y: bfloat16 [M, d]
+// = C * conv(B * X).  taps [d][n_taps] (taps_dt), state float32 [slots][n_taps - 1][d], state_slot [M].
+// norm_kind 0: X is bfloat16 [M, K];  1: X is the float32 residual stream and the RMSNorm (norm_w,
+// eps; K <= 8192) runs inside;  2: X is bf16(x * norm weight) and ss [n_ss][16] the sums of squares
+// that tuff_gemm_bf16_accum_emit left.
+TUFF_EXPORT int tuff_gemm_bf16_conv(const void* X, int norm_kind, const float* norm_w, float eps, const float* ss, int n_ss,
+                                    const void* W, void* Y, int M, int d, int K,
+                                    const void* taps, int taps_dt, int n_taps, float* state, const int* state_slot,
+                                    hipStream_t stream) {
+    if (M <= 0 || d <= 0) return 0;
+    if (K % 8 != 0 || M > 16 || d % 16 != 0 || n_taps < 2 || n_taps - 1 > CONV_MAX_TAPS) return -2;
+    Skinny16Extra x;
+    x.conv.taps_w = taps; x.conv.taps_dt = taps_dt; x.conv.taps = n_taps; x.conv.state = state; x.conv.state_slot = state_slot;
+    const bf16_t* w = (const bf16_t*)W;
+    if (norm_kind == 0) return launch_skinny16<OUT_CONV, NORM_NONE, false>(X, w, Y, M, 3 * d, K, x, stream);
+    if (norm_kind == 1) {
+        if (K > 8192) return -2;
+        x.norm_w = norm_w; x.eps = eps;
+        return launch_skinny16<OUT_CONV, NORM_INSIDE, false>(X, w, Y, M, 3 * d, K, x, stream);
+    }
+    if (norm_kind == 2) {
+        if (n_ss < 1) return -2;
+        x.ss_in = ss; x.n_ss = n_ss; x.eps = eps;
+        return launch_skinny16<OUT_CONV, NORM_SCALED, false>(X, w, Y, M, 3 * d, K, x, stream);
+    }
+    return -3;
 }

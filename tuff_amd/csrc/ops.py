@@ -44,6 +44,8 @@ _SIGNATURES = {
                                       _c_void_p, _c_void_p, _c_void_p],
         "tuff_gemm_bf16_scaled": [_c_void_p, _c_void_p, _c_int, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
                                   _c_int, _c_void_p, _c_void_p],
+        "tuff_gemm_bf16_conv": [_c_void_p, _c_int, _c_void_p, _c_float, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int,
+                                _c_int, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
         "tuff_gemm_bf16_normed": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
                                   _c_int, _c_void_p],
     },
@@ -387,6 +389,56 @@ def gemm_scaled(xw: torch.Tensor, ss: torch.Tensor, eps: float, w, out: torch.Te
     _check(load("gemm_bf16").tuff_gemm_bf16_scaled(xw.data_ptr(), ss.data_ptr(), ss.shape[0], float(eps), w.data_ptr(),
                                                    out.data_ptr(), M, N, K, mode,
                                                    None if ws is None else ws.data_ptr(), _stream()), "gemm_bf16_scaled")
+
+
+CONV_MAX_ROWS = 16                            # gemm_conv: one token a row
+
+
+def conv_group_rows(w_in: torch.Tensor) -> torch.Tensor:
+    """The input projection [3 d, K] of a gated short convolution (rows: B, then C, then X) with its
+    rows regrouped for gemm_conv: sixteen channels a group, each group as [its B rows | its C rows |
+    its X rows].  d must be a multiple of 16."""
+    three_d, K = w_in.shape
+    d = three_d // 3
+    if three_d != 3 * d or d % 16:
+        raise KernelError(f"conv_group_rows: [3 d, K] with d a multiple of 16 is needed, got {tuple(w_in.shape)}")
+    return w_in.view(3, d // 16, 16, K).permute(1, 0, 2, 3).reshape(three_d, K).contiguous()
+
+
+def gemm_conv(x: torch.Tensor, w, out: torch.Tensor, *, conv_w: torch.Tensor, state: torch.Tensor, state_slot: torch.Tensor,
+              norm_w: Optional[torch.Tensor] = None, eps: float = 0.0, ss: Optional[torch.Tensor] = None) -> None:
+    """Input projection and gated short convolution of single tokens (row r is request r's token, at
+    most 16 rows) in one kernel: out [M, d] bfloat16 = C * conv(B * X) with (B, C, X) = x @ w.T, and
+    the rows' states shifted.  w: conv_group_rows() of the projection, tiled.  x: bfloat16 [M, K]; or
+    the float32 residual stream with norm_w and eps (the RMSNorm runs inside); or bf16(x * norm weight)
+    with ss and eps as gemm_accum_emit leaves them."""
+    M, K = x.shape
+    d = out.shape[1]
+    taps = conv_w.shape[1]
+    _gpu("out", out, torch.bfloat16, (M, d))
+    w = _tiled(w, 3 * d, K)
+    _gpu("conv_w", conv_w, shape=(d, taps))
+    _gpu("state", state, torch.float32, (None, taps - 1, d))
+    _gpu("state_slot", state_slot, torch.int32, (M,))
+    if M > CONV_MAX_ROWS or K % 8 or d % 16 or not 2 <= taps <= 17:
+        raise KernelError(f"gemm_conv: at most {CONV_MAX_ROWS} rows, an inner size that is a multiple of 8, a width that is a "
+                          f"multiple of 16 and 2 to 17 taps; got {M} rows, inner size {K}, width {d}, {taps} taps")
+    kind, nw_ptr, ss_ptr, n_ss = 0, None, None, 0
+    if ss is not None:
+        _gpu("x", x, torch.bfloat16)
+        _gpu("ss", ss, torch.float32, (None, 16))
+        kind, ss_ptr, n_ss = 2, ss.data_ptr(), ss.shape[0]
+    elif norm_w is not None:
+        _gpu("x", x, torch.float32)
+        _gpu("norm_w", norm_w, torch.float32, (K,))
+        if K > NORMED_MAX_K:
+            raise KernelError(f"gemm_conv: the norm inside needs an inner size up to {NORMED_MAX_K}, got {K}")
+        kind, nw_ptr = 1, norm_w.data_ptr()
+    else:
+        _gpu("x", x, torch.bfloat16)
+    _check(load("gemm_bf16").tuff_gemm_bf16_conv(
+        x.data_ptr(), kind, nw_ptr, float(eps), ss_ptr, n_ss, w.data_ptr(), out.data_ptr(), M, d, K,
+        conv_w.data_ptr(), _dt(conv_w), taps, state.data_ptr(), state_slot.data_ptr(), _stream()), "gemm_bf16_conv")
 
 
 _plans: dict = {}

@@ -28,6 +28,7 @@ class Linear:
         self.aliases = [tuple(a) for a in aliases] if aliases else [()] * len(self.names)
         self.weight = None            # bound: ops.TiledWeight (bfloat16) or a float32 tensor [out, in]
         self.swiglu_pair = bool(swiglu_pair)
+        self.weight_grouped = None    # bound, for a conv's input projection: the weight with its rows regrouped
         if self.swiglu_pair and (len(self.names) != 2 or self.outs[0] != self.outs[1]):
             raise ValueError("a SwiGLU pair is two tensors of one shape")
         self.interleaved = False
@@ -54,6 +55,40 @@ class Linear:
                 raise ValueError(f"{self.names[0]}: the bfloat16 matrix kernels need an input size that is a "
                                  f"multiple of 8, got {self.in_features}")
             self.weight = ops.tile_weight(self.weight)       # the order the kernels stream it in
+
+    def group_rows_for_conv(self) -> bool:
+        """Call after bind(), for the input projection of a gated short convolution: keeps a second copy of
+        the weight with its rows regrouped, so that forward_conv() can run projection and convolution of
+        single tokens in one kernel.  False (and nothing kept) where the kernels cannot."""
+        w = self.weight
+        if not isinstance(w, ops.TiledWeight) or self.out_features % 48 or len(self.names) != 1:
+            return False
+        self.weight_grouped = ops.tile_weight(ops.conv_group_rows(w.rows()))
+        return True
+
+    def forward_conv(self, x, *, conv_w, state, state_slot) -> Optional[torch.Tensor]:
+        """x as for forward(), one token a row.  Returns C * conv(B * X) [T, out / 3] in bfloat16 with the
+        states shifted, or None where this needs the separate kernels (nothing is touched then)."""
+        from .norm import PendingNorm
+        if self.weight_grouped is None:
+            return None
+        pending = x if isinstance(x, PendingNorm) else None
+        T = pending.shape[0] if pending is not None else x.shape[0]
+        if T > ops.CONV_MAX_ROWS:
+            return None
+        kw = {}
+        if pending is not None:
+            if pending.pre is not None:
+                x, kw = pending.pre[0], dict(ss=pending.pre[1], eps=pending.norm.eps)
+            elif pending.rows is None and self.in_features <= ops.NORMED_MAX_K:
+                x, kw = pending.x, dict(norm_w=pending.norm.weight_f32, eps=pending.norm.eps)
+            else:
+                x = pending.tensor()
+        if not kw and x.dtype != torch.bfloat16:
+            return None
+        y = torch.empty(T, self.out_features // 3, dtype=torch.bfloat16, device=self.weight_grouped.device)
+        ops.gemm_conv(x, self.weight_grouped, y, conv_w=conv_w, state=state, state_slot=state_slot, **kw)
+        return y
 
     def forward(self, x, *, out_dtype: Optional[torch.dtype] = None,
                 accumulate_into: Optional[torch.Tensor] = None, swiglu: bool = False,

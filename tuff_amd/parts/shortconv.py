@@ -52,9 +52,16 @@ class ShortConvMixer(Mixer):
         self.in_proj.bind(weights, rt)
         self.out_proj.bind(weights, rt)
         self.conv_w = weights[self.names["conv"]].reshape(self.d, self.K).contiguous()
+        # bfloat16: projection and convolution of single tokens in one kernel, from a regrouped copy of the weight
+        self.in_proj.group_rows_for_conv()
 
     def forward(self, h, ctx, cache, residual, write_cache: bool = True, next_norm=None) -> None:
         T = h.shape[0]
+        if write_cache and ctx.max_q_len == 1:
+            y = self.in_proj.forward_conv(h, conv_w=self.conv_w, state=cache.state, state_slot=ctx.state_slot)
+            if y is not None:
+                self.out_proj.forward(y, accumulate_into=residual, next_norm=next_norm)
+                return
         bcx = self.in_proj.forward(h)
         y = self.rt.empty(T, self.d)
         if write_cache and ctx.max_q_len == 1:
