@@ -21,7 +21,8 @@
 //    second product (k = 8g + i), and the A operand V^T is one 16-byte load of eight consecutive
 //    positions of a channel from the transposed V page.
 //  * No LDS, no transposes, no barriers; K rows and V columns of the next step are loaded
-//    while the current step computes.
+//    while the current step computes, with streaming (non-temporal) loads: a step of single tokens
+//    reads every key once.
 //
 // Cache layout: K [page][kv_head][offset][hd], V [page][kv_head][hd][offset]; the page size
 // must be a multiple of 16 and the head size a multiple of 8 (the host falls back to the
@@ -205,7 +206,7 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
         const long long base = k_half ? t.base[1] : t.base[0];
         const int off0 = k_half ? t.off0[1] : t.off0[0];
         if (!live || k >= hd) return z;
-        return *(const bf16x8*)(k_cache + base + (long long)(off0 + k_off + 4 * kb) * hd + k);
+        return __builtin_nontemporal_load((const bf16x8*)(k_cache + base + (long long)(off0 + k_off + 4 * kb) * hd + k));
     };
     auto v_frag = [&](const Tile& t, int db) {
         const int dim = db * 16 + n16;
@@ -214,7 +215,7 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
         const long long base = (g / 2) ? t.base[1] : t.base[0];
         const int off0 = (g / 2) ? t.off0[1] : t.off0[0];
         if (!live || dim >= hd) return z;
-        return *(const bf16x8*)(v_cache + base + (long long)dim * page_size + off0 + (g % 2) * 8);
+        return __builtin_nontemporal_load((const bf16x8*)(v_cache + base + (long long)dim * page_size + off0 + (g % 2) * 8));
     };
     auto load_tile = [&](int key0, Tile& t) {
 #pragma unroll

@@ -67,8 +67,9 @@ __device__ __forceinline__ bf16x8 load8(const bf16_t* base, long long row, int n
 }
 
 // Piece `piece` (0..63) of block (tile, kblock) of a tile-major W with kb blocks a row tile.
+// Weights of a skinny product are read once and never again: a streaming (non-temporal) load.
 __device__ __forceinline__ bf16x8 load_w(const bf16_t* W, long long tile, int kb, int kblock, int piece) {
-    return *(const bf16x8*)(W + ((tile * kb + kblock) * 64 + piece) * 8);
+    return __builtin_nontemporal_load((const bf16x8*)(W + ((tile * kb + kblock) * 64 + piece) * 8));
 }
 
 // ------------------------------------------------------------------ tiled kernel
