@@ -114,9 +114,10 @@ def run_decode(llm, cfg, batch: int, ctx_end: int, steps: int, warmup: int, seed
     return marks["t1"] - marks["t0"], ctx_end - steps / 2.0
 
 
-def run_prefill(llm, cfg, tokens: int, repeats: int = 8):
+def run_prefill(llm, cfg, tokens: int, repeats: int = 8, warmup: int = 4):
     """One prompt of `tokens` tokens in one step, to the first generated token on the host.  Returns
-    the seconds of `repeats` runs (one more, the first, warms up and is left out)."""
+    the seconds of `repeats` runs after `warmup` untimed ones (the engine records a step size that keeps
+    coming when it comes for the third time; that one-off recording is not a prefill's time)."""
     import torch
     from tuff_amd.csrc import ops
     from tuff_amd.engine.batch import StepEntry
@@ -124,7 +125,7 @@ def run_prefill(llm, cfg, tokens: int, repeats: int = 8):
     g = torch.Generator().manual_seed(SEED + 1)
     times = []
     picked = torch.empty(1, dtype=torch.int32, device=eng.device)
-    for i in range(repeats + 1):
+    for i in range(repeats + warmup):
         prompt = torch.randint(0, cfg.vocab_size, (tokens,), generator=g).tolist()
         eng.begin(("prefill", i))
         torch.cuda.synchronize()
@@ -135,7 +136,7 @@ def run_prefill(llm, cfg, tokens: int, repeats: int = 8):
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         eng.end(("prefill", i))
-        if i > 0:
+        if i >= warmup:
             times.append(dt)
     return times
 

@@ -332,6 +332,33 @@ def test_qkv_post_heads_of_64(gpu, dt, ps):
         assert torch.equal(q, q2) and torch.equal(kc, k2) and torch.equal(vc, v2), f"steps of {step} differ"
 
 
+@pytest.mark.parametrize("H,Hkv,hd,rot,inter", [(6, 3, 64, 64, False), (4, 2, 80, 80, False), (3, 1, 48, 32, True), (2, 2, 128, 64, False)])
+def test_qkv_post_with_a_table_of_angles_gives_the_same_bits(gpu, H, Hkv, hd, rot, inter):
+    """Cosines and sines taken from rope_table() instead of computed in the kernel: the same queries and
+    the same cache, bit for bit, also for positions beyond the table's end."""
+    from tuff_amd.csrc import ops
+    T, ps, dt = 150, 16, torch.bfloat16
+    qkv = _r(T, (H + 2 * Hkv) * hd, seed=31, dtype=dt).to(gpu)
+    qw, kw = (1 + _r(hd, seed=32, scale=0.1)).to(gpu), (1 + _r(hd, seed=33, scale=0.1)).to(gpu)
+    pos = ((torch.arange(T, dtype=torch.int32) * 37) % 3000).to(gpu)
+    slots = torch.randperm(T + 10, generator=torch.Generator().manual_seed(4))[:T].to(torch.int32).to(gpu)
+    inv_freq = (1e6 ** (-2 * torch.arange(rot // 2, dtype=torch.float64) / rot)).float().to(gpu)
+    table = ops.rope_table(inv_freq, 2000)
+    assert table.shape == (2000, 2, rot // 2)
+    a = (torch.arange(2000, dtype=torch.float32, device=gpu)[:, None] * inv_freq[None]).double()
+    assert (table[:, 0].double() - torch.cos(a)).abs().max() < 1e-6 and (table[:, 1].double() - torch.sin(a)).abs().max() < 1e-6
+    outs = []
+    for angles in (None, table):
+        n_pages = (T + 10) // ps + 1
+        kc = torch.zeros(n_pages, Hkv, ps, hd, dtype=dt, device=gpu)
+        vc = torch.zeros(n_pages, Hkv, hd, ps, dtype=dt, device=gpu)
+        q = torch.empty(T, H * hd, dtype=dt, device=gpu)
+        ops.qkv_post(qkv, q, H=H, Hkv=Hkv, hd=hd, positions=pos, eps=1e-5, q_norm_w=qw, k_norm_w=kw, inv_freq=inv_freq,
+                     rotary_dim=rot, interleaved=inter, k_cache=kc, v_cache=vc, slot_mapping=slots, page_size=ps, angles=angles)
+        outs.append((q, kc, vc))
+    assert all(torch.equal(x, y) for x, y in zip(*outs))
+
+
 def test_qkv_post_many_tokens_equal_few(gpu):
     """With many tokens a wave takes several heads of a token in turn; the result is, bit for
     bit, that of the same tokens in small steps."""

@@ -923,6 +923,8 @@ SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16, bool emit = fals
 // Depends on the sizes only.
 struct TiledPlan { int shape, slices, steps_per_slice; long long ws_floats; };
 
+int tiled_shape_forced = -1;       // >= 0: every tiled product takes this shape (measurements only)
+
 TiledPlan plan_tiled(int M, int N, int K) {
     const long long large = (long long)ceil_div(N, 256) * ceil_div(M, 256);
     const long long small = (long long)ceil_div(N, 128) * ceil_div(M, 128);
@@ -930,6 +932,7 @@ TiledPlan plan_tiled(int M, int N, int K) {
     TiledPlan t;
     t.shape = large >= 160 ? 0 : small > 256 ? 1 : 2;
     t.slices = 1; t.steps_per_slice = nk; t.ws_floats = 0;
+    if (tiled_shape_forced >= 0 && K % TBK == 0) { t.shape = tiled_shape_forced; return t; }
     // blocks of 256 x 192 where they need fewer rounds of 256 workgroups times columns than 256 x 256
     // (6144 columns and 2048 rows: 256 blocks, one round, instead of 192 blocks that leave a quarter of the CUs idle)
     if (t.shape == 0 && K % TBK == 0) {
@@ -1094,6 +1097,15 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
     return launch_status();
 }
 }  // namespace
+
+// For measurements: forces the block shape of every product of more than 64 rows whose K is a multiple
+// of 64 (0: 256 x 256, 1: 128 x 128 two a CU, 2: 128 x 128 one a CU, 3: 64 x 64, 4: 256 x 192; -1: by size).
+// Returns the value before.
+TUFF_EXPORT int tuff_gemm_bf16_force_tiled_shape(int shape) {
+    const int old = tiled_shape_forced;
+    tiled_shape_forced = shape;
+    return old;
+}
 
 // How the sums of squares of tuff_gemm_bf16_accum_emit are laid out for a product of M rows:
 // *tiles tiles of columns, *rows rows each (16 for M <= 16, 64 for M <= 64).

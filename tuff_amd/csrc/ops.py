@@ -53,7 +53,7 @@ _SIGNATURES = {
         "tuff_qkv_post": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                           _c_void_p, _c_void_p, _c_int, _c_float,
                           _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
-                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_void_p],
         "tuff_rope_table": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p],
         "tuff_kv_write": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                           _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -461,7 +461,7 @@ def _gemm_workspace(M: int, N: int, K: int, device, emit: bool = False) -> Optio
 # ----------------------------------------------------------------- q/k/v post-processing
 def qkv_post(qkv, q_out, *, H, Hkv, hd, positions, eps=0.0, q_norm_w=None, k_norm_w=None,
              inv_freq=None, rotary_dim=0, interleaved=False, k_out=None,
-             k_cache=None, v_cache=None, slot_mapping=None, page_size=1) -> None:
+             k_cache=None, v_cache=None, slot_mapping=None, page_size=1, angles=None) -> None:
     T = qkv.shape[0]
     dt = qkv.dtype
     _gpu("qkv", qkv, shape=(T, (H + 2 * Hkv) * hd))
@@ -487,6 +487,7 @@ def qkv_post(qkv, q_out, *, H, Hkv, hd, positions, eps=0.0, q_norm_w=None, k_nor
         if rotary_dim <= 0 or rotary_dim > hd or rotary_dim % 2:
             raise KernelError(f"qkv_post: rotary_dim {rotary_dim} must be even and within the head size {hd}")
         _gpu("inv_freq", inv_freq, torch.float32, (rotary_dim // 2,))
+        _opt("angles", angles, torch.float32, (None, 2, rotary_dim // 2))      # rope_table(inv_freq, n)
     _gpu("positions", positions, torch.int32, (T,))
     if hd > 256:
         raise KernelError(f"qkv_post: head size {hd} above 256 is not supported")
@@ -494,7 +495,8 @@ def qkv_post(qkv, q_out, *, H, Hkv, hd, positions, eps=0.0, q_norm_w=None, k_nor
     _check(load("rope_kv").tuff_qkv_post(
         qkv.data_ptr(), q_out.data_ptr(), p(k_out), p(k_cache), p(v_cache), _dt(qkv),
         p(q_norm_w), p(k_norm_w), norm_dt, float(eps), p(inv_freq), int(rotary_dim), int(interleaved),
-        positions.data_ptr(), p(slot_mapping), T, H, Hkv, hd, page_size, _stream()), "qkv_post")
+        positions.data_ptr(), p(slot_mapping), T, H, Hkv, hd, page_size,
+        p(angles) if inv_freq is not None else None, 0 if angles is None else angles.shape[0], _stream()), "qkv_post")
 
 
 def rope_table(inv_freq: torch.Tensor, n_pos: int) -> torch.Tensor:

@@ -45,7 +45,8 @@ __global__ __launch_bounds__(POST_WAVES * WAVE) void qkv_post_kernel(
     const TW* __restrict__ q_norm_w, const TW* __restrict__ k_norm_w, float eps,
     const float* __restrict__ inv_freq, int rotary_dim, int interleaved,
     const int* __restrict__ positions, const int* __restrict__ slot_mapping,
-    int H, int Hkv, int hd, int page_size, int heads, int heads_per_wave) {
+    int H, int Hkv, int hd, int page_size, int heads, int heads_per_wave,
+    const float* __restrict__ angles, int n_angles) {
     __shared__ float vals_all[POST_WAVES][MAX_PER_LANE * WAVE];
     const int t = blockIdx.x, lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
     float* vals = vals_all[wave];
@@ -60,7 +61,8 @@ __global__ __launch_bounds__(POST_WAVES * WAVE) void qkv_post_kernel(
     int partner[MAX_PER_LANE];
     bool first[MAX_PER_LANE], turns[MAX_PER_LANE];
     if (inv_freq != nullptr && head_begin < H + Hkv) {
-        const float pos = (float)positions[t];
+        const int p = positions[t];
+        const float pos = (float)p;
 #pragma unroll
         for (int i = 0; i < MAX_PER_LANE; ++i) {
             const int j = lane + i * WAVE;
@@ -70,9 +72,14 @@ __global__ __launch_bounds__(POST_WAVES * WAVE) void qkv_post_kernel(
             else { first[i] = j < half; f = first[i] ? j : j - half; partner[i] = first[i] ? j + half : j - half; }
             rc[i] = 1.f; rs[i] = 0.f;
             if (turns[i]) {
-                const float a = pos * inv_freq[f];
-                rc[i] = cosf(a);
-                rs[i] = sinf(a);
+                if (p < n_angles) {                      // from the table: the same bits, without the two functions
+                    rc[i] = angles[((long long)p * 2) * half + f];
+                    rs[i] = angles[((long long)p * 2 + 1) * half + f];
+                } else {
+                    const float a = pos * inv_freq[f];
+                    rc[i] = cosf(a);
+                    rs[i] = sinf(a);
+                }
             }
         }
     }
@@ -160,7 +167,8 @@ __global__ __launch_bounds__(256) void qkv_post64_kernel(
     const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
     const TW* __restrict__ q_norm_w, const TW* __restrict__ k_norm_w, float eps, const float* __restrict__ inv_freq,
     const int* __restrict__ positions, const int* __restrict__ slot_mapping,
-    int n_tokens, int H, int Hkv, int page_size, int shares, int qk_blocks) {
+    int n_tokens, int H, int Hkv, int page_size, int shares, int qk_blocks,
+    const float* __restrict__ angles, int n_angles) {
     constexpr int HD = 64;
     const int tid = threadIdx.x;
     const int row_width = (H + 2 * Hkv) * HD;
@@ -172,14 +180,21 @@ __global__ __launch_bounds__(256) void qkv_post64_kernel(
         const int n_heads = k_cache ? H + Hkv : H;
         const int per = (n_heads + shares - 1) / shares;
         const int head_begin = share * per, head_end = min(n_heads, head_begin + per);
-        const float pos = (float)positions[t];
+        const int p = positions[t];
+        const float pos = (float)p;
         const bool first = l < 8;
         float rc[4], rs[4], wq[4], wk[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const float a = pos * inv_freq[(4 * l + e) & 31];
-            rc[e] = cosf(a);
-            rs[e] = sinf(a);
+            const int f = (4 * l + e) & 31;
+            if (p < n_angles) {                          // from the table: the same bits, without the two functions
+                rc[e] = angles[((long long)p * 2) * 32 + f];
+                rs[e] = angles[((long long)p * 2 + 1) * 32 + f];
+            } else {
+                const float a = pos * inv_freq[f];
+                rc[e] = cosf(a);
+                rs[e] = sinf(a);
+            }
             wq[e] = q_norm_w ? to_f32(q_norm_w[4 * l + e]) : 1.f;
             wk[e] = k_norm_w ? to_f32(k_norm_w[4 * l + e]) : 1.f;
         }
@@ -298,9 +313,11 @@ TUFF_EXPORT int tuff_qkv_post(const void* qkv, void* q_out, void* k_out, void* k
                               const void* q_norm_w, const void* k_norm_w, int norm_dt, float eps,
                               const float* inv_freq, int rotary_dim, int interleaved,
                               const int* positions, const int* slot_mapping,
-                              int n_tokens, int H, int Hkv, int hd, int page_size, hipStream_t stream) {
+                              int n_tokens, int H, int Hkv, int hd, int page_size,
+                              const float* angles, int n_angles, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (hd > MAX_PER_LANE * WAVE || rotary_dim > hd || (rotary_dim % 2) != 0) return -2;
+    if (!angles || !inv_freq) n_angles = 0;              // [n_angles][2][rotary_dim / 2] as tuff_rope_table makes it
     if (hd == 64 && inv_freq && rotary_dim == 64 && !interleaved && !k_out && page_size % 16 == 0) {
         // shares of a token's heads: enough sixteen-lane groups for the chip, whole heads each
         const int n_heads = k_cache ? H + Hkv : H;
@@ -311,7 +328,7 @@ TUFF_EXPORT int tuff_qkv_post(const void* qkv, void* q_out, void* k_out, void* k
         const int v_blocks = k_cache ? ceil_div(n_tokens, P64_TOKENS) * Hkv : 0;
 #define LAUNCH64(T, TW) hipLaunchKernelGGL((qkv_post64_kernel<T, TW>), dim3(qk_blocks + v_blocks), dim3(256), 0, stream, \
         (const T*)qkv, (T*)q_out, (T*)k_cache, (T*)v_cache, (const TW*)q_norm_w, (const TW*)k_norm_w, eps, inv_freq, \
-        positions, slot_mapping, n_tokens, H, Hkv, page_size, shares, qk_blocks)
+        positions, slot_mapping, n_tokens, H, Hkv, page_size, shares, qk_blocks, angles, n_angles)
         if (dt == DT_F32 && norm_dt == DT_F32) LAUNCH64(float, float);
         else if (dt == DT_F32) LAUNCH64(float, bf16_t);
         else if (norm_dt == DT_F32) LAUNCH64(bf16_t, float);
@@ -326,7 +343,7 @@ TUFF_EXPORT int tuff_qkv_post(const void* qkv, void* q_out, void* k_out, void* k
     dim3 grid(n_tokens, ceil_div(heads, POST_WAVES * heads_per_wave)), block(POST_WAVES * WAVE);
 #define LAUNCH(T, TW) hipLaunchKernelGGL((qkv_post_kernel<T, TW>), grid, block, 0, stream, (const T*)qkv, (T*)q_out, (T*)k_out, \
         (T*)k_cache, (T*)v_cache, (const TW*)q_norm_w, (const TW*)k_norm_w, eps, inv_freq, rotary_dim, interleaved, \
-        positions, slot_mapping, H, Hkv, hd, page_size, heads, heads_per_wave)
+        positions, slot_mapping, H, Hkv, hd, page_size, heads, heads_per_wave, angles, n_angles)
     if (dt == DT_F32 && norm_dt == DT_F32) LAUNCH(float, float);
     else if (dt == DT_F32) LAUNCH(float, bf16_t);
     else if (norm_dt == DT_F32) LAUNCH(bf16_t, float);

@@ -117,7 +117,8 @@ class AttentionMixer(Mixer):
             if fused:
                 rot = {}
                 if tables is not None:
-                    rot = dict(inv_freq=tables[0], rotary_dim=tables[1], interleaved=tables[2])
+                    rot = dict(inv_freq=tables[0], rotary_dim=tables[1], interleaved=tables[2],
+                               angles=getattr(self.position, "angle_table", lambda: None)())
                 wr = dict(k_cache=cache.k, v_cache=cache.v, slot_mapping=g.slot_mapping) if write_cache else {}
                 ops.qkv_post(qkv, q, H=H, Hkv=Hkv, hd=hd, positions=ctx.positions, page_size=cache.page_size,
                              **norm, **rot, **wr)
