@@ -33,8 +33,9 @@ SHAPE = dict(
     architectures=["Lfm2ForCausalLM"], num_hidden_layers=16, full_attn_idxs=[2, 5, 8, 10, 12, 14],
     hidden_size=2048, num_attention_heads=32, num_key_value_heads=8, block_ff_dim=12288,
     block_auto_adjust_ff_dim=True, block_multiple_of=256, vocab_size=65536, rope_theta=1000000.0,
-    conv_L_cache=3, norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=8192)
+    conv_L_cache=3, norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=131072)
 SEED = 2
+LONG_POINTS = ((8, 32768), (1, 131072))                 # (batch, context) measured beside the benchmark's own context
 PREFILL_TOKENS = 2048
 
 
@@ -266,7 +267,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--context", type=int, default=SHAPE["max_position_embeddings"])
+    ap.add_argument("--context", type=int, default=8192)
+    ap.add_argument("--no-long-points", dest="long_points", action="store_false",
+                    help="skip decode at batch 8, context 32768 and at batch 1, context 131072")
     ap.add_argument("--layers", type=int, default=SHAPE["num_hidden_layers"],
                     help="fewer layers than the shape has (sizes of a layer stay)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
@@ -308,10 +311,11 @@ def main() -> int:
         print(json.dumps({"prefill": prefill_record(run_prefill(llm, cfg, PREFILL_TOKENS), flops, args.dtype)}))
         return 0
 
-    def decode_point(batch: int, steps: int, warmup: int, seed: int) -> dict:
+    def decode_point(batch: int, steps: int, warmup: int, seed: int, context: int = 0, on=None) -> dict:
+        context = context or args.context
         secs, ctx_mean = [], 0.0
         for run in range(args.runs):
-            s_, ctx_mean = run_decode(llm, cfg, batch, args.context, steps, warmup, seed + 1000 * run)
+            s_, ctx_mean = run_decode(on or llm, cfg, batch, context, steps, warmup, seed + 1000 * run)
             secs.append(s_)
         rates = [batch * steps / s_ for s_ in secs]
         rate, spread = mean_spread(rates)
@@ -349,6 +353,21 @@ def main() -> int:
             points[f"decode_b{b}_ms_per_step"] = round(pt["ms"], 4)
             points[f"decode_b{b}_GBs"] = round(pt["GBs"], 1)
             points[f"decode_b{b}_roofline_frac"] = round(pt["GBs"] / HBM_PEAK_GBS, 4)
+        if args.long_points:
+            # the same model further out: the cache of the live requests is then most of what a step reads
+            for b, ctx in LONG_POINTS:
+                key = f"decode_b{b}_ctx{ctx}"
+                if b * ctx > max_b * args.context:
+                    continue                                  # the pool was made for max_b requests of --context
+                try:
+                    far = LLM(engine=eng, max_num_seqs=max_b, max_batched_tokens=2048, ctx_size=ctx, ignore_eos=True)
+                    pt = decode_point(b, 32, 4, SEED + ctx, context=ctx, on=far)
+                    points[key] = round(pt["tok_s"], 1)
+                    points[key + "_ms_per_step"] = round(pt["ms"], 4)
+                    points[key + "_roofline_frac"] = round(pt["GBs"] / HBM_PEAK_GBS, 4)
+                except Exception as e:                        # noqa: BLE001 - a point beside the benchmark must not lose it
+                    points[key] = None
+                    points[key + "_error"] = f"{type(e).__name__}: {e}"[:200]
         out["points"] = points
     if args.probe and args.dtype == "bf16":
         del llm

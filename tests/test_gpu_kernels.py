@@ -673,6 +673,12 @@ def test_attention_long_context(gpu):
         ops.attention_mfma(case["q"].to(gpu), case["kc"], case["vc"], out, blocks=blocks, nb=1,
                            positions=case["positions"], **common)
         _check_step(case, reqs, out.cpu().double().reshape(T, H, hd), H, hd, window, ("mfma", window))
+        # a wider block table and more (empty) partitions, as a recorded step's buckets bring: the same bits
+        wide = torch.cat([case["table"], torch.full((len(reqs), 400), -1, dtype=torch.int32, device=gpu)], dim=1).contiguous()
+        out_w = torch.full((T, H * hd), float("nan"), dtype=torch.bfloat16, device=gpu)
+        ops.attention_mfma(case["q"].to(gpu), case["kc"], case["vc"], out_w, blocks=blocks, nb=1, positions=case["positions"],
+                           **dict(common, block_table=wide, max_ctx_len=case["max_ctx_len"] + 6000))
+        assert torch.equal(out, out_w), "the merge depends on how many partitions the step has room for"
         out2 = torch.full((T, H * hd), float("nan"), dtype=torch.bfloat16, device=gpu)
         cols = ops.attention_prefill_block_columns(hd)
         blocks = torch.from_numpy(ops.query_blocks(case["q_len"], H // Hkv, cols // 16)).to(gpu)

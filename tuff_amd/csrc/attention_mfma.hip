@@ -547,56 +547,93 @@ __global__ __launch_bounds__(WAVE) void attn_combine64_kernel(const float* __res
     }
 }
 
-__global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
-                                                            bf16_t* __restrict__ out, const int* __restrict__ positions,
-                                                            int H, int hd, int window, int n_parts, int part_keys) {
+// More than 64 partitions (contexts beyond 16,384 keys): the partitions are taken in groups of 64 by
+// their absolute numbers (0..63, 64..127, ...); a wave sums a group in ascending order as above, the
+// waves of the workgroup take the groups in turn, and the groups' sums are added in ascending order.
+// The grouping is by absolute partition number, so the result still depends on the token's position only.
+constexpr int COMBINE_WAVES = 8;
+constexpr int COMBINE_GROUP = 64;
+constexpr int COMBINE_MAX_GROUPS = COMBINE_MAX_PARTS / COMBINE_GROUP;
+
+__global__ __launch_bounds__(COMBINE_WAVES * WAVE) void attn_combine_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+                                                                            bf16_t* __restrict__ out, const int* __restrict__ positions,
+                                                                            int H, int hd, int window, int n_parts, int part_keys) {
     __shared__ float wts[COMBINE_MAX_PARTS], wls[COMBINE_MAX_PARTS];
+    __shared__ float grp_acc[COMBINE_MAX_GROUPS][256], grp_l[COMBINE_MAX_GROUPS];
+    __shared__ float red[COMBINE_WAVES];
     const long long row = blockIdx.x;                      // token * H + head
-    const int lane = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
     const int pos = positions[row / H];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int p_lo = lo / part_keys, np = pos / part_keys - p_lo + 1;
-    const float* ml = ws_ml + (row * n_parts + p_lo) * 2;
+    const int p_lo = lo / part_keys, p_hi = pos / part_keys;          // the token's partitions, absolute numbers
+    const float* ml = ws_ml + row * n_parts * 2;
     float M = -INFINITY;
-    for (int i = lane; i < np; i += WAVE) M = fmaxf(M, ml[i * 2 + 1] > 0.f ? ml[i * 2] : -INFINITY);
+    for (int p = p_lo + tid; p <= p_hi; p += COMBINE_WAVES * WAVE) M = fmaxf(M, ml[p * 2 + 1] > 0.f ? ml[p * 2] : -INFINITY);
     M = wave_max(M);
-    for (int i = lane; i < np; i += WAVE) {
-        const float l = ml[i * 2 + 1];
-        const float w = l > 0.f ? __expf(ml[i * 2] - M) : 0.f;
-        wts[i] = w;
-        wls[i] = w * (l > 0.f ? l : 0.f);
+    if (lane == 0) red[wave] = M;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < COMBINE_WAVES; ++w) M = fmaxf(M, red[w]);
+    for (int p = p_lo + tid; p <= p_hi; p += COMBINE_WAVES * WAVE) {
+        const float l = ml[p * 2 + 1];
+        const float w = l > 0.f ? __expf(ml[p * 2] - M) : 0.f;
+        wts[p] = w;
+        wls[p] = w * (l > 0.f ? l : 0.f);
     }
     __syncthreads();
-    const float* o = ws_o + (row * n_parts + p_lo) * hd;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    float L = 0.f;
-    // the partial outputs of sixteen partitions are asked for together; the sums run in ascending order
+    const int g_lo = p_lo / COMBINE_GROUP, g_hi = p_hi / COMBINE_GROUP;
     const int per = (hd + WAVE - 1) / WAVE;                // channels a lane
-    for (int i0 = 0; i0 < np; i0 += 16) {
-        float ov[16][4];
+    const float* o = ws_o + row * n_parts * hd;
+    for (int grp = g_lo + wave; grp <= g_hi; grp += COMBINE_WAVES) {
+        const int a = max(p_lo, grp * COMBINE_GROUP), b = min(p_hi, grp * COMBINE_GROUP + COMBINE_GROUP - 1);
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        float L = 0.f;
+        // the partial outputs of sixteen partitions are asked for together; the sums run in ascending order
+        for (int i0 = a; i0 <= b; i0 += 16) {
+            float ov[16][4];
 #pragma unroll
-        for (int u = 0; u < 16; ++u)
+            for (int u = 0; u < 16; ++u)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int d = lane + j * WAVE;
+                    ov[u][j] = (j < per && i0 + u <= b && d < hd) ? o[(long long)(i0 + u) * hd + d] : 0.f;
+                }
+#pragma unroll
+            for (int u = 0; u < 16; ++u)
+                if (i0 + u <= b) {
+                    const float w = wts[i0 + u];
+                    L += wls[i0 + u];
+                    if (w > 0.f) {                         // a partition without weight may hold anything
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) acc[j] = fmaf(w, ov[u][j], acc[j]);
+                    }
+                }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int d = lane + j * WAVE;
+            if (d < hd) grp_acc[grp][d] = acc[j];
+        }
+        if (lane == 0) grp_l[grp] = L;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        float L = 0.f;
+        for (int grp = g_lo; grp <= g_hi; ++grp) {
+            L += grp_l[grp];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int d = lane + j * WAVE;
-                ov[u][j] = (j < per && i0 + u < np && d < hd) ? o[(long long)(i0 + u) * hd + d] : 0.f;
+                if (d < hd) acc[j] += grp_acc[grp][d];
             }
+        }
+        const float inv = 1.0f / L;
 #pragma unroll
-        for (int u = 0; u < 16; ++u)
-            if (i0 + u < np) {
-                const float w = wts[i0 + u];
-                L += wls[i0 + u];
-                if (w > 0.f) {                             // a partition without weight may hold anything
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) acc[j] = fmaf(w, ov[u][j], acc[j]);
-                }
-            }
-    }
-    const float inv = 1.0f / L;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int d = lane + j * WAVE;
-        if (d < hd) out[row * hd + d] = (bf16_t)(acc[j] * inv);
+        for (int j = 0; j < 4; ++j) {
+            const int d = lane + j * WAVE;
+            if (d < hd) out[row * hd + d] = (bf16_t)(acc[j] * inv);
+        }
     }
 }
 
@@ -635,8 +672,8 @@ static int launch_merge(const float* ws_o, const float* ws_ml, bf16_t* out, cons
         else COMBINE(4, 8);
 #undef COMBINE
     } else {
-        hipLaunchKernelGGL(attn_combine_kernel, grid, dim3(WAVE), 0, stream, ws_o, ws_ml, out, positions, H, hd, window, n_parts,
-                           part_keys);
+        hipLaunchKernelGGL(attn_combine_kernel, grid, dim3(COMBINE_WAVES * WAVE), 0, stream, ws_o, ws_ml, out, positions, H, hd,
+                           window, n_parts, part_keys);
     }
     return launch_status();
 }
