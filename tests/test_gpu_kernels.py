@@ -161,6 +161,55 @@ def test_gemm_that_prepares_the_next_norm(gpu, M, d, K1, N2):
     assert (sw.cpu().double() - ref).abs().max() <= 2 ** -6 * max(float(ref.abs().max()), 0.1 * float(want.abs().max()))
 
 
+@pytest.mark.parametrize("M,d,K1,N2", [(2048, 2048, 2048, 6144), (1000, 2048, 8192, 3072), (130, 256, 128, 512),
+                                       (700, 1536, 6912, 13824), (4096, 2048, 2048, 16384), (65, 192, 64, 384),
+                                       (512, 2040, 8192, 2048), (300, 256, 8192, 512)])
+def test_tiled_gemm_that_prepares_the_next_norm(gpu, M, d, K1, N2):
+    """The same for more than 64 rows (the tiled product): each wave of the accumulating product leaves the
+    sums of squares of its rows over its columns, and the next product scales its rows."""
+    from tuff_amd.csrc import ops
+    a = _r(M, K1, seed=1, dtype=torch.bfloat16)
+    w1 = _r(d, K1, seed=2, scale=K1 ** -0.5, dtype=torch.bfloat16)
+    res0 = _r(M, d, seed=3)
+    nw = 1 + _r(d, seed=4, scale=0.1)
+    w2 = _r(N2, d, seed=5, scale=d ** -0.5, dtype=torch.bfloat16)
+    eps = 1e-5
+    layout = ops.gemm_emit_layout(M, d, K1)
+    assert layout is not None and layout[1] == M
+    res = res0.to(gpu)
+    xw = torch.empty(M, d, dtype=torch.bfloat16, device=gpu)
+    ss = torch.full(layout, float("nan"), device=gpu)
+    ops.gemm_accum_emit(a.to(gpu), w1.to(gpu), res, nw.to(gpu), xw, ss)
+    plain_acc = res0.to(gpu)
+    ops.gemm(a.to(gpu), w1.to(gpu), plain_acc, accumulate=True)
+    assert torch.equal(plain_acc, res)                       # the residual itself is what the plain product gives
+    got_res = res.cpu().double()
+    assert (xw.cpu().double() - got_res * nw.double()).abs().max() <= 2 ** -8 * float((got_res * nw).abs().max())
+    assert (ss.cpu().double().sum(0) - (got_res ** 2).sum(1)).abs().max() <= 1e-5 * float((got_res ** 2).sum(1).max())
+    want = plain.rms_norm(got_res, nw.double(), eps) @ w2.double().T
+    assert ops.gemm_scaled_supported(M, N2, d) and not ops.gemm_scaled_supported(M, N2, d, torch.float32)
+    out = torch.empty(M, N2, dtype=torch.bfloat16, device=gpu)
+    ops.gemm_scaled(xw, ss, eps, w2.to(gpu), out)
+    assert (out.cpu().double() - want).abs().max() <= 2 ** -6 * float(want.abs().max())
+    sw = torch.empty(M, N2 // 2, device=gpu, dtype=torch.bfloat16)
+    ops.gemm_scaled(xw, ss, eps, w2.to(gpu), sw, swiglu=True)
+    g, u = want[:, 0::2], want[:, 1::2]
+    ref = g / (1 + torch.exp(-g)) * u
+    assert (sw.cpu().double() - ref).abs().max() <= 2 ** -5 * max(float(ref.abs().max()), 0.1 * float(want.abs().max()))
+
+
+def test_products_that_cannot_prepare_the_next_norm_say_so(gpu):
+    from tuff_amd.csrc import ops
+    assert ops.gemm_emit_layout(300, 2048, 8192) == (32, 300)     # cut into slices: the kernel that adds them emits
+    assert ops.gemm_emit_layout(500, 200, 256) is None            # a last block of columns that is not whole
+    assert ops.gemm_emit_layout(500, 256, 136) is None            # K no multiple of 64
+    assert not ops.gemm_scaled_supported(500, 256, 136) and ops.gemm_scaled_supported(300, 2048, 8192)
+    with pytest.raises(ops.KernelError, match="cannot leave"):
+        ops.gemm_accum_emit(torch.zeros(500, 136, dtype=torch.bfloat16, device=gpu), torch.zeros(256, 136, dtype=torch.bfloat16, device=gpu),
+                            torch.zeros(500, 256, device=gpu), torch.ones(256, device=gpu),
+                            torch.empty(500, 256, dtype=torch.bfloat16, device=gpu), torch.empty(4, 500, device=gpu))
+
+
 def test_gemm_refuses_what_it_cannot_do(gpu):
     from tuff_amd.csrc import ops
     x = torch.zeros(2, 12, dtype=torch.bfloat16, device=gpu)

@@ -122,6 +122,18 @@ __device__ __forceinline__ void store_quad(void* Y, long long row, long long col
     }
 }
 
+// What the tiled product can do around an RMSNorm, as the skinny products do (described with them below):
+// TILED_SCALED: X is bf16(x * norm weight) and ss_in [n_ss][M] holds sums of squares of each row of x over
+// n_ss groups of columns; every row of the result is scaled by 1 / sqrt(sum / K + eps).  TILED_EMIT (adding
+// into the float32 residual stream Y): the new Y is also written as bf16(Y * emit_nw[col]) to emit_xw, and
+// each workgroup leaves the sums of squares of its rows over its columns in emit_ss [block column][M] (the
+// waves that share rows add theirs in the order of their columns).
+struct TiledExtra {
+    const float* ss_in = nullptr; int n_ss = 0; float eps = 0.f;
+    const float* emit_nw = nullptr; bf16_t* emit_xw = nullptr; float* emit_ss = nullptr;
+};
+enum : int { TILED_PLAIN = 0, TILED_SCALED = 1, TILED_EMIT = 2 };
+
 template <int TM, int TN, int WAVES_M, int WAVES_N, int AHEAD, int MODE>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_tiled_kernel(
         const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, int M, int N, int K,
@@ -283,10 +295,11 @@ __device__ __forceinline__ void wait_loads_and_lds() {               // s_waitcn
     __builtin_amdgcn_s_waitcnt((VM & 15) | ((VM >> 4) << 14) | 0x0070);
 }
 
-template <int TM, int TN, int WAVES_M, int WAVES_N, int STAGES, int MODE>
+template <int TM, int TN, int WAVES_M, int WAVES_N, int STAGES, int MODE, int AROUND>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_dma_kernel(
         const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, int M, int N, int K,
-        int steps_per_slice, float* __restrict__ ws) {
+        int steps_per_slice, float* __restrict__ ws, TiledExtra ex) {
+    static_assert(AROUND != TILED_EMIT || MODE == OUT_F32_ACCUM, "the emitting epilogue adds into the residual stream");
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int BM = 16 * TM * WAVES_M, BN = 16 * TN * WAVES_N;
     constexpr int IA = BM / 8 / NW, IB = BN / 8 / NW;                  // load instructions of X and of W a wave issues a step
@@ -382,6 +395,28 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_dma_kernel(
         constexpr int st = decltype(s)::value;
         if (kt_begin + st < kt_end) issue(st, kt_begin + st);
     });
+    __shared__ float row_scale[AROUND == TILED_SCALED ? BM : 1];
+    if constexpr (AROUND == TILED_SCALED) {
+        // while the first operands are on their way: the scale of each of the block's rows, its groups' sums in order
+        // (a product cut along K leaves that to the kernel that adds the slices)
+        for (int r = tid; r < BM && gridDim.z == 1; r += 64 * NW) {
+            const long long row = m0 + r;
+            float t = 0.f;
+            if (row < M) {
+                // sixteen groups' sums are asked for together (one after the other would be as many trips to
+                // memory), then added in their order
+                for (int j0 = 0; j0 < ex.n_ss; j0 += 16) {
+                    float v[16];
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) v[u] = j0 + u < ex.n_ss ? ex.ss_in[(long long)(j0 + u) * M + row] : 0.f;
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) t += v[u];
+                }
+            }
+            row_scale[r] = 1.0f / sqrtf(t / (float)K + ex.eps);
+        }
+        // read in the epilogue, behind the barriers of the loop (every wave waits for its LDS writes before each)
+    }
     for (int kt0 = kt_begin; kt0 < kt_end; kt0 += STAGES) {
         static_for<STAGES>([&](auto u) {
             constexpr int buf = decltype(u)::value;
@@ -415,11 +450,61 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_dma_kernel(
                 store_quad<OUT_F32>(mine, m0 + wm + i * 16 + r16, n0 + wn + j * 16 + g * 4, M, N, acc[i][j]);
         return;
     }
+    if constexpr (AROUND == TILED_EMIT) {
+        // whole blocks of columns only (the host sees to it): Y += acc, the next norm's operand, the row's sum of squares
+        float wave_sq[TM];
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i) {
+            const long long row = m0 + wm + i * 16 + r16;
+            float sq = 0.f;
+            if (row < M) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-            store_quad<MODE>(Y, m0 + wm + i * 16 + r16, n0 + wn + j * 16 + g * 4, M, N, acc[i][j]);
+                for (int j = 0; j < TN; ++j) {
+                    const long long col = n0 + wn + j * 16 + g * 4;
+                    f32x4* yp = (f32x4*)((float*)Y + row * N + col);
+                    f32x4 y = *yp;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) y[e] += acc[i][j][e];
+                    *yp = y;
+                    const f32x4 nw = *(const f32x4*)(ex.emit_nw + col);
+                    bf16x4 o = {(bf16_t)(y[0] * nw[0]), (bf16_t)(y[1] * nw[1]), (bf16_t)(y[2] * nw[2]), (bf16_t)(y[3] * nw[3])};
+                    *(bf16x4*)(ex.emit_xw + row * N + col) = o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) sq = fmaf(y[e], y[e], sq);
+                }
+            }
+            sq += __shfl_xor(sq, 16, WAVE);
+            sq += __shfl_xor(sq, 32, WAVE);
+            wave_sq[i] = sq;
+        }
+        // the waves that share rows add their sums in the order of their columns, through the LDS the operands
+        // have left: one sum per row and block of columns, so that whoever reads them asks only once
+        float* red = (float*)tiles;                            // [WAVES_N][BM]
+        __syncthreads();                                       // nobody reads operands any more
+        if (g == 0) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) red[(wave % WAVES_N) * BM + wm + i * 16 + r16] = wave_sq[i];
+        }
+        __syncthreads();
+        for (int r = tid; r < BM; r += 64 * NW) {
+            float t = red[r];
+#pragma unroll
+            for (int w = 1; w < WAVES_N; ++w) t += red[w * BM + r];
+            if (m0 + r < M) ex.emit_ss[(long long)blockIdx.x * M + m0 + r] = t;
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        float sc = 1.f;
+        if constexpr (AROUND == TILED_SCALED) sc = row_scale[wm + i * 16 + r16];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            f32x4 v = acc[i][j];
+            if constexpr (AROUND == TILED_SCALED) { v[0] *= sc; v[1] *= sc; v[2] *= sc; v[3] *= sc; }
+            store_quad<MODE>(Y, m0 + wm + i * 16 + r16, n0 + wn + j * 16 + g * 4, M, N, v);
+        }
+    }
 }
 
 // ----------------------------------------------------------------- skinny kernels
@@ -805,6 +890,7 @@ __global__ __launch_bounds__(SK_NT) void gemm_bf16_skinny64_kernel(const bf16_t*
 struct FinishExtra {
     const float* ss_in = nullptr; int n_ss = 0; float eps = 0.f; int K = 0;                 // NORM_SCALED
     const float* emit_nw = nullptr; bf16_t* emit_xw = nullptr; float* emit_ss = nullptr;   // EMIT
+    int ss_rows = 64;                     // rows of a tile of sums of squares, read or written: 64, or M for the tiled product
 };
 
 template <int MODE, int NORM, bool EMIT>
@@ -818,7 +904,8 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const float* __restr
     if (NORM == NORM_SCALED) {
         // the sixteen threads of a row add the tiles q, q + 16, ... and then each other, in a fixed butterfly
         float t = 0.f;
-        for (int j = q; j < ex.n_ss; j += 16) t += ex.ss_in[(long long)j * 64 + row];
+        if (row < ex.ss_rows)
+            for (int j = q; j < ex.n_ss; j += 16) t += ex.ss_in[(long long)j * ex.ss_rows + row];
         t += __shfl_xor(t, 1, WAVE);
         t += __shfl_xor(t, 2, WAVE);
         t += __shfl_xor(t, 4, WAVE);
@@ -879,7 +966,7 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const float* __restr
         sq += __shfl_xor(sq, 2, WAVE);
         sq += __shfl_xor(sq, 4, WAVE);
         sq += __shfl_xor(sq, 8, WAVE);
-        if (q == 0) ex.emit_ss[(long long)blockIdx.x * 64 + row] = sq;      // rows M .. 63 of the tile: zero
+        if (q == 0 && row < ex.ss_rows) ex.emit_ss[(long long)blockIdx.x * ex.ss_rows + row] = sq;   // rows beyond M: zero
     }
 }
 
@@ -1040,12 +1127,27 @@ int launch_skinny64_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N
     return -3;
 }
 
-template <int MODE>
-int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, float* ws, hipStream_t stream) {
-    if (M <= 16) return launch_skinny16<MODE, NORM_NONE, false>(X, W, Y, M, N, K, Skinny16Extra(), stream);
-    if (M <= 64) {
-        return launch_skinny64<MODE, NORM_NONE, false>(X, W, Y, M, N, K, ws, FinishExtra(), stream);
-    } else {
+// How the sums of squares of a tiled product with the emitting epilogue are grouped: columns a group, or 0
+// where this product cannot emit (K no multiple of 64, K cut into slices, N no whole number of blocks).
+int tiled_emit_group(int M, int N, int K) {
+    const TiledPlan t = plan_tiled(M, N, K);
+    if (t.slices > 1) return 64;                        // the kernel that adds the slices emits, 64 columns a workgroup
+    if (K % TBK != 0) return 0;
+    const int bn = t.shape == 0 ? 256 : t.shape == 4 ? 192 : t.shape == 3 ? 64 : 128;
+    if (N % bn != 0) return 0;
+    return bn;                                          // a workgroup's columns
+}
+
+bool tiled_scaled_ok(int M, int N, int K) { return K % TBK == 0 || plan_tiled(M, N, K).slices > 1; }
+
+template <int MODE, int AROUND = TILED_PLAIN>
+int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, float* ws, hipStream_t stream,
+                const TiledExtra& ex = TiledExtra()) {
+    if constexpr (AROUND == TILED_PLAIN) {
+        if (M <= 16) return launch_skinny16<MODE, NORM_NONE, false>(X, W, Y, M, N, K, Skinny16Extra(), stream);
+        if (M <= 64) return launch_skinny64<MODE, NORM_NONE, false>(X, W, Y, M, N, K, ws, FinishExtra(), stream);
+    }
+    {
         // Large blocks where they give most CUs one.  Of the small ones a CU holds two if there are
         // enough; if not, a block is alone on its CU and hides the memory's latency by itself, with
         // the operands of four steps under way.  Where even the small blocks are fewer than half the
@@ -1065,7 +1167,7 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
                                X, W, Y, M, N, K, t.steps_per_slice, ws); \
         } while (0)
 #define TILED_DMA(TM, TN, WM, WN, STAGES) do { \
-            auto kern = gemm_bf16_dma_kernel<TM, TN, WM, WN, STAGES, MODE>; \
+            auto kern = gemm_bf16_dma_kernel<TM, TN, WM, WN, STAGES, MODE, AROUND>; \
             constexpr int bm = 16 * TM * WM, bn = 16 * TN * WN, lds = STAGES * (bm + bn) * TBK * 2; \
             static bool set = false; \
             if (!set) { \
@@ -1073,8 +1175,11 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
                 set = true; \
             } \
             hipLaunchKernelGGL(kern, dim3(ceil_div(N, bn), ceil_div(M, bm), t.slices), dim3(64 * WM * WN), lds, stream, \
-                               X, W, Y, M, N, K, t.steps_per_slice, ws); \
+                               X, W, Y, M, N, K, t.steps_per_slice, ws, ex); \
         } while (0)
+        if constexpr (AROUND != TILED_PLAIN) {
+            if (K % TBK != 0 && t.slices == 1) return -2;            // a product in slices is finished by the kernel that adds them
+        }
         if (K % TBK == 0) {
             if (t.shape == 3) TILED_DMA(2, 2, 2, 2, 4);
             else if (t.shape == 4) TILED_DMA(8, 3, 2, 4, 2);
@@ -1090,8 +1195,13 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
         if (t.slices > 1) {
             int rc = launch_status();
             if (rc) return rc;
-            hipLaunchKernelGGL((splitk_finish_kernel<MODE, NORM_NONE, false>), dim3(ceil_div(N, 64), ceil_div(M, 16)), dim3(256), 0,
-                               stream, (const float*)ws, Y, M, N, M, t.slices, FinishExtra());
+            FinishExtra fx;
+            fx.ss_rows = M;
+            fx.ss_in = ex.ss_in; fx.n_ss = ex.n_ss; fx.eps = ex.eps; fx.K = K;
+            fx.emit_nw = ex.emit_nw; fx.emit_xw = ex.emit_xw; fx.emit_ss = ex.emit_ss;
+            constexpr int FN = AROUND == TILED_SCALED ? NORM_SCALED : NORM_NONE;
+            hipLaunchKernelGGL((splitk_finish_kernel<MODE, FN, AROUND == TILED_EMIT>), dim3(ceil_div(N, 64), ceil_div(M, 16)),
+                               dim3(256), 0, stream, (const float*)ws, Y, M, N, M, t.slices, fx);
         }
     }
     return launch_status();
@@ -1110,10 +1220,23 @@ TUFF_EXPORT int tuff_gemm_bf16_force_tiled_shape(int shape) {
 // How the sums of squares of tuff_gemm_bf16_accum_emit are laid out for a product of M rows:
 // *tiles tiles of columns, *rows rows each (16 for M <= 16, 64 for M <= 64).
 TUFF_EXPORT int tuff_gemm_bf16_emit_layout(int M, int N, int K, int* tiles, int* rows) {
-    if (M > 64) return -2;
+    if (M > 64) {
+        // the tiled product: a group of columns a wave, M rows each; *tiles = 0 where it cannot emit
+        const int group = tiled_emit_group(M, N, K);
+        *tiles = group ? ceil_div(N, group) : 0;        // (a product in slices may end in a partial group of columns)
+        *rows = M;
+        return 0;
+    }
     *tiles = plan_skinny(M, N, K, 16, true).tiles;
     *rows = M <= 16 ? 16 : 64;
     return 0;
+}
+
+// 1 if tuff_gemm_bf16_scaled takes a product of these sizes (always for M <= 64; for more rows where the
+// tiled product runs it in one piece), else 0.
+TUFF_EXPORT int tuff_gemm_bf16_scaled_supported(int M, int N, int K) {
+    if (K % 8 != 0 || M <= 0 || N <= 0) return 0;
+    return M <= 64 || tiled_scaled_ok(M, N, K) ? 1 : 0;
 }
 
 // Work space a product of this shape needs: *ws_floats float32 for partial tiles (0: none).
@@ -1154,14 +1277,21 @@ TUFF_EXPORT int tuff_gemm_bf16_normed(const float* X, const int* rows, const flo
     return launch_skinny16_mode<NORM_INSIDE>(X, (const bf16_t*)W, Y, M, N, K, mode, x, stream);
 }
 
-// For M <= 64 rows:  Y += X W^T, and from the new Y (the residual stream, float32 [M, N]) the
+// Y += X W^T, and from the new Y (the residual stream, float32 [M, N]) the
 // operand of the RMSNorm that follows: xw = bf16(Y * next_norm_w) [M, N] and ss [tiles][rows] (as
-// tuff_gemm_bf16_emit_layout says), the sums of squares of each row over each tile of columns.
+// tuff_gemm_bf16_emit_layout says; 0 tiles: this product cannot, -2), the sums of squares of each row
+// over each tile of columns.
 // ws: for M > 16, the work space tuff_gemm_bf16_workspace(M, N, K, 1) asks for.
 TUFF_EXPORT int tuff_gemm_bf16_accum_emit(const void* X, const void* W, float* Y, int M, int N, int K,
                                           const float* next_norm_w, void* xw, float* ss, float* ws, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (K % 8 != 0 || M > 64) return -2;
+    if (K % 8 != 0) return -2;
+    if (M > 64) {
+        if (!tiled_emit_group(M, N, K)) return -2;
+        TiledExtra t;
+        t.emit_nw = next_norm_w; t.emit_xw = (bf16_t*)xw; t.emit_ss = ss;
+        return launch_mode<OUT_F32_ACCUM, TILED_EMIT>((const bf16_t*)X, (const bf16_t*)W, Y, M, N, K, ws, stream, t);
+    }
     if (M <= 16) {
         Skinny16Extra x;
         x.emit_nw = next_norm_w; x.emit_xw = (bf16_t*)xw; x.emit_ss = ss;
@@ -1172,13 +1302,28 @@ TUFF_EXPORT int tuff_gemm_bf16_accum_emit(const void* X, const void* W, float* Y
     return launch_skinny64<OUT_F32_ACCUM, NORM_NONE, true>((const bf16_t*)X, (const bf16_t*)W, Y, M, N, K, ws, x, stream);
 }
 
-// For M <= 64 rows:  Y (=|+=) (XW W^T) scaled per row by 1 / sqrt(sum_t ss[t][row] / K + eps), with
-// XW and ss as tuff_gemm_bf16_accum_emit leaves them for the same M (n_ss tiles).
+// Y (=|+=) (XW W^T) scaled per row by 1 / sqrt(sum_t ss[t][row] / K + eps), with
+// XW and ss as tuff_gemm_bf16_accum_emit leaves them for the same M (n_ss tiles); see
+// tuff_gemm_bf16_scaled_supported for M > 64.
 // ws: for M > 16, the work space tuff_gemm_bf16_workspace(M, N, K, 0) asks for.
 TUFF_EXPORT int tuff_gemm_bf16_scaled(const void* XW, const float* ss, int n_ss, float eps, const void* W, void* Y,
                                       int M, int N, int K, int mode, float* ws, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (K % 8 != 0 || M > 64 || n_ss < 1) return -2;
+    if (K % 8 != 0 || n_ss < 1) return -2;
+    if (M > 64) {
+        // ss [n_ss][M]; bfloat16 and SwiGLU outputs (what reads a norm in a layer)
+        if (!tiled_scaled_ok(M, N, K)) return -2;
+        TiledExtra t;
+        t.ss_in = ss; t.n_ss = n_ss; t.eps = eps;
+        const bf16_t* x = (const bf16_t*)XW;
+        const bf16_t* w = (const bf16_t*)W;
+        if (mode == OUT_BF16) return launch_mode<OUT_BF16, TILED_SCALED>(x, w, Y, M, N, K, ws, stream, t);
+        if (mode == OUT_SWIGLU) {
+            if (N % 2) return -2;
+            return launch_mode<OUT_SWIGLU, TILED_SCALED>(x, w, Y, M, N, K, ws, stream, t);
+        }
+        return -3;
+    }
     if (M <= 16) {
         Skinny16Extra x;
         x.ss_in = ss; x.n_ss = n_ss; x.eps = eps;

@@ -40,6 +40,7 @@ _SIGNATURES = {
         "tuff_gemm_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
         "tuff_gemm_bf16_workspace": [_c_int, _c_int, _c_int, _c_int, ctypes.POINTER(_c_ll)],
         "tuff_gemm_bf16_emit_layout": [_c_int, _c_int, _c_int, ctypes.POINTER(_c_int), ctypes.POINTER(_c_int)],
+        "tuff_gemm_bf16_scaled_supported": [_c_int, _c_int, _c_int],
         "tuff_gemm_bf16_accum_emit": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                                       _c_void_p, _c_void_p, _c_void_p],
         "tuff_gemm_bf16_scaled": [_c_void_p, _c_void_p, _c_int, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
@@ -312,7 +313,7 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
 
 
 NORMED_MAX_ROWS, NORMED_MAX_K = 16, 8192      # gemm_normed: the norm inside the product's kernel
-EMIT_MAX_ROWS = 64                            # gemm_accum_emit / gemm_scaled
+EMIT_MAX_ROWS = 64                            # gemm_accum_emit / gemm_scaled: the skinny products; beyond, the tiled one
 
 
 def gemm_normed(x: torch.Tensor, norm_w: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor, *,
@@ -339,22 +340,23 @@ def gemm_normed(x: torch.Tensor, norm_w: torch.Tensor, eps: float, w: torch.Tens
 _emit_layouts: dict = {}
 
 
-def gemm_emit_layout(M: int, N: int, K: int) -> tuple:
+def gemm_emit_layout(M: int, N: int, K: int) -> Optional[tuple]:
     """(tiles, rows): shape of the sums of squares gemm_accum_emit leaves for a product of M rows
-    with N outputs and inner size K."""
-    key = (M <= 16, N, K)
+    with N outputs and inner size K, or None where such a product cannot leave them (more than 64 rows
+    and an inner size that is no multiple of 64, a product cut along K, a last block of columns that is
+    not whole)."""
+    key = (M if M > EMIT_MAX_ROWS else M <= 16, N, K)
     if key not in _emit_layouts:
         t, r = _c_int(0), _c_int(0)
         _check(load("gemm_bf16").tuff_gemm_bf16_emit_layout(M, N, K, ctypes.byref(t), ctypes.byref(r)), "gemm_emit_layout")
-        _emit_layouts[key] = (int(t.value), int(r.value))
+        _emit_layouts[key] = (int(t.value), int(r.value)) if t.value > 0 else None
     return _emit_layouts[key]
 
 
 def gemm_accum_emit(x: torch.Tensor, w, residual: torch.Tensor, next_norm_w: torch.Tensor,
                     xw: torch.Tensor, ss: torch.Tensor) -> None:
-    """residual += x @ w.T for at most 64 rows, and for the RMSNorm that follows: xw = the new
-    residual times next_norm_w as bfloat16, ss [gemm_emit_layout(M, N, K)] = per-tile sums of squares
-    of each row."""
+    """residual += x @ w.T, and for the RMSNorm that follows: xw = the new residual times next_norm_w as
+    bfloat16, ss [gemm_emit_layout(M, N, K)] = per-tile sums of squares of each row."""
     M, K = x.shape
     N = w.shape[0]
     _gpu("x", x, torch.bfloat16)
@@ -362,14 +364,34 @@ def gemm_accum_emit(x: torch.Tensor, w, residual: torch.Tensor, next_norm_w: tor
     _gpu("residual", residual, torch.float32, (M, N))
     _gpu("next_norm_w", next_norm_w, torch.float32, (N,))
     _gpu("xw", xw, torch.bfloat16, (M, N))
-    if M > EMIT_MAX_ROWS or K % 8:
-        raise KernelError(f"gemm_accum_emit: at most {EMIT_MAX_ROWS} rows, inner size a multiple of 8")
-    _gpu("ss", ss, torch.float32, gemm_emit_layout(M, N, K))
+    layout = gemm_emit_layout(M, N, K) if K % 8 == 0 else None
+    if layout is None:
+        raise KernelError(f"gemm_accum_emit: a product of {M} rows, {N} outputs and inner size {K} cannot leave the next "
+                          f"norm's operand (ask gemm_emit_layout first)")
+    _gpu("ss", ss, torch.float32, layout)
     ws = _gemm_workspace(M, N, K, x.device, emit=True)
     _check(load("gemm_bf16").tuff_gemm_bf16_accum_emit(x.data_ptr(), w.data_ptr(), residual.data_ptr(), M, N, K,
                                                        next_norm_w.data_ptr(), xw.data_ptr(), ss.data_ptr(),
                                                        None if ws is None else ws.data_ptr(), _stream()),
            "gemm_bf16_accum_emit")
+
+
+_scaled_ok: dict = {}
+
+
+def gemm_scaled_supported(M: int, N: int, K: int, out_dtype=torch.bfloat16, accumulate: bool = False) -> bool:
+    """Whether gemm_scaled takes this product: any with at most 64 rows; with more, bfloat16 (or SwiGLU)
+    outputs of products that run in one piece."""
+    if K % 8:
+        return False
+    if M <= EMIT_MAX_ROWS:
+        return True
+    if accumulate or out_dtype != torch.bfloat16:
+        return False
+    key = (M, N, K)
+    if key not in _scaled_ok:
+        _scaled_ok[key] = bool(load("gemm_bf16").tuff_gemm_bf16_scaled_supported(M, N, K))
+    return _scaled_ok[key]
 
 
 def gemm_scaled(xw: torch.Tensor, ss: torch.Tensor, eps: float, w, out: torch.Tensor, *,
@@ -380,9 +402,10 @@ def gemm_scaled(xw: torch.Tensor, ss: torch.Tensor, eps: float, w, out: torch.Te
     M, K = xw.shape
     N = w.shape[0]
     _gpu("xw", xw, torch.bfloat16)
-    if M > EMIT_MAX_ROWS or K % 8:
-        raise KernelError(f"gemm_scaled: at most {EMIT_MAX_ROWS} rows, inner size a multiple of 8")
-    _gpu("ss", ss, torch.float32, (None, 16 if M <= 16 else 64))
+    if not gemm_scaled_supported(M, N, K, out.dtype, accumulate):
+        raise KernelError(f"gemm_scaled: a product of {M} rows, {N} outputs, inner size {K} into {out.dtype} is not "
+                          f"supported (ask gemm_scaled_supported first)")
+    _gpu("ss", ss, torch.float32, (None, 16 if M <= 16 else 64 if M <= EMIT_MAX_ROWS else M))
     w = _tiled(w, N, K)
     mode = _bf16_mode(out, accumulate, swiglu, M, N)
     ws = _gemm_workspace(M, N, K, xw.device)

@@ -105,9 +105,11 @@ class Linear:
         pending = x if isinstance(x, PendingNorm) else None
         if pending is not None:
             T = pending.shape[0]
-            # the row scales left by the product before (any T up to 64), or the norm inside this product
+            # the row scales left by the product before, or the norm inside this product
+            want_out = torch.float32 if accumulate_into is not None else (out_dtype or self.rt.dtype)
             fused = w.dtype == torch.bfloat16 and self.in_features % 8 == 0 and (
-                T <= ops.EMIT_MAX_ROWS if pending.pre is not None
+                ops.gemm_scaled_supported(T, self.out_features, self.in_features, want_out, accumulate_into is not None)
+                if pending.pre is not None
                 else T <= ops.NORMED_MAX_ROWS and self.in_features <= ops.NORMED_MAX_K)
             if not fused:
                 x, pending = pending.tensor(), None
@@ -134,11 +136,14 @@ class Linear:
         dev = w.device
         if accumulate_into is not None:
             nxt = next_norm
+            layout = None
             if (nxt is not None and pending is None and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
-                    and T <= ops.EMIT_MAX_ROWS):
+                    and self.in_features % 8 == 0):
+                layout = ops.gemm_emit_layout(T, self.out_features, self.in_features)
+            if layout is not None:
                 # the norm that follows reads the sum just made: leave it its operand and row sums
                 xw = torch.empty(T, self.out_features, dtype=torch.bfloat16, device=dev)
-                ss = torch.empty(ops.gemm_emit_layout(T, self.out_features, self.in_features), dtype=torch.float32, device=dev)
+                ss = torch.empty(layout, dtype=torch.float32, device=dev)
                 ops.gemm_accum_emit(x, w, accumulate_into, nxt.weight_f32, xw, ss)
                 nxt.announce_operand(accumulate_into, xw, ss)
                 return None
