@@ -325,7 +325,7 @@ def main() -> int:
 
     head = decode_point(args.batch, args.steps, args.warmup, SEED)
     out = {
-        "metric": "decode tok/s at batch 8, context 8192 (LFM2.5-1.2B shape)", "value": round(head["tok_s"], 1),
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} (LFM2.5-1.2B shape)", "value": round(head["tok_s"], 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(head["ms"], 4),
         "runs": args.runs, "spread": round(head["spread"], 1),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,

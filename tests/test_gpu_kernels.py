@@ -660,6 +660,49 @@ def test_attention_of_single_tokens_is_the_same_with_one_wave_or_four_a_partitio
         assert torch.isfinite(many).all() and torch.equal(few, many[:3]), f"fused={fused}"
 
 
+@pytest.mark.parametrize("H,Hkv", [(32, 8), (6, 3), (5, 5), (16, 1)])
+def test_attention_of_single_tokens_does_not_depend_on_the_order_of_its_workgroups(gpu, H, Hkv):
+    """Large launches number their workgroups with the kv head changing fastest, small ones with the
+    partition: the same bits either way (forced both ways here), fused and not."""
+    import ctypes
+    from tuff_amd.csrc import ops
+    hd, ps = 64, 16
+    lens = [700, 1, 257, 256, 33, 1025, 64]
+    R = len(lens)
+    inv_freq = (1e6 ** (-2 * torch.arange(hd // 2, dtype=torch.float64) / hd)).float().to(gpu)
+    qw = (1 + _r(hd, seed=5, scale=0.1)).to(gpu)
+    lib = ops.load("attention_mfma")
+    lib.tuff_attention_kv_fast_waves.argtypes = [ctypes.c_int]
+    lib.tuff_attention_kv_fast_waves.restype = ctypes.c_int
+
+    def run(fused):
+        c = _decode_case(gpu, R, H, Hkv, ps, lens)
+        common = dict(block_table=c["table"], req_info=c["req_info"], positions=c["positions"], H=H, Hkv=Hkv,
+                      page_size=ps, max_ctx_len=c["max_ctx_len"])
+        out = torch.full((R, H * hd), float("nan"), dtype=torch.bfloat16, device=gpu)
+        if fused:
+            ops.attention_decode_fused(c["qkv"], c["kc"], c["vc"], out, inv_freq=inv_freq, slot_mapping=c["slots"],
+                                       q_norm_w=qw, k_norm_w=qw, eps=1e-5, **common)
+        else:
+            c["kc"].nan_to_num_(0.0); c["vc"].nan_to_num_(0.0)             # the step's own key is not written here
+            ops.attention_mfma(c["qkv"][:, :H * hd].contiguous(), c["kc"], c["vc"], out, blocks=None, nb=1, hd=hd, **common)
+        torch.cuda.synchronize()
+        return out.float().cpu(), c["kc"].float().cpu()
+
+    before = lib.tuff_attention_kv_fast_waves(-1)
+    try:
+        for fused in (False, True):
+            lib.tuff_attention_kv_fast_waves(1 << 30)
+            o_part, k_part = run(fused)
+            lib.tuff_attention_kv_fast_waves(0)
+            o_kv, k_kv = run(fused)
+            assert torch.isfinite(o_part).all()
+            assert torch.equal(o_part, o_kv), f"fused={fused}"
+            assert torch.equal(torch.nan_to_num(k_part, nan=1e9), torch.nan_to_num(k_kv, nan=1e9))
+    finally:
+        lib.tuff_attention_kv_fast_waves(before)
+
+
 @pytest.mark.parametrize("H,Hkv,hd,ps", [(4, 2, 16, 16), (4, 1, 24, 16), (3, 3, 80, 16), (2, 1, 256, 32),
                                           (32, 8, 64, 16), (8, 2, 128, 64), (32, 1, 64, 16), (5, 5, 40, 48),
                                           (6, 2, 96, 80)])

@@ -96,12 +96,15 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
     float* __restrict__ ws_o, float* __restrict__ ws_ml,
     const int* __restrict__ block_table, int max_blocks,
     const int2* __restrict__ blk, const int4* __restrict__ req_info,
-    int H, int Hkv, int hd, int page_size, int window, float scale, int n_parts, FusedQKV fq) {
+    int H, int Hkv, int hd, int page_size, int window, float scale, int n_parts, FusedQKV fq, int kv_fast) {
     static_assert(NW == 1 || NW == UNITS, "one wave a partition or one a unit");
     static_assert(!FUSED || (HDP == 64 && NB == 1), "the fused form is for heads of 64 and one column block");
     constexpr int KC = HDP / 32;          // 32-wide chunks of the head dimension
     constexpr int DB = HDP / 16;          // 16-wide blocks of output channels
-    const int part = blockIdx.x, qb = blockIdx.y, kvh = blockIdx.z;
+    // Workgroups that run side by side read neighbouring memory when the kv head is what changes fastest
+    // from one to the next (a page holds its kv heads one after the other): that order for launches of
+    // several rounds of waves, partitions first for the others.
+    const int part = kv_fast ? blockIdx.x / Hkv : blockIdx.x, qb = blockIdx.y, kvh = kv_fast ? blockIdx.x % Hkv : blockIdx.z;
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n16 = lane % 16, g = lane / 16;
     const int G = H / Hkv;
     // Every load that depends on another costs a trip to memory, so the chain is kept short:
@@ -640,22 +643,28 @@ __global__ __launch_bounds__(COMBINE_WAVES * WAVE) void attn_combine_kernel(cons
 // Workgroups of four waves where one wave a partition would leave most of the chip idle (a step of a
 // few single tokens); the result is the same bit for bit.
 int few_waves = 2048;
+// From how many workgroups on the kv head is the fastest-changing part of a workgroup's number: with
+// several rounds of waves on the chip (it holds about 3,000 of them) that is 7 to 11 % faster, with one
+// round it is not.
+int kv_fast_waves = 6144;
 
 template <int HDP, int NB, bool FUSED>
 void launch_partition(dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* kc, bf16_t* vc, float* ws_o,
                       float* ws_ml, const int* bt, int max_blocks, const int2* blk, const int4* req_info,
                       int H, int Hkv, int hd, int ps, int window, float scale, int n_parts, const FusedQKV& fq) {
     const long long waves = (long long)grid.x * grid.y * grid.z;
+    const int kv_fast = waves >= kv_fast_waves ? 1 : 0;
+    if (kv_fast) grid = dim3(grid.x * grid.z, grid.y, 1);
     if constexpr (HDP * NB <= 128) {
         // the fused form prepares its queries in every wave: four waves pay for that four times
         if (waves < (FUSED ? few_waves / 2 : few_waves)) {
             hipLaunchKernelGGL((attn_partition_kernel<HDP, NB, UNITS, FUSED>), grid, dim3(UNITS * WAVE), 0, stream, q, kc, vc, ws_o,
-                               ws_ml, bt, max_blocks, blk, req_info, H, Hkv, hd, ps, window, scale, n_parts, fq);
+                               ws_ml, bt, max_blocks, blk, req_info, H, Hkv, hd, ps, window, scale, n_parts, fq, kv_fast);
             return;
         }
     }
     hipLaunchKernelGGL((attn_partition_kernel<HDP, NB, 1, FUSED>), grid, dim3(WAVE), 0, stream, q, kc, vc, ws_o, ws_ml, bt,
-                       max_blocks, blk, req_info, H, Hkv, hd, ps, window, scale, n_parts, fq);
+                       max_blocks, blk, req_info, H, Hkv, hd, ps, window, scale, n_parts, fq, kv_fast);
 }
 }  // namespace
 
@@ -718,6 +727,14 @@ static int launch_attention(const void* q, const void* k_cache, const void* v_ca
 TUFF_EXPORT int tuff_attention_few_waves(int n) {
     const int old = few_waves;
     if (n >= 0) few_waves = n;
+    return old;
+}
+
+// From how many workgroups on the kv head changes fastest in the order of the workgroups.  For
+// measurements and tests; the result does not depend on it.  Returns the value before.
+TUFF_EXPORT int tuff_attention_kv_fast_waves(int n) {
+    const int old = kv_fast_waves;
+    if (n >= 0) kv_fast_waves = n;
     return old;
 }
 
