@@ -727,6 +727,18 @@ def test_attention_prefill(gpu, H, Hkv, hd, ps, window):
 
     reqs = [(699, 1), (230, 150), (0, 333), (0, 1), (255, 3), (1100, 70)]
     case, got = run(reqs)
+    # the blocks listed with the most keys first, as the attention part lists them: the same bits
+    T = case["q"].shape[0]
+    ctx_len = [past + n for past, n in reqs]
+    sorted_blocks = ops.query_blocks(case["q_len"], H // Hkv, cols // 16, ctx_len)
+    plain_blocks = ops.query_blocks(case["q_len"], H // Hkv, cols // 16)
+    assert sorted(map(tuple, sorted_blocks.tolist())) == sorted(map(tuple, plain_blocks.tolist()))
+    assert sorted_blocks[0].tolist() == [5, (70 * (H // Hkv) - 1) // cols * cols]      # the last block of the request at 1,170
+    out = torch.full((T, H * hd), float("nan"), dtype=torch.bfloat16, device=gpu)
+    ops.attention_prefill(case["q"].to(gpu), case["kc"], case["vc"], out, block_table=case["table"],
+                          blocks=torch.from_numpy(sorted_blocks).to(gpu), req_info=case["req_info"], H=H, Hkv=Hkv, hd=hd,
+                          page_size=ps, max_ctx_len=case["max_ctx_len"], window=window)
+    assert torch.equal(out.cpu().double().reshape(T, H, hd), got), "the result depends on the order of the blocks"
     # tokens 70..149 of request 1 (positions 300..379) again, as a step of their own that starts
     # at position 300: bit for bit the same
     first = sum(n for _, n in reqs[:1]) + 70

@@ -62,8 +62,11 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     bf16_t* Vs = lds + 2 * KBUF;          // [2][VBUF]
 
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE, n16 = lane % 16, g = lane / 16;
-    const int qb = gridDim.x - 1 - blockIdx.x;      // late blocks have the most keys: start them first
-    const int kvh = blockIdx.y;
+    // Workgroups are numbered with the kv head changing fastest: the eight XCDs take the numbers in
+    // turn, so with eight kv heads an XCD's L2 holds one head's keys and values.  The host lists the
+    // blocks with the most keys first, so that the long ones start first and the short ones fill in.
+    const int qb = blockIdx.x / Hkv;
+    const int kvh = blockIdx.x % Hkv;
     const int G = H / Hkv;
     int r = qb, col0 = 0;
     if (blk) { const int2 b = blk[qb]; r = b.x; col0 = b.y; }
@@ -145,14 +148,18 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     // ---- copies: what this thread moves each step.  Memory answers later than a step lasts, so
     // the keys and values of AHEAD steps are on their way at any time, each in a register set.
     // Per piece the thread keeps what does not change from step to step: the granule (16 keys, one
-    // page) it lies in, its offset inside the granule's rows, and where it goes in LDS.
+    // page) it lies in, its offset inside the granule's rows, and where it goes in LDS.  The pieces
+    // are dealt so that the 64 of a wave lie in one granule: where the granule's rows start in the
+    // caches is then scalar arithmetic, once a piece and wave, not a choice among four addresses in
+    // every lane.
     bf16x8 kreg[AHEAD][KPT], vreg[AHEAD][VPT];
     int k_gran[KPT], k_key[KPT], k_off[KPT], k_lds[KPT], v_gran[VPT], v_key[VPT], v_off[VPT], v_lds[VPT];
     bool k_ok[KPT], v_ok[VPT];
+    static_assert((16 * HC) % WAVE == 0 && (2 * HDP) % WAVE == 0 && NT % WAVE == 0, "a wave's pieces lie in one granule");
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
         const int id = tid + i * NT, key = id / HC, c = id % HC;
-        k_gran[i] = key / 16;
+        k_gran[i] = __builtin_amdgcn_readfirstlane(key / 16);
         k_key[i] = key;
         k_off[i] = (key % 16) * hd + c * 8;
         k_ok[i] = c * 8 < hd;
@@ -160,60 +167,70 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     }
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-        const int id = tid + i * NT, dim = id / 8, c8 = id % 8;
-        v_gran[i] = c8 / 2;
+        const int id = tid + i * NT, c8 = id / HDP, dim = id % HDP;      // lanes run over the channels
+        v_gran[i] = __builtin_amdgcn_readfirstlane(c8 / 2);
         v_key[i] = c8 * 8;
         v_off[i] = dim * page_size + (c8 % 2) * 8;
         v_ok[i] = dim < hd;
         v_lds[i] = dim * VROW + c8 * 8;
     }
     const bool whole_rows = hd == HDP;
+    const long long page_stride = (long long)Hkv * page_size * hd;       // elements of a page in either cache
+    const long long head_off = (long long)kvh * page_size * hd;          // this kv head's share of it
     int ld_off = key_start % page_size;                 // offset in its page of the first key of the next step to load
-    auto pick = [](int gsel, long long b0, long long b1, long long b2, long long b3) {
-        return gsel == 0 ? b0 : gsel == 1 ? b1 : gsel == 2 ? b2 : b3;
-    };
     auto load_step = [&](int set, int s, int pages) {   // step s of the block -> register set; zeros beyond pos_max
         const int key0 = key_start + s * STEP;
         const int gslot0 = (s % 16) * 4;                // granule of the step's first key within `pages`
-        // per granule, the same for all threads: where its rows start in both caches
-        long long bk[4], bv[4];
-        bool all_live = key0 + STEP - 1 <= pos_max;
-        int go = ld_off;
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
+        // per piece, the same for the lanes of a wave: where its granule's rows start (-1: no such page)
+        auto granule = [&](int g4, long long& base, int& go) {
             const int page = __builtin_amdgcn_readlane(pages, gslot0 + g4);
-            all_live = all_live && page >= 0;
-            const long long head = (long long)max(page, 0) * Hkv + kvh;
-            bk[g4] = page >= 0 ? (head * page_size + go) * hd : -1;
-            bv[g4] = head * hd * page_size + go;
-            go += 16;
-            if (go >= page_size) go -= page_size;
+            go = ld_off + 16 * g4;
+#pragma unroll
+            for (int w = 0; w < 3; ++w)
+                if (go >= page_size) go -= page_size;
+            base = page >= 0 ? page * page_stride + head_off : -1;
+        };
+        long long bk[KPT], bv[VPT];
+        bool all_live = key0 + STEP - 1 <= pos_max;
+#pragma unroll
+        for (int i = 0; i < KPT; ++i) {
+            int go;
+            granule(k_gran[i], bk[i], go);
+            all_live = all_live && bk[i] >= 0;
+            bk[i] += (long long)go * hd;                // (-1 stays negative: go * hd < page_stride)
         }
-        ld_off = go;
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+            int go;
+            granule(v_gran[i], bv[i], go);
+            all_live = all_live && bv[i] >= 0;
+            bv[i] += go;
+        }
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            ld_off += 16;
+            if (ld_off >= page_size) ld_off -= page_size;
+        }
         if (all_live && whole_rows) {
 #pragma unroll
-            for (int i = 0; i < KPT; ++i)
-                kreg[set][i] = *(const bf16x8*)(k_cache + pick(k_gran[i], bk[0], bk[1], bk[2], bk[3]) + k_off[i]);
+            for (int i = 0; i < KPT; ++i) kreg[set][i] = *(const bf16x8*)(k_cache + bk[i] + k_off[i]);
 #pragma unroll
-            for (int i = 0; i < VPT; ++i)
-                vreg[set][i] = *(const bf16x8*)(v_cache + pick(v_gran[i], bv[0], bv[1], bv[2], bv[3]) + v_off[i]);
+            for (int i = 0; i < VPT; ++i) vreg[set][i] = *(const bf16x8*)(v_cache + bv[i] + v_off[i]);
             return;
         }
         // first steps under a window, the last step, narrow heads: pieces that do not exist read as zero
         const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int i = 0; i < KPT; ++i) {
-            const long long base = pick(k_gran[i], bk[0], bk[1], bk[2], bk[3]);
-            const bool live = base >= 0 && key0 + k_key[i] <= pos_max && k_ok[i];
-            const bf16x8 v = *(const bf16x8*)(k_cache + (live ? base + k_off[i] : 0));
+            const bool live = bk[i] >= 0 && key0 + k_key[i] <= pos_max && k_ok[i];
+            const bf16x8 v = *(const bf16x8*)(k_cache + (live ? bk[i] + k_off[i] : 0));
             kreg[set][i] = live ? v : z;
         }
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
-            const long long base = pick(v_gran[i], bv[0], bv[1], bv[2], bv[3]);
             const int kabs = key0 + v_key[i];
-            const bool live = pick(v_gran[i], bk[0], bk[1], bk[2], bk[3]) >= 0 && kabs <= pos_max && v_ok[i];
-            bf16x8 v = *(const bf16x8*)(v_cache + (live ? base + v_off[i] : 0));
+            const bool live = bv[i] >= 0 && kabs <= pos_max && v_ok[i];
+            bf16x8 v = *(const bf16x8*)(v_cache + (live ? bv[i] + v_off[i] : 0));
             v = live ? v : z;
 #pragma unroll
             for (int e = 0; e < 8; ++e)                  // positions beyond the last were never written
@@ -400,8 +417,8 @@ int launch(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, con
 // Columns a block of the list must hold for this head size.
 TUFF_EXPORT int tuff_attention_prefill_block_columns(int hd) { return hd <= 128 ? 128 : 64; }
 
-// Query blocks are listed by the host: block b holds the columns blk[b].y .. + block_columns - 1
-// of request blk[b].x (a request's columns are numbered (token - its first token) * G + head
+// Query blocks are listed by the host, best those with the most keys first: block b holds the columns
+// blk[b].y .. + block_columns - 1 of request blk[b].x (a request's columns are numbered (token - its first token) * G + head
 // within the kv group); blk == null: block b is request b from column 0.
 // req_info [R]: (first token of the request in the step, its tokens, position of the first, -).
 // n_segs > 1: the keys are cut into segments of seg_keys (a multiple of 64) and `out` is not written:
@@ -421,7 +438,8 @@ TUFF_EXPORT int tuff_attention_prefill(const void* q, const void* k_cache, const
     const bf16_t* Q = (const bf16_t*)q;
     const bf16_t* K = (const bf16_t*)k_cache;
     const bf16_t* V = (const bf16_t*)v_cache;
-    dim3 grid(n_qblocks, Hkv, n_segs);
+    if ((long long)n_qblocks * Hkv > 0x7fffffffll) return -2;
+    dim3 grid(n_qblocks * Hkv, 1, n_segs);
     const float sl = scale * 1.4426950408889634f;
 #define GO(HDP, NBW, AHEAD) return launch<HDP, NBW, AHEAD>(grid, stream, Q, K, V, (bf16_t*)out, block_table, max_blocks, (const int2*)blk, \
                                              (const int4*)req_info, H, Hkv, hd, page_size, window, sl, seg_keys, ws_o, ws_ml)

@@ -751,16 +751,25 @@ def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info
                "attention_merge")
 
 
-def query_blocks(q_len, G: int, nb: int):
-    """Host list of query blocks for attention_mfma: for request r with q_len[r] tokens the
-    columns (token, head in group) are cut into blocks of 16 * nb.  Returns int32 [n_blocks, 2]
-    = (request, first column)."""
+def query_blocks(q_len, G: int, nb: int, ctx_len=None):
+    """Host list of query blocks for attention_mfma and attention_prefill: for request r with q_len[r]
+    tokens the columns (token, head in group) are cut into blocks of 16 * nb.  Returns int32
+    [n_blocks, 2] = (request, first column).  With ctx_len (tokens of each request in the cache after
+    the step) the blocks whose last column sees the most keys come first (attention_prefill starts
+    its workgroups in the list's order, and the longest should not start last); the order has no
+    influence on any result."""
     import numpy as np
     q_len = np.asarray(q_len, dtype=np.int64)
     per = -(-(q_len * G) // (16 * nb))
     blk_req = np.repeat(np.arange(len(q_len)), per)
     starts = np.concatenate([[0], np.cumsum(per)])[:-1]
     blk_col0 = (np.arange(int(per.sum())) - np.repeat(starts, per)) * 16 * nb
+    if ctx_len is not None and len(blk_req):
+        ctx_len = np.asarray(ctx_len, dtype=np.int64)
+        last_tok = np.minimum(q_len[blk_req] - 1, (blk_col0 + 16 * nb - 1) // G)
+        keys = ctx_len[blk_req] - q_len[blk_req] + last_tok + 1
+        order = np.argsort(-keys, kind="stable")
+        blk_req, blk_col0 = blk_req[order], blk_col0[order]
     return np.stack([blk_req, blk_col0], axis=1).astype(np.int32)
 
 

@@ -139,14 +139,15 @@ class AttentionMixer(Mixer):
         return torch.from_numpy(array).pin_memory().to(device, non_blocking=True)
 
     @classmethod
-    def _blocks(cls, ctx, G, nb, device, skip_single: bool = False):
-        key = ("query_blocks", G, nb, skip_single)
+    def _blocks(cls, ctx, G, nb, device, skip_single: bool = False, longest_first: bool = False):
+        key = ("query_blocks", G, nb, skip_single, longest_first)
         blocks = ctx.host.get(key)
         if blocks is None:
             q_len = ctx.host["q_len"]
             if skip_single:
                 q_len = np.where(q_len == 1, 0, q_len)
-            blocks = ctx.host[key] = cls._upload(ops.query_blocks(q_len, G, nb), device)
+            ctx_len = ctx.host["ctx_len"] if longest_first else None
+            blocks = ctx.host[key] = cls._upload(ops.query_blocks(q_len, G, nb, ctx_len), device)
         return blocks
 
     @classmethod
@@ -186,7 +187,7 @@ class AttentionMixer(Mixer):
                 nb = ops.attention_prefill_block_columns(self.hd) // 16
                 runs = self._single_token_runs(ctx, G, q.device)
                 # (first: with key segments it writes every row of o, the single tokens' rows come after)
-                ops.attention_prefill(q, cache.k, cache.v, o, blocks=self._blocks(ctx, G, nb, q.device, skip_single=bool(runs)),
+                ops.attention_prefill(q, cache.k, cache.v, o, blocks=self._blocks(ctx, G, nb, q.device, skip_single=bool(runs), longest_first=True),
                                       positions=ctx.positions, **common)
                 for tok_lo, n, blocks, info, ctx_len in runs:
                     ops.attention_mfma(q[tok_lo:tok_lo + n], cache.k, cache.v, o[tok_lo:tok_lo + n], blocks=blocks, nb=1,
