@@ -951,9 +951,8 @@ def test_shortconv(gpu, d, K, dt):
         out = torch.empty(bcx.shape[0], d, dtype=dt, device=gpu)
         meta = dict(q_start=torch.tensor(q_start, dtype=torch.int32, device=gpu),
                     state_slot=torch.tensor([[2, 0][r] for r in who], dtype=torch.int32, device=gpu))
-        ops.shortconv_fwd(bcx, w.to(gpu), state, out, req_of_token=torch.tensor(req_of, dtype=torch.int32, device=gpu),
-                          K=K, **meta)
-        ops.shortconv_state(bcx, state, q_len=torch.tensor(q_len, dtype=torch.int32, device=gpu), K=K, **meta)
+        _conv_both_ways(ops, bcx, w.to(gpu), state, out, req_of_token=torch.tensor(req_of, dtype=torch.int32, device=gpu),
+                        q_len=torch.tensor(q_len, dtype=torch.int32, device=gpu), K=K, **meta)
         for i, r in enumerate(who):
             outs[r].append(out[q_start[i]:q_start[i] + q_len[i]].cpu())
     for r in range(2):
@@ -963,6 +962,18 @@ def test_shortconv(gpu, d, K, dt):
         assert (got - want).abs().max() <= tol * float(want.abs().max())
         assert (state[int(slots[r])].cpu().double() - want_state).abs().max() <= 1e-6
     assert (state[1] == 0).all() and (state[3] == 0).all()       # other requests' slots untouched
+
+
+def _conv_both_ways(ops, bcx, w, state, out, *, req_of_token, q_start, q_len, state_slot, K):
+    """The kernel that only reads the state followed by the one that rewrites it, and the kernel that
+    does both (the one the mixer runs): the same output and the same state, bit for bit.  Leaves the
+    result in `state` and `out`."""
+    state2, out2 = state.clone(), torch.full_like(out, float("nan"))
+    ops.shortconv_fwd(bcx, w, state, out, req_of_token=req_of_token, q_start=q_start, state_slot=state_slot, K=K)
+    ops.shortconv_state(bcx, state, q_start=q_start, q_len=q_len, state_slot=state_slot, K=K)
+    ops.shortconv_fwd(bcx, w, state2, out2, req_of_token=req_of_token, q_start=q_start, state_slot=state_slot, K=K, q_len=q_len)
+    assert torch.equal(out, out2), "output of the kernel that also rewrites the state"
+    assert torch.equal(state, state2), "state of the kernel that also rewrites the state"
 
 
 @pytest.mark.parametrize("d,K", [(64, 3), (96, 4), (240, 2), (300, 7)])
@@ -980,8 +991,7 @@ def test_shortconv_single_token_kernel_equals_the_general_pair(gpu, d, K, dt):
         bcx = _r(R, 3 * d, seed=30 + step, dtype=dt).to(gpu)
         o1 = torch.empty(R, d, dtype=dt, device=gpu)
         o2 = torch.empty(R, d, dtype=dt, device=gpu)
-        ops.shortconv_fwd(bcx, w, s1, o1, req_of_token=ar, q_start=ar, state_slot=slots, K=K)
-        ops.shortconv_state(bcx, s1, q_start=ar, q_len=ones, state_slot=slots, K=K)
+        _conv_both_ways(ops, bcx, w, s1, o1, req_of_token=ar, q_start=ar, q_len=ones, state_slot=slots, K=K)
         ops.shortconv_decode(bcx, w, s2, o2, state_slot=slots, K=K)
         assert torch.equal(o1, o2) and torch.equal(s1, s2), step
 
@@ -1016,8 +1026,8 @@ def test_shortconv_long_portions_equal_single_tokens(gpu, d, K):
         bcx = torch.cat([bcx_all[r][done[r]:done[r] + n] for r, n in zip(who, q_len)])
         out = torch.empty(bcx.shape[0], d, dtype=dt, device=gpu)
         meta = dict(q_start=i32(q_start), state_slot=i32([slots[r] for r in who]))
-        ops.shortconv_fwd(bcx, w, s2, out, req_of_token=i32([i for i, n in enumerate(q_len) for _ in range(n)]), K=K, **meta)
-        ops.shortconv_state(bcx, s2, q_len=i32(q_len), K=K, **meta)
+        _conv_both_ways(ops, bcx, w, s2, out, req_of_token=i32([i for i, n in enumerate(q_len) for _ in range(n)]),
+                        q_len=i32(q_len), K=K, **meta)
         for i, r in enumerate(who):
             got[r].append(out[q_start[i]:q_start[i] + q_len[i]])
             done[r] += q_len[i]

@@ -116,12 +116,19 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         }
     }
 
-    float m_run[NBW], l_run[NBW];
+    // The sums of the weights come out of the matrix cores too: V^T is given one more block of rows
+    // whose first row is all ones, so row 0 of that block of O^T is the sum of a column's weights (as
+    // they are multiplied: rounded to bfloat16, summed in float32), in the lanes of group 0.
+    float m_run[NBW];
+    f32x4 l_acc[NBW];
+    bf16x8 ones;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ones[e] = (bf16_t)(n16 == 0 ? 1.f : 0.f);
     f32x4 o[DB][NBW];
 #pragma unroll
     for (int nb = 0; nb < NBW; ++nb) {
         m_run[nb] = -INFINITY;
-        l_run[nb] = 0.f;
+        l_acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int db = 0; db < DB; ++db) o[db][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -175,8 +182,9 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         v_lds[i] = dim * VROW + c8 * 8;
     }
     const bool whole_rows = hd == HDP;
-    const long long page_stride = (long long)Hkv * page_size * hd;       // elements of a page in either cache
-    const long long head_off = (long long)kvh * page_size * hd;          // this kv head's share of it
+    const unsigned page_stride = (unsigned)(Hkv * page_size * hd);       // elements of a page in either cache (the host checks that it fits)
+    const unsigned head_off = (unsigned)(kvh * page_size * hd);          // this kv head's share of it
+    const int ps_mask = (page_size & (page_size - 1)) == 0 ? page_size - 1 : 0;   // a power of two: offsets wrap by a mask
     int ld_off = key_start % page_size;                 // offset in its page of the first key of the next step to load
     auto load_step = [&](int set, int s, int pages) {   // step s of the block -> register set; zeros beyond pos_max
         const int key0 = key_start + s * STEP;
@@ -185,10 +193,13 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         auto granule = [&](int g4, long long& base, int& go) {
             const int page = __builtin_amdgcn_readlane(pages, gslot0 + g4);
             go = ld_off + 16 * g4;
+            if (ps_mask) go &= ps_mask;
+            else {
 #pragma unroll
-            for (int w = 0; w < 3; ++w)
-                if (go >= page_size) go -= page_size;
-            base = page >= 0 ? page * page_stride + head_off : -1;
+                for (int w = 0; w < 3; ++w)
+                    if (go >= page_size) go -= page_size;
+            }
+            base = page >= 0 ? (long long)((unsigned long long)(unsigned)page * page_stride + head_off) : -1;
         };
         long long bk[KPT], bv[VPT];
         bool all_live = key0 + STEP - 1 <= pos_max;
@@ -206,10 +217,13 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
             all_live = all_live && bv[i] >= 0;
             bv[i] += go;
         }
+        if (ps_mask) ld_off = (ld_off + STEP) & ps_mask;
+        else {
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            ld_off += 16;
-            if (ld_off >= page_size) ld_off -= page_size;
+            for (int w = 0; w < 4; ++w) {
+                ld_off += 16;
+                if (ld_off >= page_size) ld_off -= page_size;
+            }
         }
         if (all_live && whole_rows) {
 #pragma unroll
@@ -306,16 +320,13 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
             const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
             corr[nb] = __builtin_amdgcn_exp2f(m_run[nb] - m_safe);           // 0 while nothing was seen yet
             same = same && (m_new == m_run[nb]);
-            float sum = 0.f;
 #pragma unroll
             for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const float p = ok[sub][i] ? __builtin_amdgcn_exp2f(fmaf(sc[sub].v[i / 4][nb][i % 4], scale_log2e, -m_safe)) : 0.f;
-                    sum += p;
                     pf[sub][nb][i] = (bf16_t)p;
                 }
-            l_run[nb] = fmaf(l_run[nb], corr[nb], sum);
             m_run[nb] = m_new;
         }
         if (!__all(same)) {                                  // rare; corr is exactly 1 where the reference stayed
@@ -326,6 +337,8 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
                 for (int nb = 0; nb < NBW; ++nb)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) o[db][nb][e] *= corr[nb];
+#pragma unroll
+            for (int nb = 0; nb < NBW; ++nb) l_acc[nb][0] *= corr[nb];
         }
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub) {
@@ -336,6 +349,8 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
 #pragma unroll
                 for (int nb = 0; nb < NBW; ++nb) o[db][nb] = mfma32(vf, pf[sub][nb], o[db][nb]);
             }
+#pragma unroll
+            for (int nb = 0; nb < NBW; ++nb) l_acc[nb] = mfma32(ones, pf[sub][nb], l_acc[nb]);
         }
     };
 
@@ -369,9 +384,7 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     // ---- normalise and write
 #pragma unroll
     for (int nb = 0; nb < NBW; ++nb) {
-        float l = l_run[nb];
-        l += __shfl_xor(l, 16, WAVE);
-        l += __shfl_xor(l, 32, WAVE);
+        const float l = __shfl(l_acc[nb][0], n16, WAVE);       // from the lane of group 0 that holds the column's sum
         if (qrow[nb] < 0) continue;
         if (n_segs > 1) {
             const long long slot = qrow[nb] * n_segs + seg;
@@ -434,6 +447,7 @@ TUFF_EXPORT int tuff_attention_prefill(const void* q, const void* k_cache, const
     if (hd > 256 || hd % 8 != 0 || page_size % 16 != 0 || Hkv <= 0 || H % Hkv != 0) return -2;
     if (Hkv > 65535 || !(scale > 0.f)) return -2;
     if (n_segs < 1 || n_segs > 65535) return -2;
+    if ((long long)Hkv * page_size * hd > 0x7fffffffll) return -2;
     if (n_segs > 1 && (seg_keys <= 0 || seg_keys % STEP != 0 || !ws_o || !ws_ml)) return -2;
     const bf16_t* Q = (const bf16_t*)q;
     const bf16_t* K = (const bf16_t*)k_cache;

@@ -86,7 +86,7 @@ _SIGNATURES = {
     },
     "shortconv": {
         "tuff_shortconv_fwd": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
-                               _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+                               _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_shortconv_decode": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p,
                                   _c_int, _c_int, _c_int, _c_void_p],
         "tuff_shortconv_state": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
@@ -774,7 +774,10 @@ def query_blocks(q_len, G: int, nb: int, ctx_len=None):
 
 
 # ------------------------------------------------------------------------- short conv
-def shortconv_fwd(bcx, conv_w, state, out, *, req_of_token, q_start, state_slot, K) -> None:
+def shortconv_fwd(bcx, conv_w, state, out, *, req_of_token, q_start, state_slot, K, q_len=None) -> None:
+    """The gated short convolution of a step's tokens, each request's earlier values from its state slot.
+    With q_len (int32 [requests]) the state of every request with tokens in the step is rewritten too,
+    as shortconv_state would afterwards; without, the state is only read."""
     T, d = out.shape
     dt = out.dtype
     _gpu("bcx", bcx, dt, (T, 3 * d))
@@ -785,9 +788,12 @@ def shortconv_fwd(bcx, conv_w, state, out, *, req_of_token, q_start, state_slot,
     _gpu("req_of_token", req_of_token, torch.int32, (T,))
     _gpu("q_start", q_start, torch.int32, (R,))
     _gpu("state_slot", state_slot, torch.int32, (R,))
+    if q_len is not None:
+        _gpu("q_len", q_len, torch.int32, (R,))
     _check(load("shortconv").tuff_shortconv_fwd(
         bcx.data_ptr(), conv_w.data_ptr(), _dt(conv_w), state.data_ptr(), out.data_ptr(), _dt(out),
-        req_of_token.data_ptr(), q_start.data_ptr(), state_slot.data_ptr(), T, d, K, _stream()), "shortconv_fwd")
+        req_of_token.data_ptr(), q_start.data_ptr(), None if q_len is None else q_len.data_ptr(), state_slot.data_ptr(),
+        T, d, K, _stream()), "shortconv_fwd")
 
 
 def shortconv_decode(bcx, conv_w, state, out, *, state_slot, K) -> None:

@@ -309,6 +309,15 @@ __global__ __launch_bounds__(WAVE) void kv_write_kernel(const T* __restrict__ k,
 // norm weights.  Null q_norm_w / k_norm_w: no norm.  Null inv_freq: no rotation.
 // Null k_cache: nothing is written to the cache (then only the H query heads and, if
 // k_out is given, the key heads are processed).
+// How many (token, share of its heads) items the kernel for heads of 64 wants at least: a token's heads
+// are dealt to more sixteen-lane groups until there are that many.  For measurements; no result depends on it.
+static int post64_items = 8192;
+TUFF_EXPORT int tuff_qkv_post64_items(int n) {
+    const int old = post64_items;
+    if (n > 0) post64_items = n;
+    return old;
+}
+
 TUFF_EXPORT int tuff_qkv_post(const void* qkv, void* q_out, void* k_out, void* k_cache, void* v_cache, int dt,
                               const void* q_norm_w, const void* k_norm_w, int norm_dt, float eps,
                               const float* inv_freq, int rotary_dim, int interleaved,
@@ -322,7 +331,8 @@ TUFF_EXPORT int tuff_qkv_post(const void* qkv, void* q_out, void* k_out, void* k
         // shares of a token's heads: enough sixteen-lane groups for the chip, whole heads each
         const int n_heads = k_cache ? H + Hkv : H;
         int shares = 1;
-        while (shares < n_heads && (long long)n_tokens * shares < 8192) shares *= 2;
+        const long long items = n_tokens >= 1024 ? 2ll * post64_items : post64_items;   // measured: 2,048 tokens 12.1 -> 10.5 us
+        while (shares < n_heads && (long long)n_tokens * shares < items) shares *= 2;
         shares = min(shares, n_heads);
         const int qk_blocks = (int)ceil_div_ll((long long)n_tokens * shares, P64_GROUPS);
         const int v_blocks = k_cache ? ceil_div(n_tokens, P64_TOKENS) * Hkv : 0;

@@ -13,25 +13,21 @@
 // same chain of operations wherever the portion was cut.  The state holds u in float32
 // (a product of two bfloat16 values is exact in float32).
 //
-// The forward kernel only reads the state; a second kernel, launched after it on the
-// same stream, rewrites each (slot, channel) column from registers.
+// The forward kernel comes in two forms.  Reading only: every token is a thread's own, and a second
+// kernel (shortconv_state), launched after it on the same stream, rewrites each (slot, channel) column.
+// Updating: the thread of a request's first token also computes the other tokens that read the old
+// state (the first K-1 of the portion) and then writes the new state, rows in ascending order; no
+// other thread touches that column of the state, so nothing races and no second kernel is needed.
 #include "common.h"
 
 namespace {
 constexpr int MAX_TAPS = 16;
 
+// Token i of its request's portion (row t = t0 + i of the step), channel c.
 template <typename T, typename TW>
-__global__ void shortconv_fwd_kernel(const T* __restrict__ bcx, const TW* __restrict__ conv_w,
-                                     const float* __restrict__ state, T* __restrict__ out,
-                                     const int* __restrict__ req_of_token, const int* __restrict__ q_start,
-                                     const int* __restrict__ state_slot, int d, int K) {
-    const int t = blockIdx.x;
-    const int c = blockIdx.y * blockDim.x + threadIdx.x;
-    if (c >= d) return;
-    const int r = req_of_token[t];
-    const int t0 = q_start[r];
-    const int i = t - t0;
-    const float* st = state + (long long)state_slot[r] * (K - 1) * d;
+__device__ __forceinline__ void conv_token(const T* __restrict__ bcx, const TW* __restrict__ conv_w, const float* st,
+                                           T* __restrict__ out, int t0, int i, int c, int d, int K) {
+    const int t = t0 + i;
     float y = 0.f;
     for (int k = 0; k < K; ++k) {
         const int src = i - (K - 1) + k;
@@ -49,21 +45,54 @@ __global__ void shortconv_fwd_kernel(const T* __restrict__ bcx, const TW* __rest
     out[(long long)t * d + c] = from_f32<T>(cg * y);
 }
 
-// The same for bfloat16 activations, eight channels a thread (16-byte loads and stores); d must
-// be a multiple of 8.  Every channel goes through the chain of operations of the kernel above.
-template <typename TW, int KT>                    // KT: the kernel length if it is 2, 3 or 4, else 0 (read K)
-__global__ void shortconv_fwd_vec_kernel(const bf16_t* __restrict__ bcx, const TW* __restrict__ conv_w,
-                                         const float* __restrict__ state, bf16_t* __restrict__ out,
-                                         const int* __restrict__ req_of_token, const int* __restrict__ q_start,
-                                         const int* __restrict__ state_slot, int d, int K_arg) {
-    const int K = KT ? KT : K_arg;
+template <typename T, typename TW, bool UPDATE>
+__global__ void shortconv_fwd_kernel(const T* __restrict__ bcx, const TW* __restrict__ conv_w,
+                                     float* state, T* __restrict__ out,
+                                     const int* __restrict__ req_of_token, const int* __restrict__ q_start,
+                                     const int* __restrict__ q_len, const int* __restrict__ state_slot, int d, int K) {
     const int t = blockIdx.x;
-    const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
     if (c >= d) return;
     const int r = req_of_token[t];
     const int t0 = q_start[r];
     const int i = t - t0;
-    const float* st = state + (long long)state_slot[r] * (K - 1) * d;
+    float* st = state + (long long)state_slot[r] * (K - 1) * d;
+    if (!UPDATE || i >= K - 1) {
+        conv_token(bcx, conv_w, st, out, t0, i, c, d, K);
+        return;
+    }
+    if (i > 0) return;                              // done by the thread of the request's first token
+    const int n = q_len[r];
+    for (int ii = 0; ii < min(n, K - 1); ++ii) conv_token(bcx, conv_w, st, out, t0, ii, c, d, K);
+    for (int j = 0; j < K - 1; ++j) {               // row j <- u of token n - (K-1) + j, or the old row j + n (not yet rewritten)
+        const int src = n - (K - 1) + j;
+        float u;
+        if (src >= 0) {
+            const T* row = bcx + (long long)(t0 + src) * 3 * d;
+            u = to_f32(row[c]) * to_f32(row[2 * d + c]);
+        } else {
+            u = st[(long long)(j + n) * d + c];
+        }
+        st[(long long)j * d + c] = u;
+    }
+}
+
+// The same for bfloat16 activations, eight channels a thread (16-byte loads and stores); d must
+// be a multiple of 8.  Every channel goes through the chain of operations of the kernel above.
+template <typename TW, int KT, bool UPDATE>       // KT: the kernel length if it is 2, 3 or 4, else 0 (read K)
+__global__ void shortconv_fwd_vec_kernel(const bf16_t* __restrict__ bcx, const TW* __restrict__ conv_w,
+                                         float* state, bf16_t* __restrict__ out,
+                                         const int* __restrict__ req_of_token, const int* __restrict__ q_start,
+                                         const int* __restrict__ q_len, const int* __restrict__ state_slot, int d, int K_arg) {
+    const int K = KT ? KT : K_arg;
+    const int t_own = blockIdx.x;
+    const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+    if (c >= d) return;
+    const int r = req_of_token[t_own];
+    const int t0 = q_start[r];
+    const int i_own = t_own - t0;
+    if (UPDATE && i_own > 0 && i_own < K - 1) return;      // done by the thread of the request's first token
+    float* st = state + (long long)state_slot[r] * (K - 1) * d;
     // the taps of the thread's eight channels are 8 K neighbouring weights: with a known K they come
     // in whole pieces of eight
     float wl[KT ? 8 * KT : 1];
@@ -73,11 +102,7 @@ __global__ void shortconv_fwd_vec_kernel(const bf16_t* __restrict__ bcx, const T
 #pragma unroll
             for (int e = 0; e < 8; ++e) wl[p * 8 + e] = to_f32(conv_w[(long long)c * KT + p * 8 + e]);
     }
-    float y[8];
-#pragma unroll
-    for (int k = 0; k < (KT ? KT : 1) * (KT ? 1 : K); ++k) {
-        const int src = i - (K - 1) + k;
-        float u[8];
+    auto u_of = [&](int src, float (&u)[8]) {       // u of the portion's token src, or of the state's row K-1+src
         if (src >= 0) {
             const bf16_t* row = bcx + (long long)(t0 + src) * 3 * d;
             const bf16x8 b = *(const bf16x8*)(row + c), x = *(const bf16x8*)(row + 2 * d + c);
@@ -89,17 +114,39 @@ __global__ void shortconv_fwd_vec_kernel(const bf16_t* __restrict__ bcx, const T
 #pragma unroll
             for (int e = 0; e < 4; ++e) { u[e] = u0[e]; u[4 + e] = u1[e]; }
         }
+    };
+    auto token = [&](int i) {
+        const int t = t0 + i;
+        float y[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float w = KT ? wl[e * (KT ? KT : 1) + k] : to_f32(conv_w[(long long)(c + e) * K + k]);
-            y[e] = (k == 0) ? u[e] * w : fmaf(u[e], w, y[e]);
+        for (int k = 0; k < (KT ? KT : 1) * (KT ? 1 : K); ++k) {
+            float u[8];
+            u_of(i - (K - 1) + k, u);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float w = KT ? wl[e * (KT ? KT : 1) + k] : to_f32(conv_w[(long long)(c + e) * K + k]);
+                y[e] = (k == 0) ? u[e] * w : fmaf(u[e], w, y[e]);
+            }
         }
-    }
-    const bf16x8 cg = *(const bf16x8*)(bcx + (long long)t * 3 * d + d + c);
-    bf16x8 o;
+        const bf16x8 cg = *(const bf16x8*)(bcx + (long long)t * 3 * d + d + c);
+        bf16x8 o;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) o[e] = (bf16_t)((float)cg[e] * y[e]);
-    *(bf16x8*)(out + (long long)t * d + c) = o;
+        for (int e = 0; e < 8; ++e) o[e] = (bf16_t)((float)cg[e] * y[e]);
+        *(bf16x8*)(out + (long long)t * d + c) = o;
+    };
+    if (!UPDATE || i_own > 0) {
+        token(i_own);
+        return;
+    }
+    const int n = q_len[r];
+    for (int ii = 0; ii < min(n, K - 1); ++ii) token(ii);
+    for (int j = 0; j < K - 1; ++j) {               // row j <- u of token n - (K-1) + j, or the old row j + n (not yet rewritten)
+        float u[8];
+        u_of(n - (K - 1) + j, u);
+        float* p = st + (long long)j * d + c;
+        *(f32x4*)p = f32x4{u[0], u[1], u[2], u[3]};
+        *(f32x4*)(p + 4) = f32x4{u[4], u[5], u[6], u[7]};
+    }
 }
 
 template <typename T>
@@ -174,30 +221,36 @@ TUFF_EXPORT int tuff_shortconv_decode(const void* bcx, const void* conv_w, int w
     return launch_status();
 }
 
-TUFF_EXPORT int tuff_shortconv_fwd(const void* bcx, const void* conv_w, int w_dt, const float* state, void* out, int dt,
-                                   const int* req_of_token, const int* q_start, const int* state_slot,
+// q_len: null, the state is only read; else [requests], and the state of every request with tokens in the
+// step is rewritten as well (the last K-1 values of u, as tuff_shortconv_state leaves them).
+TUFF_EXPORT int tuff_shortconv_fwd(const void* bcx, const void* conv_w, int w_dt, float* state, void* out, int dt,
+                                   const int* req_of_token, const int* q_start, const int* q_len, const int* state_slot,
                                    int n_tokens, int d, int K, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (K < 2 || K - 1 > MAX_TAPS) return -2;
     if (dt == DT_BF16 && d % 8 == 0 && n_tokens > 16) {
         const int threads = d / 8 < 256 ? ((d / 8 + 63) / 64) * 64 : 256;
         dim3 vblock(threads), vgrid(n_tokens, ceil_div(d / 8, threads));
-#define VEC(TW, KT) hipLaunchKernelGGL((shortconv_fwd_vec_kernel<TW, KT>), vgrid, vblock, 0, stream, (const bf16_t*)bcx, (const TW*)conv_w, \
-                                          state, (bf16_t*)out, req_of_token, q_start, state_slot, d, K)
+#define VEC_U(TW, KT, U) hipLaunchKernelGGL((shortconv_fwd_vec_kernel<TW, KT, U>), vgrid, vblock, 0, stream, (const bf16_t*)bcx, \
+                                             (const TW*)conv_w, state, (bf16_t*)out, req_of_token, q_start, q_len, state_slot, d, K)
+#define VEC(TW, KT) do { if (q_len) VEC_U(TW, KT, true); else VEC_U(TW, KT, false); } while (0)
 #define VEC_K(TW) do { if (K == 2) VEC(TW, 2); else if (K == 3) VEC(TW, 3); else if (K == 4) VEC(TW, 4); else VEC(TW, 0); } while (0)
         if (w_dt == DT_F32) VEC_K(float); else VEC_K(bf16_t);
 #undef VEC_K
 #undef VEC
+#undef VEC_U
         return launch_status();
     }
     dim3 block(256), grid(n_tokens, ceil_div(d, 256));
-#define LAUNCH(T, TW) hipLaunchKernelGGL((shortconv_fwd_kernel<T, TW>), grid, block, 0, stream, (const T*)bcx, (const TW*)conv_w, \
-        state, (T*)out, req_of_token, q_start, state_slot, d, K)
+#define LAUNCH_U(T, TW, U) hipLaunchKernelGGL((shortconv_fwd_kernel<T, TW, U>), grid, block, 0, stream, (const T*)bcx, (const TW*)conv_w, \
+        state, (T*)out, req_of_token, q_start, q_len, state_slot, d, K)
+#define LAUNCH(T, TW) do { if (q_len) LAUNCH_U(T, TW, true); else LAUNCH_U(T, TW, false); } while (0)
     if (dt == DT_F32 && w_dt == DT_F32) LAUNCH(float, float);
     else if (dt == DT_F32) LAUNCH(float, bf16_t);
     else if (w_dt == DT_F32) LAUNCH(bf16_t, float);
     else LAUNCH(bf16_t, bf16_t);
 #undef LAUNCH
+#undef LAUNCH_U
     return launch_status();
 }
 

@@ -69,9 +69,8 @@ class ShortConvMixer(Mixer):
             ops.shortconv_decode(bcx, self.conv_w, cache.state, y, state_slot=ctx.state_slot, K=self.K)
             self.out_proj.forward(y, accumulate_into=residual, next_norm=next_norm)
             return
+        # output and, unless the cache is only read, the new state in one kernel
         ops.shortconv_fwd(bcx, self.conv_w, cache.state, y, req_of_token=ctx.req_of_token,
-                          q_start=ctx.q_start, state_slot=ctx.state_slot, K=self.K)
-        if write_cache:
-            ops.shortconv_state(bcx, cache.state, q_start=ctx.q_start, q_len=ctx.q_len,
-                                state_slot=ctx.state_slot, K=self.K)
+                          q_start=ctx.q_start, state_slot=ctx.state_slot, K=self.K,
+                          q_len=ctx.q_len if write_cache else None)
         self.out_proj.forward(y, accumulate_into=residual, next_norm=next_norm)
