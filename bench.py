@@ -115,42 +115,63 @@ def run_decode(llm, cfg, batch: int, ctx_end: int, steps: int, warmup: int, seed
     return marks["t1"] - marks["t0"], ctx_end - steps / 2.0
 
 
-def run_prefill(llm, cfg, tokens: int, repeats: int = 8, warmup: int = 4):
-    """One prompt of `tokens` tokens in one step, to the first generated token on the host.  Returns
-    the seconds of `repeats` runs after `warmup` untimed ones (the engine records a step size that keeps
-    coming when it comes for the third time; that one-off recording is not a prefill's time)."""
+PREFILL_STREAM = 8               # prefill steps between two time marks
+
+
+def run_prefill(llm, cfg, tokens: int, runs: int = 3, warmup: int = 4):
+    """Prompts of `tokens` tokens, each in one step, to the first generated token.  Returns
+    (seconds a step in a stream, seconds of a step from an idle GPU): the first as decode steps are
+    timed, PREFILL_STREAM steps of as many requests between two synchronisations, `runs` times; the
+    second one step at a time with the GPU idle before it (the host packs the step first, and the
+    part's clocks take milliseconds to come back up), `PREFILL_STREAM` times.  Before either, `warmup`
+    untimed steps (the engine records a step size that keeps coming when it comes for the third time;
+    that one-off recording is not a prefill's time)."""
     import torch
     from tuff_amd.csrc import ops
     from tuff_amd.engine.batch import StepEntry
     eng = llm.engine
     g = torch.Generator().manual_seed(SEED + 1)
-    times = []
     picked = torch.empty(1, dtype=torch.int32, device=eng.device)
-    for i in range(repeats + warmup):
-        prompt = torch.randint(0, cfg.vocab_size, (tokens,), generator=g).tolist()
-        eng.begin(("prefill", i))
+    count = [0]
+
+    def stream(n: int) -> float:
+        ids = [("prefill", count[0] + i) for i in range(n)]
+        count[0] += n
+        prompts = [torch.randint(0, cfg.vocab_size, (tokens,), generator=g).tolist() for _ in ids]
+        for rid in ids:
+            eng.begin(rid)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        logits = eng.step([StepEntry(("prefill", i), prompt, [tokens - 1])])
-        ops.argmax(logits, picked)
-        nxt = int(picked.cpu()[0])                        # the first generated token reaches the host
+        for rid, prompt in zip(ids, prompts):
+            logits = eng.step([StepEntry(rid, prompt, [tokens - 1])])
+            ops.argmax(logits, picked)
+        int(picked.cpu()[0])                              # the last first token reaches the host
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        eng.end(("prefill", i))
-        if i >= warmup:
-            times.append(dt)
-    return times
+        for rid in ids:
+            eng.end(rid)
+        return dt / n
+
+    for _ in range(warmup):
+        stream(1)
+    stream(PREFILL_STREAM)                                # untimed: the stream's own warm-up
+    in_stream = [stream(PREFILL_STREAM) for _ in range(runs)]
+    alone = [stream(1) for _ in range(PREFILL_STREAM)]
+    return in_stream, alone
+
+
+def prefill_record(times, flops: float, dtype: str) -> dict:
+    in_stream, alone = times
+    dt, spread = mean_spread(in_stream)
+    dt_alone, spread_alone = mean_spread(alone)
+    return {"value": round(PREFILL_TOKENS / dt, 1), "tokens": PREFILL_TOKENS, "ms": round(dt * 1e3, 3),
+            "frac": round(flops / dt / (PEAK_TFLOPS[dtype] * 1e12), 4), "runs": len(in_stream),
+            "steps_a_run": PREFILL_STREAM, "spread_ms": round(spread * 1e3, 3),
+            "from_idle_ms": round(dt_alone * 1e3, 3), "from_idle_spread_ms": round(spread_alone * 1e3, 3)}
 
 
 def mean_spread(values):
     return sum(values) / len(values), (max(values) - min(values)) / 2.0
-
-
-def prefill_record(times, flops: float, dtype: str) -> dict:
-    dt, spread = mean_spread(times)
-    return {"value": round(PREFILL_TOKENS / dt, 1), "tokens": PREFILL_TOKENS, "ms": round(dt * 1e3, 3),
-            "frac": round(flops / dt / (PEAK_TFLOPS[dtype] * 1e12), 4), "runs": len(times),
-            "spread_ms": round(spread * 1e3, 3)}
 
 
 def probe(device) -> dict:
@@ -278,6 +299,7 @@ def main() -> int:
     ap.add_argument("--runs", type=int, default=3, help="runs a point (mean and spread over them)")
     ap.add_argument("--no-probe", dest="probe", action="store_false",
                     help="skip the measurement of the machine's own read bandwidth and matrix rate")
+    ap.add_argument("--prefill-warmup", type=int, default=4, help="untimed prefill runs before the timed ones")
     ap.add_argument("--only-prefill", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiling) and print its record")
     ap.add_argument("--scenario", choices=sorted(SCENARIOS),
@@ -301,14 +323,15 @@ def main() -> int:
     cfg = shape_config(args.layers)
     page = 16
     max_b = args.batch if args.no_points else max(args.batch, 64)
-    pages = max_b * (-(-args.context // page)) + PREFILL_TOKENS // page + 8
-    eng = Engine.from_config(cfg, SEED, dtype=args.dtype, page_size=page, num_pages=pages, max_requests=max_b + 1)
+    pages = max(max_b * (-(-args.context // page)), PREFILL_STREAM * (PREFILL_TOKENS // page)) + PREFILL_TOKENS // page + 8
+    eng = Engine.from_config(cfg, SEED, dtype=args.dtype, page_size=page, num_pages=pages,
+                             max_requests=max(max_b, PREFILL_STREAM) + 1)
     llm = LLM(engine=eng, max_num_seqs=max_b, max_batched_tokens=2048, ctx_size=args.context, ignore_eos=True)
     model = eng.model
 
     flops = prefill_flops(cfg, model, PREFILL_TOKENS)
     if args.only_prefill:
-        print(json.dumps({"prefill": prefill_record(run_prefill(llm, cfg, PREFILL_TOKENS), flops, args.dtype)}))
+        print(json.dumps({"prefill": prefill_record(run_prefill(llm, cfg, PREFILL_TOKENS, runs=args.runs, warmup=args.prefill_warmup), flops, args.dtype)}))
         return 0
 
     def decode_point(batch: int, steps: int, warmup: int, seed: int, context: int = 0, on=None) -> dict:
@@ -344,7 +367,7 @@ def main() -> int:
                      "frac": round(head["GBs"] / HBM_PEAK_GBS, 4)},
     }
     if not args.no_points:
-        out["prefill"] = prefill_record(run_prefill(llm, cfg, PREFILL_TOKENS), flops, args.dtype)
+        out["prefill"] = prefill_record(run_prefill(llm, cfg, PREFILL_TOKENS, runs=args.runs, warmup=args.prefill_warmup), flops, args.dtype)
         points = {}
         for b in (1, 64):
             pt = decode_point(b, args.point_steps, 8, SEED + b)
