@@ -252,6 +252,22 @@ def test_embed_and_swiglu(gpu):
     out = torch.empty(4, 24, device=gpu)
     ops.embed_rows(table.to(gpu), toks.to(gpu), out)
     assert torch.equal(out.cpu(), table[toks.long()].float())
+    ops.embed_rows(table.to(gpu), toks.to(gpu), out, scale=1.5)
+    assert torch.equal(out.cpu(), table[toks.long()].float() * 1.5)
+    # a bias onto rows of either type, and logits scaled under a soft cap
+    bias = _r(24, seed=12)
+    for dt in (torch.float32, torch.bfloat16):
+        y = _r(5, 24, seed=11, dtype=dt)
+        got = y.to(gpu)
+        ops.add_bias(got, bias.to(gpu))
+        assert torch.equal(got.cpu(), (y.float() + bias).to(dt))
+    x = _r(3, 37, seed=13, scale=4.0)
+    got = x.to(gpu)
+    ops.scale_cap(got, 0.5, 1.25)
+    assert (got.cpu().double() - 1.25 * torch.tanh(x.double() * 0.5 / 1.25)).abs().max() < 1e-6
+    got = x.to(gpu)
+    ops.scale_cap(got, 2.0)
+    assert torch.equal(got.cpu(), x * 2.0)
     for dt in (torch.float32, torch.bfloat16):
         gu = _r(7, 2 * 13, seed=10, scale=2.0, dtype=dt)
         act = torch.empty(7, 13, device=gpu, dtype=dt)

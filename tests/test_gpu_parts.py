@@ -608,3 +608,102 @@ def test_toy_feed_forward_with_routing_beside_the_frameworks_parts(gpu):
     finally:
         registry.unregister_architecture("ToyRoutedForCausalLM")
         FEED_FORWARDS.unregister("toy_routed")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_with_biases_a_scaled_embedding_and_capped_logits(gpu, dtype):
+    """What the reference's architecture has none of, declared by a toy one without a change to the
+    framework: projections with a bias (a gated feed-forward defined here from two `Linear`s), embedding
+    rows times sqrt(d), logits times a factor under a soft cap.  Whole and mixed plans against the
+    formulas written out here."""
+    from tuff_amd.config.base import ModelConfig
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.models import registry
+    from tuff_amd.models.decoder import DecoderModel
+    from tuff_amd.parts.base import FEED_FORWARDS, FeedForward, WeightDecl
+    from tuff_amd.parts.block import PreNormBlock
+    from tuff_amd.parts.linear import Linear
+    from tuff_amd.parts.norm import RMSNorm
+    from tuff_amd.parts.shortconv import ShortConvMixer
+    from tuff_amd.weights.random_init import random_weights
+    from tuff_amd.csrc import ops
+    d, F, V, K, eps = 48, 40, 131, 3, 1e-5
+    emb_scale, logit_scale, cap = math.sqrt(d), 0.5, 3.0
+
+    class BiasedGatedFF(FeedForward):
+        graph_safe = True
+
+        def __init__(self, d, F, prefix):
+            self.gate_up = Linear([f"{prefix}.g", f"{prefix}.u"], d, [F, F], swiglu_pair=True,
+                                  bias=[f"{prefix}.gb", f"{prefix}.ub"])
+            self.down = Linear(f"{prefix}.d", F, d, bias=f"{prefix}.db")
+            self.F = F
+
+        def weight_decls(self):
+            return self.gate_up.weight_decls() + self.down.weight_decls()
+
+        def kernel_modules(self):
+            return ["elementwise"]
+
+        def bind(self, weights, rt):
+            self.rt = rt
+            self.gate_up.bind(weights, rt)
+            self.down.bind(weights, rt)
+
+        def forward(self, h, ctx, residual):
+            gu = self.gate_up.forward(h)
+            act = self.rt.empty(h.shape[0], self.F, dtype=gu.dtype)
+            ops.swiglu(gu, act)
+            self.down.forward(act, accumulate_into=residual)
+
+    @dataclasses.dataclass
+    class BiasedConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyBiasedForCausalLM"
+        vocab_size: int
+
+    def build(cfg):
+        blocks = [PreNormBlock(RMSNorm(d, eps, f"l{i}.n1"),
+                               ShortConvMixer(d, K, names={"in_proj": f"l{i}.in", "conv": f"l{i}.conv", "out_proj": f"l{i}.out"}),
+                               RMSNorm(d, eps, f"l{i}.n2"), FEED_FORWARDS.get("toy_biased")(d, F, f"l{i}.ff")) for i in range(2)]
+        return DecoderModel(vocab_size=cfg.vocab_size, hidden_size=d, embedding=WeightDecl("emb", (cfg.vocab_size, d)),
+                            blocks=blocks, final_norm=RMSNorm(d, eps, "fn"), embedding_scale=emb_scale,
+                            logit_scale=logit_scale, logit_softcap=cap)
+
+    FEED_FORWARDS.register("toy_biased", BiasedGatedFF)
+    registry.register_architecture("ToyBiasedForCausalLM", BiasedConfig, build)
+    try:
+        cfg = registry.config_from_dict({"architectures": ["ToyBiasedForCausalLM"], "vocab_size": V})
+        model = registry.build_model(cfg)
+        stored = torch.float32 if dtype == "float32" else torch.bfloat16
+        weights = random_weights(model.weight_decls(), 8, stored, "cpu", stored_dtype=stored)
+        for k in list(weights):
+            if k.endswith("b"):                                           # biases large enough to matter
+                weights[k] = (weights[k].float() * 20).to(stored)
+            elif ".ff." in k or k == "emb":
+                weights[k] = (weights[k].float() * 6).to(stored)          # logits wide enough to reach the cap
+        eng = Engine(model, {k: v.to(gpu) for k, v in weights.items()}, dtype=dtype, max_tokens=256)
+        reqs = {"a": util.rand_tokens(33, V, 1), "b": util.rand_tokens(20, V, 2), "c": util.rand_tokens(9, V, 3)}
+        whole = util.run_plan(eng, util.plan_whole(reqs))
+        mixed = util.run_plan(eng, util.plan_mixed(reqs, seed=2, decode_tail=5))
+        w = {k: v.double() for k, v in weights.items()}
+        capped = 0
+        for rid, toks in reqs.items():
+            x = w["emb"][toks] * emb_scale
+            for i in range(2):
+                x = x + plain.short_conv(plain.rms_norm(x, w[f"l{i}.n1"], eps), w[f"l{i}.in"], w[f"l{i}.conv"], w[f"l{i}.out"])
+                h = plain.rms_norm(x, w[f"l{i}.n2"], eps)
+                g = h @ w[f"l{i}.ff.g"].T + w[f"l{i}.ff.gb"]
+                u = h @ w[f"l{i}.ff.u"].T + w[f"l{i}.ff.ub"]
+                x = x + (g / (1 + torch.exp(-g)) * u) @ w[f"l{i}.ff.d"].T + w[f"l{i}.ff.db"]
+            raw = plain.rms_norm(x, w["fn"], eps) @ w["emb"].T * logit_scale
+            want = cap * torch.tanh(raw / cap)
+            capped += int((raw.abs() > cap).sum())
+            for got in (whole[rid], mixed[rid]):
+                if dtype == "float32":
+                    util.assert_close_f32(got, want, rid)
+                else:
+                    util.assert_close_bf16(got, want, rid)
+        assert capped > 50                                                # the cap does something here
+    finally:
+        registry.unregister_architecture("ToyBiasedForCausalLM")
+        FEED_FORWARDS.unregister("toy_biased")

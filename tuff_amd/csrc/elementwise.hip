@@ -4,26 +4,60 @@
 #include "common.h"
 
 // ------------------------------------------------------------------ embedding
-// out[t, :] = table[tokens[t], :] as float32.  Reference: one row gather per token
-// with no scale (src/lfm25_gpu.cu:725-741).
+// out[t, :] = table[tokens[t], :] * scale as float32.  Reference: one row gather per token
+// with no scale (src/lfm25_gpu.cu:725-741), which is scale = 1: the product with 1 is exact.
 template <typename T>
 __global__ void embed_rows_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
-                                  float* __restrict__ out, int d) {
+                                  float* __restrict__ out, int d, float scale) {
     const int t = blockIdx.x;
     const long long row = tokens[t];
     const T* src = table + row * (long long)d;
     float* dst = out + (long long)t * d;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) dst[i] = to_f32(src[i]);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) dst[i] = to_f32(src[i]) * scale;
 }
 
 TUFF_EXPORT int tuff_embed_rows(const void* table, int table_dt, const int* tokens, float* out,
-                                int n_tokens, int d, hipStream_t stream) {
+                                int n_tokens, int d, float scale, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     dim3 grid(n_tokens), block(256);
     if (table_dt == DT_F32)
-        hipLaunchKernelGGL(embed_rows_kernel<float>, grid, block, 0, stream, (const float*)table, tokens, out, d);
+        hipLaunchKernelGGL(embed_rows_kernel<float>, grid, block, 0, stream, (const float*)table, tokens, out, d, scale);
     else
-        hipLaunchKernelGGL(embed_rows_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, tokens, out, d);
+        hipLaunchKernelGGL(embed_rows_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, tokens, out, d, scale);
+    return launch_status();
+}
+
+// ----------------------------------------------------------------------- bias
+// y[r, c] += bias[c], the sum in float32: for projections with a bias, after their product (the
+// products' epilogues have none).
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ y, const float* __restrict__ bias, long long n, int N) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = from_f32<T>(to_f32(y[i]) + bias[i % N]);
+}
+
+TUFF_EXPORT int tuff_add_bias(void* y, int dt, const float* bias, long long rows, int N, hipStream_t stream) {
+    const long long n = rows * N;
+    if (n <= 0) return 0;
+    dim3 grid((unsigned)ceil_div_ll(n, 256)), block(256);
+    if (dt == DT_F32) hipLaunchKernelGGL(add_bias_kernel<float>, grid, block, 0, stream, (float*)y, bias, n, N);
+    else hipLaunchKernelGGL(add_bias_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)y, bias, n, N);
+    return launch_status();
+}
+
+// --------------------------------------------------------------- logits: scale and soft cap
+// x <- x * scale, then, with cap > 0, x <- cap * tanh(x / cap).
+__global__ void scale_cap_kernel(float* __restrict__ x, long long n, float scale, float cap) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float v = x[i] * scale;
+    if (cap > 0.f) v = cap * tanhf(v / cap);
+    x[i] = v;
+}
+
+TUFF_EXPORT int tuff_scale_cap(float* x, long long n, float scale, float cap, hipStream_t stream) {
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(scale_cap_kernel, dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, stream, x, n, scale, cap);
     return launch_status();
 }
 

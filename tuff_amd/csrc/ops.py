@@ -26,7 +26,9 @@ class KernelError(RuntimeError):
 
 _SIGNATURES = {
     "elementwise": {
-        "tuff_embed_rows": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+        "tuff_embed_rows": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_float, _c_void_p],
+        "tuff_add_bias": [_c_void_p, _c_int, _c_void_p, _c_ll, _c_int, _c_void_p],
+        "tuff_scale_cap": [_c_void_p, _c_ll, _c_float, _c_float, _c_void_p],
         "tuff_rmsnorm": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_float, _c_void_p],
         "tuff_swiglu": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_cast": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_void_p],
@@ -171,11 +173,26 @@ def _check(code: int, what: str) -> None:
 
 
 # ------------------------------------------------------------------------ row kernels
-def embed_rows(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
+def embed_rows(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    """out[t] = table[tokens[t]] * scale, float32."""
     n, d = out.shape
     _check(load("elementwise").tuff_embed_rows(
         _gpu("table", table, shape=(None, d)), _dt(table), _gpu("tokens", tokens, torch.int32, (n,)),
-        _gpu("out", out, torch.float32), n, d, _stream()), "embed_rows")
+        _gpu("out", out, torch.float32), n, d, float(scale), _stream()), "embed_rows")
+
+
+def add_bias(y: torch.Tensor, bias: torch.Tensor) -> None:
+    """y[r, c] += bias[c] in place (y float32 or bfloat16 [rows, N], bias float32 [N])."""
+    rows, N = y.shape
+    _gpu("y", y)
+    _gpu("bias", bias, torch.float32, (N,))
+    _check(load("elementwise").tuff_add_bias(y.data_ptr(), _dt(y), bias.data_ptr(), rows, N, _stream()), "add_bias")
+
+
+def scale_cap(x: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> None:
+    """x <- x * scale, then, with cap > 0, x <- cap * tanh(x / cap); float32, in place."""
+    _gpu("x", x, torch.float32)
+    _check(load("elementwise").tuff_scale_cap(x.data_ptr(), x.numel(), float(scale), float(cap), _stream()), "scale_cap")
 
 
 def rmsnorm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, eps: float,

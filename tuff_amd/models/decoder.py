@@ -32,13 +32,19 @@ class DecoderModel:
     def __init__(self, *, vocab_size: int, hidden_size: int, embedding: WeightDecl,
                  blocks: list[Block], final_norm: Norm, head: Optional[WeightDecl] = None,
                  schedule: Optional[list[LayerRun]] = None, max_positions: Optional[int] = None,
-                 eos_token_id: Optional[int] = None):
+                 eos_token_id: Optional[int] = None, embedding_scale: float = 1.0,
+                 logit_scale: float = 1.0, logit_softcap: Optional[float] = None):
         """head=None: the head is the embedding (tied), as the reference does when the file has
-        no output matrix (src/lfm25_model.c:128-131)."""
+        no output matrix (src/lfm25_model.c:128-131).
+        embedding_scale: the embedding rows are multiplied by it on their way into the residual stream.
+        logit_scale, logit_softcap: logits = head(norm(x)) * logit_scale, then, with a cap c,
+        c * tanh(logits / c).  The reference has none of the three (scale 1, no cap), which are the defaults."""
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.embedding_decl, self.head_decl = embedding, head
         self.blocks, self.final_norm = list(blocks), final_norm
         self.max_positions, self.eos_token_id = max_positions, eos_token_id
+        self.embedding_scale, self.logit_scale = float(embedding_scale), float(logit_scale)
+        self.logit_softcap = None if not logit_softcap else float(logit_softcap)
         runs = schedule if schedule is not None else [LayerRun(i) for i in range(len(self.blocks))]
         self.schedule: list[LayerRun] = []
         next_id = 0
@@ -141,7 +147,7 @@ class DecoderModel:
         [len(ctx.logit_rows), vocab], or None when no logits are wanted."""
         rt = self.rt
         x = torch.empty(ctx.T, self.hidden_size, dtype=torch.float32, device=rt.device)
-        ops.embed_rows(self.embedding, ctx.tokens, x)
+        ops.embed_rows(self.embedding, ctx.tokens, x, self.embedding_scale)
         head_fused, all_rows = self._head_fused(ctx)
         for i, run in enumerate(self.schedule):
             block = self.blocks[run.block]
@@ -192,6 +198,12 @@ class DecoderModel:
         return fused, all_rows
 
     def _head(self, x, ctx) -> Optional[torch.Tensor]:
+        logits = self._head_product(x, ctx)
+        if logits is not None and (self.logit_scale != 1.0 or self.logit_softcap is not None):
+            ops.scale_cap(logits, self.logit_scale, self.logit_softcap or 0.0)
+        return logits
+
+    def _head_product(self, x, ctx) -> Optional[torch.Tensor]:
         if ctx.n_logits == 0:
             return None
         rt = self.rt

@@ -15,10 +15,14 @@ from .base import Runtime, WeightDecl
 class Linear:
     def __init__(self, names: Sequence[str] | str, in_features: int,
                  out_features: Sequence[int] | int, aliases: Sequence[Sequence[str]] | None = None,
-                 swiglu_pair: bool = False):
+                 swiglu_pair: bool = False, bias: Sequence[str] | str | None = None):
         """swiglu_pair: the two stacked tensors are the gate and the up matrix of a SwiGLU; with
         bfloat16 weights their rows are interleaved so that forward(..., swiglu=True) can apply
-        silu(gate) * up in the product's epilogue."""
+        silu(gate) * up in the product's epilogue.
+        bias: checkpoint names of a bias vector per stacked tensor ([out] each), y = x W^T + b.  The
+        products' epilogues have no bias: it is added by a kernel of its own after the product, and a
+        projection with one takes none of the fused ways (activation, convolution or the next norm in
+        the product's epilogue); the result is the same function."""
         self.names = [names] if isinstance(names, str) else list(names)
         outs = [out_features] if isinstance(out_features, int) else list(out_features)
         if len(outs) != len(self.names):
@@ -32,10 +36,17 @@ class Linear:
         if self.swiglu_pair and (len(self.names) != 2 or self.outs[0] != self.outs[1]):
             raise ValueError("a SwiGLU pair is two tensors of one shape")
         self.interleaved = False
+        self.bias_names = None if bias is None else ([bias] if isinstance(bias, str) else list(bias))
+        if self.bias_names is not None and len(self.bias_names) != len(self.names):
+            raise ValueError("one bias per stacked tensor")
+        self.bias = None              # bound: float32 [out]
 
     def weight_decls(self) -> list[WeightDecl]:
-        return [WeightDecl(n, (o, self.in_features), "normal", aliases=a)
-                for n, o, a in zip(self.names, self.outs, self.aliases)]
+        decls = [WeightDecl(n, (o, self.in_features), "normal", aliases=a)
+                 for n, o, a in zip(self.names, self.outs, self.aliases)]
+        if self.bias_names is not None:
+            decls += [WeightDecl(n, (o,), "normal") for n, o in zip(self.bias_names, self.outs)]
+        return decls
 
     def bind(self, weights: dict[str, torch.Tensor], rt: Runtime) -> None:
         self.rt = rt
@@ -45,7 +56,7 @@ class Linear:
         else:
             if len({w.dtype for w in ws}) != 1:
                 ws = [w.to(torch.float32) for w in ws]
-            if self.swiglu_pair and ws[0].dtype == torch.bfloat16:
+            if self.swiglu_pair and ws[0].dtype == torch.bfloat16 and self.bias_names is None:
                 self.weight = torch.stack(ws, dim=1).reshape(self.out_features, self.in_features).contiguous()
                 self.interleaved = True
             else:
@@ -55,13 +66,15 @@ class Linear:
                 raise ValueError(f"{self.names[0]}: the bfloat16 matrix kernels need an input size that is a "
                                  f"multiple of 8, got {self.in_features}")
             self.weight = ops.tile_weight(self.weight)       # the order the kernels stream it in
+        if self.bias_names is not None:
+            self.bias = torch.cat([weights[n].to(torch.float32).reshape(-1) for n in self.bias_names]).contiguous()
 
     def group_rows_for_conv(self) -> bool:
         """Call after bind(), for the input projection of a gated short convolution: keeps a second copy of
         the weight with its rows regrouped, so that forward_conv() can run projection and convolution of
         single tokens in one kernel.  False (and nothing kept) where the kernels cannot."""
         w = self.weight
-        if not isinstance(w, ops.TiledWeight) or self.out_features % 48 or len(self.names) != 1:
+        if not isinstance(w, ops.TiledWeight) or self.out_features % 48 or len(self.names) != 1 or self.bias is not None:
             return False
         self.weight_grouped = ops.tile_weight(ops.conv_group_rows(w.rows()))
         return True
@@ -103,6 +116,8 @@ class Linear:
         if swiglu and not self.interleaved:
             raise TypeError(f"{self.names[0]}: no fused SwiGLU for this weight")
         pending = x if isinstance(x, PendingNorm) else None
+        if pending is not None and self.bias is not None:
+            x, pending = pending.tensor(), None        # with a bias: the plain product, then the bias
         if pending is not None:
             T = pending.shape[0]
             # the row scales left by the product before, or the norm inside this product
@@ -135,7 +150,7 @@ class Linear:
 
         dev = w.device
         if accumulate_into is not None:
-            nxt = next_norm
+            nxt = next_norm if self.bias is None else None      # the sum is not final before the bias is in
             layout = None
             if (nxt is not None and pending is None and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
                     and self.in_features % 8 == 0):
@@ -148,15 +163,29 @@ class Linear:
                 nxt.announce_operand(accumulate_into, xw, ss)
                 return None
             product(accumulate_into, accumulate=True)
+            if self.bias is not None:
+                ops.add_bias(accumulate_into, self.bias)
             return None
         want = out_dtype or self.rt.dtype
         width = self.out_features // 2 if swiglu else self.out_features
         if w.dtype == torch.float32 and want != torch.float32:
             y32 = torch.empty(T, width, dtype=torch.float32, device=dev)
             product(y32)
+            if self.bias is not None:
+                ops.add_bias(y32, self.bias)
+            y = torch.empty(T, width, dtype=want, device=dev)
+            ops.cast(y32, y)
+            return y
+        if self.bias is not None and want != torch.float32:
+            # the bias goes onto the float32 sum, which is then rounded once
+            y32 = torch.empty(T, width, dtype=torch.float32, device=dev)
+            product(y32)
+            ops.add_bias(y32, self.bias)
             y = torch.empty(T, width, dtype=want, device=dev)
             ops.cast(y32, y)
             return y
         y = torch.empty(T, width, dtype=want, device=dev)
         product(y)
+        if self.bias is not None:
+            ops.add_bias(y, self.bias)
         return y
