@@ -62,6 +62,20 @@ def test_loud_conv_mixers(gpu, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page_size", [16, 48, 64])
+def test_heads_of_64_and_other_page_sizes(gpu, page_size, dtype):
+    """Heads of 64 channels (the single-token kernels that do norm, rotation, cache write and attention in
+    one, and projection and convolution in one, are for them) on pages of 16, 48 and 64 positions:
+    a head and single tokens, changing portions, and mixed with pages that are used again."""
+    reqs = requests_for("E")
+    check_plan("E", dtype, util.plan_tail(reqs, 32), reqs, page_size=page_size)
+    check_plan("E", dtype, util.plan_chunks(reqs, sizes=(2, 3, 2, 29, 5)), reqs, page_size=page_size)
+    plan = util.plan_mixed(reqs, seed=8)
+    peak = -(-util.live_tokens_peak(plan) // page_size) * page_size + 4 * page_size
+    check_plan("E", dtype, plan, reqs, page_size=page_size, max_tokens=peak, max_requests=4)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_feed_forward_width_that_is_no_multiple_of_8(gpu, dtype):
     reqs = requests_for("D")
     check_plan("D", dtype, util.plan_whole(reqs), reqs)

@@ -40,13 +40,22 @@ TINY_D = dict(
     hidden_size=32, num_attention_heads=2, num_key_value_heads=1,
     block_ff_dim=100, block_auto_adjust_ff_dim=False, vocab_size=333, rope_theta=10000.0,
     conv_L_cache=3, norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=512)
+# heads of 64 channels, which the single-token steps of bfloat16 take through kernels of their own (norm,
+# rotation, cache write and attention in one; the convolution in the input projection's epilogue)
+TINY_E = dict(
+    architectures=["Lfm2ForCausalLM"], num_hidden_layers=4,
+    layer_types=["conv", "full_attention", "full_attention", "conv"],
+    hidden_size=192, num_attention_heads=3, num_key_value_heads=1,
+    block_ff_dim=200, block_auto_adjust_ff_dim=False, vocab_size=601, rope_theta=100000.0,
+    conv_L_cache=3, norm_eps=2e-5, tie_word_embeddings=True, max_position_embeddings=2048)
 # Three layers with the sizes of a 1.2B model (feed-forward 8192 after the adjustment): not tiny, used by one test.
 FULL_SIZE_LAYERS = dict(
     architectures=["Lfm2ForCausalLM"], num_hidden_layers=3, layer_types=["conv", "full_attention", "conv"],
     hidden_size=2048, num_attention_heads=32, num_key_value_heads=8, block_ff_dim=12288,
     block_auto_adjust_ff_dim=True, block_multiple_of=256, block_ffn_dim_multiplier=1.0, vocab_size=65536,
     rope_theta=1000000.0, conv_L_cache=3, norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=8192)
-CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 5), "D": (TINY_D, 9), "F": (FULL_SIZE_LAYERS, 2)}
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 5), "D": (TINY_D, 9), "E": (TINY_E, 11),
+           "F": (FULL_SIZE_LAYERS, 2)}
 
 _TMP = tempfile.TemporaryDirectory(prefix="tuff_amd_tests_")
 
