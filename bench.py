@@ -170,6 +170,38 @@ def prefill_record(times, flops: float, dtype: str) -> dict:
             "from_idle_ms": round(dt_alone * 1e3, 3), "from_idle_spread_ms": round(spread_alone * 1e3, 3)}
 
 
+LONG_PROMPT = 32768             # tokens of the long prompt point, fed in portions of PREFILL_TOKENS
+
+
+def run_long_prompt(llm, cfg, tokens: int, runs: int = 3):
+    """One prompt of `tokens` tokens through the step function in portions of PREFILL_TOKENS, to its
+    first generated token.  Returns the seconds of `runs` runs after one untimed one."""
+    import torch
+    from tuff_amd.csrc import ops
+    from tuff_amd.engine.batch import StepEntry
+    eng = llm.engine
+    g = torch.Generator().manual_seed(SEED + 7)
+    picked = torch.empty(1, dtype=torch.int32, device=eng.device)
+    times = []
+    for run in range(runs + 1):
+        prompt = torch.randint(0, cfg.vocab_size, (tokens,), generator=g).tolist()
+        rid = ("long prompt", run)
+        eng.begin(rid)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(0, tokens, PREFILL_TOKENS):
+            part = prompt[i:i + PREFILL_TOKENS]
+            last = i + PREFILL_TOKENS >= tokens
+            logits = eng.step([StepEntry(rid, part, [len(part) - 1] if last else [])])
+        ops.argmax(logits, picked)
+        int(picked.cpu()[0])
+        torch.cuda.synchronize()
+        if run:
+            times.append(time.perf_counter() - t0)
+        eng.end(rid)
+    return times
+
+
 def mean_spread(values):
     return sum(values) / len(values), (max(values) - min(values)) / 2.0
 
@@ -376,6 +408,16 @@ def main() -> int:
             points[f"decode_b{b}_ms_per_step"] = round(pt["ms"], 4)
             points[f"decode_b{b}_GBs"] = round(pt["GBs"], 1)
             points[f"decode_b{b}_roofline_frac"] = round(pt["GBs"] / HBM_PEAK_GBS, 4)
+        if args.long_points and LONG_PROMPT <= max_b * args.context:
+            # a long prompt in portions: the attention over what earlier portions left is most of its work
+            try:
+                dt, spread = mean_spread(run_long_prompt(llm, cfg, LONG_PROMPT, args.runs))
+                points[f"prompt_{LONG_PROMPT}_tok_s"] = round(LONG_PROMPT / dt, 1)
+                points[f"prompt_{LONG_PROMPT}_ms"] = round(dt * 1e3, 2)
+                points[f"prompt_{LONG_PROMPT}_spread_ms"] = round(spread * 1e3, 2)
+            except Exception as e:                            # noqa: BLE001 - a point beside the benchmark must not lose it
+                points[f"prompt_{LONG_PROMPT}_tok_s"] = None
+                points[f"prompt_{LONG_PROMPT}_error"] = f"{type(e).__name__}: {e}"[:200]
         if args.long_points:
             # the same model further out: the cache of the live requests is then most of what a step reads
             for b, ctx in LONG_POINTS:
