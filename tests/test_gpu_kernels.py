@@ -1106,6 +1106,63 @@ def test_gemm_with_the_convolution_in_its_epilogue(gpu, M, d, K, taps, norm):
                       conv_w=conv_w.to(gpu), state=state, state_slot=torch.zeros(17, dtype=torch.int32, device=gpu))
 
 
+@pytest.mark.parametrize("M,d,K,taps", [(17, 64, 64, 3), (64, 2048, 2048, 3), (33, 240, 328, 4), (48, 48, 96, 2), (20, 96, 8192, 7)])
+@pytest.mark.parametrize("norm", ["none", "scaled"])
+def test_gemm_with_the_convolution_in_the_kernel_that_adds_its_slices(gpu, M, d, K, taps, norm):
+    """17 to 64 single tokens: the kernel that adds the projection's partial tiles runs the convolution.
+    Against the plain formulas, and bit for bit against the projection followed by the kernel for single
+    tokens (the same sums in the same order, rounded to bfloat16 at the same place)."""
+    from tuff_amd.csrc import ops
+    eps = 1e-5
+    w_in = _r(3 * d, K, seed=1, scale=K ** -0.5, dtype=torch.bfloat16)
+    conv_w = _r(d, taps, seed=2, scale=0.5, dtype=torch.bfloat16).to(gpu)
+    slots = torch.randperm(M + 3, generator=torch.Generator().manual_seed(3))[:M].to(torch.int32)
+    state0 = _r(M + 3, taps - 1, d, seed=4)
+    x32 = _r(M, K, seed=5)
+    nw = 1 + _r(K, seed=6, scale=0.1)
+    w = ops.tile_weight(w_in.to(gpu))
+    state, state2 = state0.clone().to(gpu), state0.clone().to(gpu)
+    out = torch.full((M, d), float("nan"), dtype=torch.bfloat16, device=gpu)
+    bcx = torch.empty(M, 3 * d, dtype=torch.bfloat16, device=gpu)
+    kw = dict(conv_w=conv_w, state=state, state_slot=slots.to(gpu))
+    if norm == "none":
+        h = x32.to(torch.bfloat16)
+        ops.gemm_conv64(h.to(gpu), w, out, **kw)
+        ops.gemm(h.to(gpu), w, bcx)
+        h = h.double()
+    else:
+        xw = (x32 * nw).to(torch.bfloat16)
+        tiles = 5
+        ss = torch.zeros(tiles, 64)
+        cut = [K * t // tiles for t in range(tiles + 1)]
+        for t in range(tiles):
+            ss[t, :M] = (x32[:, cut[t]:cut[t + 1]] ** 2).sum(-1)
+        ops.gemm_conv64(xw.to(gpu), w, out, ss=ss.to(gpu), eps=eps, **kw)
+        ops.gemm_scaled(xw.to(gpu), ss.to(gpu), eps, w, bcx)
+        h = xw.double() / torch.sqrt((x32.double() ** 2).mean(-1, keepdim=True) + eps)
+    ref = (h @ w_in.double().T).to(torch.bfloat16).double()
+    B, C, X = ref[:, :d], ref[:, d:2 * d], ref[:, 2 * d:]
+    u = B * X
+    st = state0[slots.long()].double()
+    y = (st * conv_w.cpu().double().T[:taps - 1][None]).sum(1) + u * conv_w.cpu().double()[:, taps - 1]
+    want = C * y
+    got = out.cpu().double()
+    assert torch.isfinite(got).all()
+    assert (got - want).abs().max() <= 2 ** -6 * float(want.abs().max()), (got - want).abs().max()
+    want_state = torch.cat([st[:, 1:], u[:, None]], dim=1)
+    assert (state.cpu().double()[slots.long()] - want_state).abs().max() <= 2 ** -6 * float(want_state.abs().max())
+    others = torch.ones(M + 3, dtype=torch.bool)
+    others[slots.long()] = False
+    assert torch.equal(state.cpu()[others], state0[others])               # nobody else's state was touched
+    # the two-kernel way from the projected rows
+    out2 = torch.empty(M, d, dtype=torch.bfloat16, device=gpu)
+    ops.shortconv_decode(bcx, conv_w, state2, out2, state_slot=slots.to(gpu), K=taps)
+    if norm == "none":
+        assert torch.equal(out, out2) and torch.equal(state, state2)
+    else:                                      # with one slice the projection adds the sums of squares in another order
+        assert (out.float() - out2.float()).abs().max() <= 2 ** -7 * float(out2.float().abs().max())
+
+
 def test_shortconv_last_tap_is_the_current_token(gpu):
     from tuff_amd.csrc import ops
     d, K = 32, 3

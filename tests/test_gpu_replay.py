@@ -76,6 +76,24 @@ def test_heads_of_64_and_other_page_sizes(gpu, page_size, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,n_req", [("A+", 20), ("E", 37), ("B+", 64)])
+def test_many_requests_decode_together(gpu, name, n_req, dtype):
+    """17 to 64 requests bring one token each in a step: the products of that many rows, the convolution in
+    the kernel that adds their slices, attention over many short requests.  Heads of the prompts in one
+    step of portions, then twelve steps of single tokens of all requests."""
+    V = util.CONFIGS[name.rstrip("+")][0]["vocab_size"]
+    tail = 12
+    reqs = {f"r{i}": util.rand_tokens(tail + 2 + (7 * i) % 19, V, 300 + i) for i in range(n_req)}
+    steps = [{"step": 0, "entries": [{"id": rid, "tokens": toks[:len(toks) - tail], "want": list(range(len(toks) - tail))}
+                                     for rid, toks in reqs.items()], "end": []}]
+    for j in range(tail):
+        steps.append({"step": len(steps), "end": [],
+                      "entries": [{"id": rid, "tokens": [toks[len(toks) - tail + j]], "want": [0]} for rid, toks in reqs.items()]})
+    steps[-1]["end"] = list(reqs)
+    check_plan(name, dtype, steps, reqs, max_tokens=64 * n_req, max_requests=n_req)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_feed_forward_width_that_is_no_multiple_of_8(gpu, dtype):
     reqs = requests_for("D")
     check_plan("D", dtype, util.plan_whole(reqs), reqs)

@@ -970,6 +970,100 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const float* __restr
     }
 }
 
+// The same for the input projection of a gated short convolution over 17 to 64 single tokens (row r is
+// request r's token): from the partial tiles of the projection [3 d] wide (B | C | X, as the checkpoint
+// has them) the thread of (row, four channels) adds the slices of its twelve columns in slice order,
+// scales and rounds them to bfloat16 as a projected row would hold them, and then does what the kernel
+// for single tokens does: y = C * (taps . (state, B * X)), the state shifted by one.  The projected
+// rows are never written.  grid (tiles of 64 channels, groups of 4 rows), one wave a workgroup: with twelve
+// columns a thread there is three times the work of the kernel above in a thread, so more and smaller
+// workgroups.  Two trips to memory one after the other remain (the row's slot, then its state beside the
+// slices): 7.1 us at 64 rows of 2,048 channels, where the kernel above and the convolution's own took 9.5.
+constexpr int FC_ROWS = 4;
+template <int NORM>
+__global__ __launch_bounds__(FC_ROWS * 16) void splitk_finish_conv_kernel(const float* __restrict__ ws, bf16_t* __restrict__ Y, int M, int d,
+                                                                 int rows_padded, int n_slices, FinishExtra ex, ConvTail cv) {
+    const int tid = threadIdx.x, q = tid % 16;
+    const long long row = (long long)blockIdx.y * FC_ROWS + tid / 16;
+    const long long ch0 = (long long)blockIdx.x * 64 + q * 4;
+    const int N = 3 * d;
+    float scale = 1.f;
+    if (NORM == NORM_SCALED) {
+        float t = 0.f;
+        if (row < ex.ss_rows)
+            for (int j = q; j < ex.n_ss; j += 16) t += ex.ss_in[(long long)j * ex.ss_rows + row];
+        t += __shfl_xor(t, 1, WAVE);
+        t += __shfl_xor(t, 2, WAVE);
+        t += __shfl_xor(t, 4, WAVE);
+        t += __shfl_xor(t, 8, WAVE);
+        scale = 1.0f / sqrtf(t / (float)ex.K + ex.eps);
+    }
+    if (row >= M || ch0 >= d) return;                      // d is a multiple of 16: four channels or none
+    // The state's rows and the taps are asked for now, before the slices: they depend on nothing that is
+    // computed here, and a load at the end would cost another trip to memory.  (Up to four older rows are
+    // kept in registers; a longer convolution reads the rest when it needs them.)
+    const int Kc = cv.taps;
+    float* st = cv.state + (long long)cv.state_slot[row] * (Kc - 1) * d;
+    constexpr int KEEP = 4;
+    f32x4 sv[KEEP];
+    float wv[KEEP + 1][4];
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+        sv[k] = k < Kc - 1 ? *(const f32x4*)(st + (long long)k * d + ch0) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) wv[k][e] = k < Kc - 1 ? cv.tap((int)ch0 + e, k) : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) wv[KEEP][e] = cv.tap((int)ch0 + e, Kc - 1);
+    float v[3][4];
+    const long long stride = (long long)rows_padded * N;
+#pragma unroll
+    for (int part = 0; part < 3; ++part) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[part][e] = 0.f;
+        const float* p0 = ws + row * N + (long long)part * d + ch0;
+        for (int s0 = 0; s0 < n_slices; s0 += 8) {         // as the kernel above: eight slices asked for together, added in order
+            f32x4 t[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (s0 + u < n_slices) t[u] = *(const f32x4*)(p0 + (s0 + u) * stride);
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (s0 + u < n_slices) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[part][e] += t[u][e];
+                }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[part][e] = (float)(bf16_t)(v[part][e] * scale);
+    }
+    f32x4 y, u4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { u4[e] = v[0][e] * v[2][e]; y[e] = 0.f; }
+    // y = taps . (state rows in order, then u), one chain of operations a channel; row k moves to k - 1
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k)
+        if (k < Kc - 1) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) y[e] = (k == 0) ? sv[k][e] * wv[k][e] : fmaf(sv[k][e], wv[k][e], y[e]);
+            if (k > 0) *(f32x4*)(st + (long long)(k - 1) * d + ch0) = sv[k];
+        }
+    for (int k = KEEP; k < Kc - 1; ++k) {
+        const f32x4 s4 = *(const f32x4*)(st + (long long)k * d + ch0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[e] = fmaf(s4[e], cv.tap((int)ch0 + e, k), y[e]);
+        *(f32x4*)(st + (long long)(k - 1) * d + ch0) = s4;
+    }
+    bf16x4 o4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        y[e] = fmaf(u4[e], wv[KEEP][e], y[e]);
+        o4[e] = (bf16_t)(v[1][e] * y[e]);
+    }
+    *(f32x4*)(st + (long long)(Kc - 2) * d + ch0) = u4;
+    *(bf16x4*)(Y + row * d + ch0) = o4;
+}
+
 struct SkinnyPlan { int tiles, waves, slices, chunks_per_slice, cols; long long ws_floats; };
 
 // How a skinny product is cut.  Depends on N and K (and on which of the two kernels M selects).
@@ -1111,6 +1205,27 @@ int launch_skinny64(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int
         hipLaunchKernelGGL((splitk_finish_kernel<MODE, NORM, EMIT>), dim3(p.tiles, EMIT ? 4 : mt), dim3(256), 0, stream,
                            (const float*)ws, Y, M, N, mt * 16, p.slices, ex);
     }
+    return launch_status();
+}
+
+// 16 < M <= 64: the projection's partial tiles into the work space (always: also with one slice), then the
+// kernel that adds them and runs the convolution.
+template <int NORM>
+int launch_skinny64_conv(const bf16_t* X, const bf16_t* W, bf16_t* Y, int M, int d, int K, float* ws, const FinishExtra& ex,
+                         const ConvTail& cv, hipStream_t stream) {
+    const int N = 3 * d;
+    const SkinnyPlan p = plan_skinny(M, N, K, 16, true);
+    if (!ws) return -4;
+    const int mt = ceil_div(M, 16);
+    dim3 grid(p.tiles, p.slices), block(SK_NT);
+#define GO(MT) hipLaunchKernelGGL((gemm_bf16_skinny64_kernel<MT, OUT_BF16, NORM_NONE>), grid, block, 0, stream, X, W, (void*)nullptr, \
+                                  M, N, K, p.chunks_per_slice, ws, true, (const float*)nullptr, 0, 0.f)
+    if (mt == 2) GO(2); else if (mt == 3) GO(3); else GO(4);
+#undef GO
+    int rc = launch_status();
+    if (rc) return rc;
+    hipLaunchKernelGGL((splitk_finish_conv_kernel<NORM>), dim3(ceil_div(d, 64), ceil_div(M, FC_ROWS)), dim3(FC_ROWS * 16), 0, stream,
+                       (const float*)ws, Y, M, d, mt * 16, p.slices, ex, cv);
     return launch_status();
 }
 
@@ -1341,6 +1456,26 @@ TUFF_EXPORT int tuff_gemm_bf16_scaled(const void* XW, const float* ss, int n_ss,
 // norm_kind 0: X is bfloat16 [M, K];  1: X is the float32 residual stream and the RMSNorm (norm_w,
 // eps; K <= 8192) runs inside;  2: X is bf16(x * norm weight) and ss [n_ss][16] the sums of squares
 // that tuff_gemm_bf16_accum_emit left.
+// The same for 17 to 64 rows, in two kernels (the projection's partial tiles, then the kernel that adds
+// them and runs the convolution), from the projection as the checkpoint has it: W [3 d, K] tile-major,
+// rows B | C | X.  X: bfloat16 [M, K], or with ss [n_ss][64] (and eps) bf16(x * norm weight) and the sums of
+// squares that tuff_gemm_bf16_accum_emit left for these M rows.  ws: tuff_gemm_bf16_workspace(M, 3 d, K, 1).
+TUFF_EXPORT int tuff_gemm_bf16_conv64(const void* X, const float* ss, int n_ss, float eps, const void* W, void* Y,
+                                      int M, int d, int K, const void* taps, int taps_dt, int n_taps, float* state,
+                                      const int* state_slot, float* ws, hipStream_t stream) {
+    if (M <= 0 || d <= 0) return 0;
+    if (K % 8 != 0 || M <= 16 || M > 64 || d % 16 != 0 || n_taps < 2 || n_taps - 1 > CONV_MAX_TAPS) return -2;
+    ConvTail cv;
+    cv.taps_w = taps; cv.taps_dt = taps_dt; cv.taps = n_taps; cv.state = state; cv.state_slot = state_slot;
+    FinishExtra x;
+    if (ss) {
+        if (n_ss < 1) return -2;
+        x.ss_in = ss; x.n_ss = n_ss; x.eps = eps; x.K = K;
+        return launch_skinny64_conv<NORM_SCALED>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, d, K, ws, x, cv, stream);
+    }
+    return launch_skinny64_conv<NORM_NONE>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, d, K, ws, x, cv, stream);
+}
+
 TUFF_EXPORT int tuff_gemm_bf16_conv(const void* X, int norm_kind, const float* norm_w, float eps, const float* ss, int n_ss,
                                     const void* W, void* Y, int M, int d, int K,
                                     const void* taps, int taps_dt, int n_taps, float* state, const int* state_slot,

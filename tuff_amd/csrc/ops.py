@@ -49,6 +49,8 @@ _SIGNATURES = {
                                   _c_int, _c_void_p, _c_void_p],
         "tuff_gemm_bf16_conv": [_c_void_p, _c_int, _c_void_p, _c_float, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int,
                                 _c_int, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
+        "tuff_gemm_bf16_conv64": [_c_void_p, _c_void_p, _c_int, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                                  _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
         "tuff_gemm_bf16_normed": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
                                   _c_int, _c_void_p],
     },
@@ -479,6 +481,37 @@ def gemm_conv(x: torch.Tensor, w, out: torch.Tensor, *, conv_w: torch.Tensor, st
     _check(load("gemm_bf16").tuff_gemm_bf16_conv(
         x.data_ptr(), kind, nw_ptr, float(eps), ss_ptr, n_ss, w.data_ptr(), out.data_ptr(), M, d, K,
         conv_w.data_ptr(), _dt(conv_w), taps, state.data_ptr(), state_slot.data_ptr(), _stream()), "gemm_bf16_conv")
+
+
+CONV64_MAX_ROWS = 64                          # gemm_conv64: one token a row
+
+
+def gemm_conv64(x: torch.Tensor, w, out: torch.Tensor, *, conv_w: torch.Tensor, state: torch.Tensor, state_slot: torch.Tensor,
+                eps: float = 0.0, ss: Optional[torch.Tensor] = None) -> None:
+    """gemm_conv for 17 to 64 rows, in two kernels (the projection's partial tiles; the kernel that adds
+    them and runs the convolution), without the projected rows ever being written.  w: the projection
+    [3 d, K] as the checkpoint has it (B | C | X), tiled.  x: bfloat16 [M, K], or bf16(x * norm weight)
+    with ss [tiles][64] and eps as gemm_accum_emit leaves them for these rows."""
+    M, K = x.shape
+    d = out.shape[1]
+    taps = conv_w.shape[1]
+    _gpu("x", x, torch.bfloat16)
+    _gpu("out", out, torch.bfloat16, (M, d))
+    w = _tiled(w, 3 * d, K)
+    _gpu("conv_w", conv_w, shape=(d, taps))
+    _gpu("state", state, torch.float32, (None, taps - 1, d))
+    _gpu("state_slot", state_slot, torch.int32, (M,))
+    if not 16 < M <= CONV64_MAX_ROWS or K % 8 or d % 16 or not 2 <= taps <= 17:
+        raise KernelError(f"gemm_conv64: 17 to {CONV64_MAX_ROWS} rows, an inner size that is a multiple of 8, a width that is "
+                          f"a multiple of 16 and 2 to 17 taps; got {M} rows, inner size {K}, width {d}, {taps} taps")
+    ss_ptr, n_ss = None, 0
+    if ss is not None:
+        _gpu("ss", ss, torch.float32, (None, 64))
+        ss_ptr, n_ss = ss.data_ptr(), ss.shape[0]
+    ws = _gemm_workspace(M, 3 * d, K, x.device, emit=True)
+    _check(load("gemm_bf16").tuff_gemm_bf16_conv64(
+        x.data_ptr(), ss_ptr, n_ss, float(eps), w.data_ptr(), out.data_ptr(), M, d, K,
+        conv_w.data_ptr(), _dt(conv_w), taps, state.data_ptr(), state_slot.data_ptr(), ws.data_ptr(), _stream()), "gemm_bf16_conv64")
 
 
 _plans: dict = {}

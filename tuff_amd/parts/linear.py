@@ -81,26 +81,31 @@ class Linear:
 
     def forward_conv(self, x, *, conv_w, state, state_slot) -> Optional[torch.Tensor]:
         """x as for forward(), one token a row.  Returns C * conv(B * X) [T, out / 3] in bfloat16 with the
-        states shifted, or None where this needs the separate kernels (nothing is touched then)."""
+        states shifted, or None where this needs the separate kernels (nothing is touched then).  Up to 16
+        rows: one kernel, from the regrouped weight; 17 to 64 rows: the kernel that adds the projection's
+        partial tiles runs the convolution."""
         from .norm import PendingNorm
         if self.weight_grouped is None:
             return None
         pending = x if isinstance(x, PendingNorm) else None
         T = pending.shape[0] if pending is not None else x.shape[0]
-        if T > ops.CONV_MAX_ROWS:
+        if T > ops.CONV64_MAX_ROWS:
             return None
         kw = {}
         if pending is not None:
             if pending.pre is not None:
                 x, kw = pending.pre[0], dict(ss=pending.pre[1], eps=pending.norm.eps)
-            elif pending.rows is None and self.in_features <= ops.NORMED_MAX_K:
+            elif T <= ops.CONV_MAX_ROWS and pending.rows is None and self.in_features <= ops.NORMED_MAX_K:
                 x, kw = pending.x, dict(norm_w=pending.norm.weight_f32, eps=pending.norm.eps)
             else:
                 x = pending.tensor()
         if not kw and x.dtype != torch.bfloat16:
             return None
         y = torch.empty(T, self.out_features // 3, dtype=torch.bfloat16, device=self.weight_grouped.device)
-        ops.gemm_conv(x, self.weight_grouped, y, conv_w=conv_w, state=state, state_slot=state_slot, **kw)
+        if T <= ops.CONV_MAX_ROWS:
+            ops.gemm_conv(x, self.weight_grouped, y, conv_w=conv_w, state=state, state_slot=state_slot, **kw)
+        else:
+            ops.gemm_conv64(x, self.weight, y, conv_w=conv_w, state=state, state_slot=state_slot, **kw)
         return y
 
     def forward(self, x, *, out_dtype: Optional[torch.dtype] = None,
