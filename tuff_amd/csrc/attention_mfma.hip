@@ -211,6 +211,10 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
         if (!live || k >= hd) return z;
         return __builtin_nontemporal_load((const bf16x8*)(k_cache + base + (long long)(off0 + k_off + 4 * kb) * hd + k));
     };
+    // A page's V^T rows are 2 * page_size bytes: with pages of 16 positions a step of 32 keys reads whole rows and
+    // never comes back to them; with larger pages it reads a part of each row's cache lines and the steps after it
+    // read the rest, so those loads are ordinary ones (a line asked for as streaming does not wait for them).
+    const bool stream_v = page_size <= 16;
     auto v_frag = [&](const Tile& t, int db) {
         const int dim = db * 16 + n16;
         bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -218,7 +222,8 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
         const long long base = (g / 2) ? t.base[1] : t.base[0];
         const int off0 = (g / 2) ? t.off0[1] : t.off0[0];
         if (!live || dim >= hd) return z;
-        return __builtin_nontemporal_load((const bf16x8*)(v_cache + base + (long long)dim * page_size + off0 + (g % 2) * 8));
+        const bf16x8* at = (const bf16x8*)(v_cache + base + (long long)dim * page_size + off0 + (g % 2) * 8);
+        return stream_v ? __builtin_nontemporal_load(at) : *at;
     };
     auto load_tile = [&](int key0, Tile& t) {
 #pragma unroll
