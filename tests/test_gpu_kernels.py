@@ -41,7 +41,7 @@ def test_gemm_f32(gpu, M, N, K):
                                    (200, 300, 328), (300, 64, 2048), (128, 128, 64), (2, 2048, 8192),
                                    (72, 2048, 8192), (512, 2050, 2048), (130, 1026, 1000),
                                    (33, 100, 2048), (64, 2048, 8192), (20, 64, 1024), (48, 200, 512), (16, 24, 4096),
-                                   (8, 6144, 2048),
+                                   (8, 6144, 2048), (32, 6144, 2048), (24, 2048, 8192), (31, 40, 72), (32, 16400, 2048),
                                    # each shape of block of the tiled kernel, with ragged edges and a partial last step
                                    (1100, 8200, 72), (1030, 8190, 136), (1100, 4001, 200), (257, 129, 520),
                                    # the same with K a multiple of 64: operands go straight into LDS
@@ -75,7 +75,7 @@ def test_gemm_bf16(gpu, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 32, 64), (8, 512, 240), (16, 6144, 2048), (5, 200, 96), (64, 384, 256),
-                                   (40, 2050, 2048), (300, 130, 136), (2048, 512, 128), (1100, 8200, 72),
+                                   (40, 2050, 2048), (24, 2050, 2048), (32, 16384, 2048), (300, 130, 136), (2048, 512, 128), (1100, 8200, 72),
                                    (200, 384, 1024), (72, 4100, 2048),
                                    (1030, 8202, 136), (1100, 4002, 200), (1030, 8202, 128), (1100, 4002, 192), (120, 13826, 1536)])
 def test_gemm_bf16_swiglu_epilogue(gpu, M, N, K):
@@ -127,7 +127,7 @@ def test_gemm_with_the_norm_inside(gpu, M, N, K, use_rows):
 
 
 @pytest.mark.parametrize("M,d,K1,N2", [(1, 64, 192, 512), (8, 2048, 8192, 6144), (16, 240, 328, 777 * 2), (5, 96, 96, 40),
-                                       (17, 96, 96, 40), (40, 2048, 8192, 6144), (64, 240, 328, 777 * 2), (33, 64, 192, 512),
+                                       (17, 96, 96, 40), (32, 2048, 8192, 6144), (24, 240, 328, 777 * 2), (40, 2048, 8192, 6144), (64, 240, 328, 777 * 2), (33, 64, 192, 512),
                                        (64, 2048, 2048, 65536)])
 def test_gemm_that_prepares_the_next_norm(gpu, M, d, K1, N2):
     """residual += a @ w1.T leaves bf16(residual * norm weight) and per-tile row sums of squares;
@@ -1052,13 +1052,16 @@ def test_shortconv_long_portions_equal_single_tokens(gpu, d, K):
     assert torch.equal(s1, s2)
 
 
-@pytest.mark.parametrize("M,d,K,taps", [(1, 64, 64, 3), (8, 2048, 2048, 3), (16, 240, 328, 4), (5, 48, 96, 2), (3, 96, 8192, 7)])
+@pytest.mark.parametrize("M,d,K,taps", [(1, 64, 64, 3), (8, 2048, 2048, 3), (16, 240, 328, 4), (5, 48, 96, 2), (3, 96, 8192, 7),
+                                        (17, 64, 64, 3), (32, 2048, 2048, 3), (24, 240, 328, 4), (20, 96, 8192, 7)])
 @pytest.mark.parametrize("norm", ["none", "inside", "scaled"])
 def test_gemm_with_the_convolution_in_its_epilogue(gpu, M, d, K, taps, norm):
     """Input projection and gated short convolution of single tokens in one kernel, against the plain
     formulas on the same bfloat16 inputs: out = C * conv(B * X) over each row's state, and the state
     shifted by u = B * X.  With the norm inside the product and with the row scales another product left."""
     from tuff_amd.csrc import ops
+    if norm == "inside" and M > 16:
+        pytest.skip("the norm inside the product is for at most 16 rows")
     eps = 1e-5
     w_in = _r(3 * d, K, seed=1, scale=K ** -0.5, dtype=torch.bfloat16)
     conv_w = _r(d, taps, seed=2, scale=0.5, dtype=torch.bfloat16)
@@ -1080,7 +1083,7 @@ def test_gemm_with_the_convolution_in_its_epilogue(gpu, M, d, K, taps, norm):
     else:
         xw = (x32 * nw).to(torch.bfloat16)
         tiles = 5
-        ss = torch.zeros(tiles, 16)
+        ss = torch.zeros(tiles, 16 if M <= 16 else 64)
         cut = [K * t // tiles for t in range(tiles + 1)]
         for t in range(tiles):
             ss[t, :M] = (x32[:, cut[t]:cut[t + 1]] ** 2).sum(-1)
@@ -1101,15 +1104,15 @@ def test_gemm_with_the_convolution_in_its_epilogue(gpu, M, d, K, taps, norm):
     others = torch.ones(M + 3, dtype=torch.bool)
     others[slots.long()] = False
     assert torch.equal(new_state[others], state0[others].double())      # nobody else's state was touched
-    with pytest.raises(ops.KernelError, match="at most 16 rows"):
-        ops.gemm_conv(torch.zeros(17, K, dtype=torch.bfloat16, device=gpu), w, torch.empty(17, d, dtype=torch.bfloat16, device=gpu),
-                      conv_w=conv_w.to(gpu), state=state, state_slot=torch.zeros(17, dtype=torch.int32, device=gpu))
+    with pytest.raises(ops.KernelError, match="at most 32 rows"):
+        ops.gemm_conv(torch.zeros(33, K, dtype=torch.bfloat16, device=gpu), w, torch.empty(33, d, dtype=torch.bfloat16, device=gpu),
+                      conv_w=conv_w.to(gpu), state=state, state_slot=torch.zeros(33, dtype=torch.int32, device=gpu))
 
 
-@pytest.mark.parametrize("M,d,K,taps", [(17, 64, 64, 3), (64, 2048, 2048, 3), (33, 240, 328, 4), (48, 48, 96, 2), (20, 96, 8192, 7)])
+@pytest.mark.parametrize("M,d,K,taps", [(33, 64, 64, 3), (64, 2048, 2048, 3), (40, 240, 328, 4), (48, 48, 96, 2), (50, 96, 8192, 7)])
 @pytest.mark.parametrize("norm", ["none", "scaled"])
 def test_gemm_with_the_convolution_in_the_kernel_that_adds_its_slices(gpu, M, d, K, taps, norm):
-    """17 to 64 single tokens: the kernel that adds the projection's partial tiles runs the convolution.
+    """33 to 64 single tokens: the kernel that adds the projection's partial tiles runs the convolution.
     Against the plain formulas, and bit for bit against the projection followed by the kernel for single
     tokens (the same sums in the same order, rounded to bfloat16 at the same place)."""
     from tuff_amd.csrc import ops

@@ -7,23 +7,25 @@
 // instead of 64 bytes from each of sixteen rows that lie a whole row apart; measured on streams of
 // the shapes of a decode step, the run-wise reads are 17 % faster.
 //
-// Three kernels, chosen by M on the host:
+// Three kernels, chosen by the sizes on the host:
 //  * tiled     M > 64: 128x128 or 256x256 block tiles staged through LDS (compute bound), in two
 //    forms: operands loaded straight into LDS (K a multiple of 64) or through registers (other K);
-//  * skinny64  16 < M <= 64: a workgroup owns 64 rows of W, one MFMA column tile a wave; the
-//    activations of a K chunk are staged once in LDS for all four waves (bandwidth bound);
-//  * skinny16  M <= 16: a workgroup owns 16 rows of W; its four waves split K (bandwidth bound).
+//  * skinny64  up to 64 rows that skinny16 does not take: a workgroup owns 64 rows of W, one MFMA column
+//    tile a wave; the activations of a K chunk are staged once in LDS for all four waves (bandwidth bound);
+//  * skinny16  M <= 16, and up to 32 rows (two row tiles a wave) where few_rows_kernel() says so:
+//    a workgroup owns 8 to 64 rows of W; its waves split K (bandwidth bound), no barrier in the loop.
 // The skinny kernels stream each weight byte once from HBM straight into MFMA operands.  Where
 // N alone gives too little parallelism to fill 256 CUs, skinny16 uses more waves a workgroup
 // (8 or 16, partials added in wave order through LDS) and skinny64 splits K over workgroups
 // (partial tiles in a work space, added in slice order by a second kernel, which also does the
-// epilogue).  The cut depends
-// on N and K only, never on M, so the order of additions is fixed.
+// epilogue).  Within a kernel the cut depends on N and K only (and on whether M is beyond 16), so the
+// order of additions is fixed.
 //
 // All use v_mfma_f32_16x16x32_bf16.  Lane l of a wave supplies row (l % 16) of an operand tile
 // and eight consecutive k at 8 * (l / 16); it receives rows 4 * (l / 16) + 0..3, column (l % 16)
 // of the 16x16 result.
 #include "common.h"
+#include <stdlib.h>
 
 // OUT_SWIGLU: the rows of W are gate and up rows interleaved (2f: gate f, 2f+1: up f); the
 // output is bfloat16 [M, N/2] with y[m, f] = silu(g) * u, silu(g) = g / (1 + exp(-g)).
@@ -543,7 +545,12 @@ struct ConvTail {
     }
 };
 
-template <int NW, int MODE, int NORM, bool EMIT, int COLS>
+// MT: row tiles of 16 (1: up to 16 rows, 2: up to 32).  With two, a wave multiplies every block of W
+// with two tiles of X rows; the sums of squares that go from product to product then have 64 rows a tile
+// in memory (SS_ROWS), as for every product of 17 to 64 rows.
+constexpr int SS_ROWS_WIDE = 64;
+
+template <int NW, int MODE, int NORM, bool EMIT, int COLS, int MT>
 __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const void* __restrict__ Xv, const bf16_t* __restrict__ W,
                                                                        void* __restrict__ Y, int M, int N, int K,
                                                                        const float* __restrict__ norm_w, float eps,
@@ -554,10 +561,15 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
                                                                        ConvTail cv) {
     constexpr bool CONV = MODE == OUT_CONV;
     static_assert(!CONV || COLS == 8, "the convolution's epilogue takes eight channels a workgroup");
+    static_assert(MT == 1 || NORM != NORM_INSIDE, "the norm inside is for at most 16 rows");
     constexpr int TN = CONV ? 3 : (COLS > 16 ? COLS / 16 : 1);           // MFMA tiles side by side: they share the rows of X
     static_assert(!EMIT || TN == 1, "the emitting epilogue works on one tile");
-    __shared__ float red[TN][NW][WAVE][4];
-    __shared__ float ssq[16][16];                                        // [wave or part][row]
+    constexpr int ROWS = 16 * MT;
+    constexpr int SSR = MT == 1 ? 16 : SS_ROWS_WIDE;                     // rows of a tile of sums of squares in memory
+    constexpr int NT_ = NW * WAVE;
+    constexpr int PAIRS = (16 * ROWS + NT_ - 1) / NT_;                   // (row, part) sums a thread adds for NORM_SCALED
+    __shared__ float red[MT][TN][NW][WAVE][4];
+    __shared__ float ssq[16][ROWS];                                      // [wave or part][row]
     extern __shared__ __attribute__((aligned(16))) float nw_lds[];       // NORM_INSIDE: the norm weight, K floats
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
     const int r16 = lane % 16, g = lane / 16;
@@ -575,29 +587,39 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
     if (NORM == NORM_INSIDE && r16 < M) xrow = (const float*)Xv + (long long)(rows ? rows[r16] : r16) * K;
 
     // What the epilogue adds to is read now, not after the last product: a load at the end would
-    // cost one more trip to memory.
-    float y_old[TN], emit_w = 0.f;
+    // cost one more trip to memory.  (Thread t of every 256 -> element (row (t / 64) * 4 + t % 4,
+    // column (t / 4) % 16) of a 16 x 16 tile; the groups of 256 threads take the row tiles in turn.)
+    constexpr int EPI_GROUPS = NT_ / 256;                                // groups of 256 threads a workgroup
+    constexpr int EPI_TILES = (MT + EPI_GROUPS - 1) / EPI_GROUPS;        // row tiles a group finishes
+    float y_old[EPI_TILES][TN], emit_w = 0.f;
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn) {
-        y_old[tn] = 0.f;
-        if (MODE == OUT_F32_ACCUM && tid < 256) {
-            const long long row = (tid / 64) * 4 + tid % 4, col = n0 + tn * 16 + (tid / 4) % 16;
-            if (row < M && col < w_rows) {
-                y_old[tn] = ((const float*)Y)[row * N + col];
-                if (EMIT) emit_w = emit_nw[col];
+    for (int i = 0; i < EPI_TILES; ++i) {
+        const int mt = tid / 256 + i * EPI_GROUPS;
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) {
+            y_old[i][tn] = 0.f;
+            if (MODE == OUT_F32_ACCUM && mt < MT) {
+                const int t = tid % 256;
+                const long long row = mt * 16 + (t / 64) * 4 + t % 4, col = n0 + tn * 16 + (t / 4) % 16;
+                if (row < M && col < w_rows) {
+                    y_old[i][tn] = ((const float*)Y)[row * N + col];
+                    if (EMIT) emit_w = emit_nw[col];
+                }
             }
         }
     }
 
-    f32x4 acc[TN];
+    f32x4 acc[MT][TN];
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn) acc[tn] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) acc[mt][tn] = f32x4{0.f, 0.f, 0.f, 0.f};
     float ss = 0.f;
-    struct Operands { bf16x8 a[4]; bf16x8 b[TN][4]; f32x4 x[NORM == NORM_INSIDE ? 4 : 1][2]; };
+    struct Operands { bf16x8 a[MT][4]; bf16x8 b[TN][4]; f32x4 x[NORM == NORM_INSIDE ? 4 : 1][2]; };
     Operands o0, o1;
     auto load = [&](int c, Operands& o) {
         // instruction j of the wave reads block 4 c + j of its row tile (1 KB) and bytes 64 j .. 64 j + 63 of
-        // the chunk of each of the 16 rows of X
+        // the chunk of each of the rows of X
         const int k0 = c * SK_CHUNK + g * 8;
         const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
@@ -613,7 +635,8 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
                 o.x[j][0] = ok ? *(const f32x4*)(xrow + k) : f32x4{0.f, 0.f, 0.f, 0.f};
                 o.x[j][1] = ok ? *(const f32x4*)(xrow + k + 4) : f32x4{0.f, 0.f, 0.f, 0.f};
             } else {
-                o.a[j] = load8(X, r16, M, k, K);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) o.a[mt][j] = load8(X, mt * 16 + r16, M, k, K);
             }
         }
     };
@@ -629,15 +652,17 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
                     const float x0 = o.x[j][0][e], x1 = o.x[j][1][e];
                     ss = fmaf(x0, x0, ss);
                     ss = fmaf(x1, x1, ss);
-                    o.a[j][e] = (bf16_t)(x0 * w0[e]);
-                    o.a[j][4 + e] = (bf16_t)(x1 * w1[e]);
+                    o.a[0][j][e] = (bf16_t)(x0 * w0[e]);
+                    o.a[0][j][4 + e] = (bf16_t)(x1 * w1[e]);
                 }
             }
         }
 #pragma unroll
-        for (int tn = 0; tn < TN; ++tn)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[tn] = mfma16(o.a[j], o.b[tn][j], acc[tn]);
+            for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[mt][tn] = mfma16(o.a[mt][j], o.b[tn][j], acc[mt][tn]);
     };
     // Workgroups start at different chunks (a rotation by the tile index), so that at any moment
     // the chip reads from all columns of W and not from one.  The order of a tile's additions
@@ -651,15 +676,22 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
         for (int k = tid * 4; k < K; k += NW * WAVE * 4) *(f32x4*)(&nw_lds[k]) = *(const f32x4*)(norm_w + k);
         __syncthreads();
     }
-    // NORM_SCALED: 16 parts x 16 rows; part p adds the tiles p, p + 16, ... of its row.  The first
+    // NORM_SCALED: 16 parts x ROWS rows; part p adds the tiles p, p + 16, ... of its row.  The first
     // sixteen of them are only asked for here and added after the products, when they have long
     // arrived; a wider matrix adds the rest right away.
-    float ss_part[16], ss_rest = 0.f;
-    if (NORM == NORM_SCALED && tid < 256) {
-        const int row = tid % 16, part = tid / 16;
+    float ss_part[PAIRS][16], ss_rest[PAIRS];
+    if (NORM == NORM_SCALED) {
 #pragma unroll
-        for (int u = 0; u < 16; ++u) ss_part[u] = (part + 16 * u < n_ss) ? ss_in[(long long)(part + 16 * u) * 16 + row] : 0.f;
-        for (int j = part + 256; j < n_ss; j += 16) ss_rest += ss_in[(long long)j * 16 + row];
+        for (int q = 0; q < PAIRS; ++q) {
+            const int pr = tid + q * NT_;
+            const int row = pr % ROWS, part = pr / ROWS;
+            ss_rest[q] = 0.f;
+            if (pr < 16 * ROWS) {
+#pragma unroll
+                for (int u = 0; u < 16; ++u) ss_part[q][u] = (part + 16 * u < n_ss) ? ss_in[(long long)(part + 16 * u) * SSR + row] : 0.f;
+                for (int j = part + 256; j < n_ss; j += 16) ss_rest[q] += ss_in[(long long)j * SSR + row];
+            }
+        }
     }
     for (; i < nchunks; i += 2 * NW) {
         const bool more = i + NW < nchunks;
@@ -671,14 +703,22 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
         }
     }
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) red[tn][wave][lane][e] = acc[tn][e];
-    if (NORM == NORM_SCALED && tid < 256) {
-        float t = ss_rest;
+        for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-        for (int u = 0; u < 16; ++u) t += ss_part[u];
-        ssq[tid / 16][tid % 16] = t;
+            for (int e = 0; e < 4; ++e) red[mt][tn][wave][lane][e] = acc[mt][tn][e];
+    if (NORM == NORM_SCALED) {
+#pragma unroll
+        for (int q = 0; q < PAIRS; ++q) {
+            const int pr = tid + q * NT_;
+            if (pr < 16 * ROWS) {
+                float t = ss_rest[q];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) t += ss_part[q][u];
+                ssq[pr / ROWS][pr % ROWS] = t;
+            }
+        }
     }
     if (NORM == NORM_INSIDE) {
         ss += __shfl_xor(ss, 16, WAVE);
@@ -686,16 +726,20 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
         if (g == 0) ssq[wave][r16] = ss;
     }
     __syncthreads();
-    if (tid < 256) {
+#pragma unroll
+    for (int ei = 0; ei < EPI_TILES; ++ei) {
+        const int mt = tid / 256 + ei * EPI_GROUPS;
+        if (mt >= MT) break;
         // thread -> (lane l, element e) of each 16x16 tile; the wave partials in wave order
-        const int e = tid % 4, l = tid / 4;
+        const int t256 = tid % 256;
+        const int e = t256 % 4, l = t256 / 4;
+        const int trow = mt * 16 + (l / 16) * 4 + e;                     // the thread's row of the product
         float scale = 1.f;
         if (NORM != NORM_NONE) {
             constexpr int PARTS = NORM == NORM_INSIDE ? NW : 16;
-            const int row = (l / 16) * 4 + e;
-            float total = ssq[0][row];
+            float total = ssq[0][trow];
 #pragma unroll
-            for (int w = 1; w < PARTS; ++w) total += ssq[w][row];
+            for (int w = 1; w < PARTS; ++w) total += ssq[w][trow];
             scale = 1.0f / sqrtf(total / (float)K + eps);
         }
         if constexpr (CONV) {
@@ -704,13 +748,13 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
             float bcx[3];
 #pragma unroll
             for (int tn = 0; tn < 3; ++tn) {
-                float v = red[tn][0][l][e];
+                float v = red[mt][tn][0][l][e];
 #pragma unroll
-                for (int w = 1; w < NW; ++w) v += red[tn][w][l][e];
+                for (int w = 1; w < NW; ++w) v += red[mt][tn][w][l][e];
                 if (NORM != NORM_NONE) v *= scale;
                 bcx[tn] = (float)(bf16_t)v;
             }
-            const int row = (l / 16) * 4 + e, d = N / 3, Kc = cv.taps;
+            const int row = trow, d = N / 3, Kc = cv.taps;
             const int ch = (int)(blockIdx.x) * 8 + (l % 16);
             if ((l % 16) < 8 && row < M && ch < d) {
                 float* st = cv.state + (long long)cv.state_slot[row] * (Kc - 1) * d;
@@ -733,35 +777,35 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
                 st[(long long)(Kc - 2) * d + ch] = u;
                 ((bf16_t*)Y)[(long long)row * d + ch] = (bf16_t)(bcx[1] * y);
             }
-            return;
+            continue;
         }
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
-            float v = red[tn][0][l][e];
+            float v = red[mt][tn][0][l][e];
 #pragma unroll
-            for (int w = 1; w < NW; ++w) v += red[tn][w][l][e];
+            for (int w = 1; w < NW; ++w) v += red[mt][tn][w][l][e];
             const long long col = n0 + tn * 16 + (l % 16);
-            const long long row = col < w_rows ? (l / 16) * 4 + e : 16;     // columns beyond the tile: no row
+            const long long row = col < w_rows ? trow : ROWS;                // columns beyond the tile: no row
             if (NORM != NORM_NONE) v *= scale;
             if (EMIT) {
                 // y += v; the new y also as the next norm's operand, and its square into the row's tile sum
                 float y = 0.f;
                 if (row < M && col < N) {
-                    y = y_old[tn] + v;
+                    y = y_old[ei][tn] + v;
                     ((float*)Y)[row * N + col] = y;
                     emit_xw[row * N + col] = (bf16_t)(y * emit_w);
                 }
-                float sq = y * y;                       // tid = (16 q + c) * 4 + e: the 16 columns c are tid bits 2..5
+                float sq = y * y;                       // t256 = (16 q + c) * 4 + e: the 16 columns c are its bits 2..5
                 sq += __shfl_xor(sq, 4, WAVE);
                 sq += __shfl_xor(sq, 8, WAVE);
                 sq += __shfl_xor(sq, 16, WAVE);
                 sq += __shfl_xor(sq, 32, WAVE);
-                if ((l % 16) == 0 && row < 16) emit_ss[(long long)blockIdx.x * 16 + row] = sq;
+                if ((l % 16) == 0 && row < ROWS) emit_ss[(long long)blockIdx.x * SSR + row] = sq;
             } else if (MODE == OUT_F32_ACCUM) {
-                if (row < M && col < N) ((float*)Y)[row * N + col] = y_old[tn] + v;
+                if (row < M && col < N) ((float*)Y)[row * N + col] = y_old[ei][tn] + v;
             } else {
-                const float partner = (MODE == OUT_SWIGLU) ? __shfl_xor(v, 4, WAVE) : 0.f;   // thread tid ^ 4 holds column col ^ 1
-                store_elem<MODE>(Y, row, col, min(M, 16), N, v, partner);
+                const float partner = (MODE == OUT_SWIGLU) ? __shfl_xor(v, 4, WAVE) : 0.f;   // thread t ^ 4 holds column col ^ 1
+                store_elem<MODE>(Y, row, col, min(M, ROWS), N, v, partner);
             }
         }
     }
@@ -1066,13 +1110,30 @@ __global__ __launch_bounds__(FC_ROWS * 16) void splitk_finish_conv_kernel(const 
 
 struct SkinnyPlan { int tiles, waves, slices, chunks_per_slice, cols; long long ws_floats; };
 
+constexpr int SKINNY_ROWS = 32;     // the most rows of the kernel whose waves split K inside the workgroup (two row tiles)
+
+// Whether a product of M rows goes through that kernel (else, up to 64 rows: K cut over workgroups and a
+// second kernel that adds the slices).  Up to 16 rows always.  17 to 32 rows: every workgroup reads all M
+// rows of X again, M / (its columns) times the bytes of its share of W, and has half the waves; measured
+// on the shapes of a 1.2B model (against the two kernels of the other way, at 32 rows): 2,048 columns
+// 14.8 us against 11.9, 3,072 columns 8.8 against 10.7, a conv's input projection with the convolution
+// 12.5 against 15.2, 16,384 columns 21.7 against 21.3, 65,536 columns 67.7 against 52.2; at 17 rows
+// it wins everywhere.  So: narrow outputs up to 20 rows, medium ones up to 32, wide ones up to 24.
+bool few_rows_kernel(int M, int N, int K, bool conv = false) {
+    (void)K;
+    if (M <= 16) return true;
+    if (M > SKINNY_ROWS) return false;
+    if (conv) return true;
+    return N <= 2048 ? M <= 20 : N <= 8192 ? true : M <= 24;
+}
+
 // How a skinny product is cut.  Depends on N and K (and on which of the two kernels M selects).
-SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16, bool emit = false) {
+SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16, bool emit = false, bool conv = false) {
     const int nchunks = ceil_div(K, SK_CHUNK);
     SkinnyPlan p;
     p.slices = 1; p.chunks_per_slice = nchunks; p.ws_floats = 0; p.waves = 4;
     p.cols = 16;
-    if (M <= 16) {
+    if (few_rows_kernel(M, N, K, conv)) {
         // Narrow outputs: tiles of 8 columns, where 16 would leave CUs without a workgroup (half of
         // each MFMA idles, which costs nothing here: these products wait for memory).  Wide outputs:
         // 32 or 64 columns, whose MFMA tiles share the rows of X: with 16 columns the rows of X
@@ -1083,6 +1144,11 @@ SkinnyPlan plan_skinny(int M, int N, int K, int max_waves = 16, bool emit = fals
         else if (tiles16 >= 512) p.cols = 32;
         if ((max_waves < 16 || emit) && p.cols > 16) p.cols = 16;       // the norm inside keeps float32 rows in registers;
                                                                         // the emitting epilogue works on one tile
+        if (M > 16) {
+            // two row tiles: twice the operands of X a wave, so at most two tiles of W side by side and eight waves
+            p.cols = min(p.cols, 32);
+            max_waves = min(max_waves, 8);
+        }
         p.tiles = ceil_div(N, p.cols);
         // enough waves in flight to cover the latency of HBM, at least one chunk a wave
         while (p.waves < max_waves && p.tiles * p.waves < 3072 && nchunks >= 2 * p.waves) p.waves *= 2;
@@ -1145,11 +1211,17 @@ struct Skinny16Extra {
 template <int MODE, int NORM, bool EMIT>
 int launch_skinny16(const void* X, const bf16_t* W, void* Y, int M, int N, int K, const Skinny16Extra& x, hipStream_t stream) {
     // the in-kernel norm needs more registers a wave: at most 8 waves a workgroup
-    SkinnyPlan p = plan_skinny(M, N, K, NORM == NORM_INSIDE ? 8 : 16, EMIT);
+    SkinnyPlan p = plan_skinny(M, N, K, NORM == NORM_INSIDE ? 8 : 16, EMIT, MODE == OUT_CONV);
     const size_t lds = NORM == NORM_INSIDE ? (size_t)K * sizeof(float) : 0;
-#define GO(NW, COLS) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<NW, MODE, NORM, EMIT, COLS>), grid, dim3(NW * WAVE), lds, stream, \
+    const int mt = M > 16 ? 2 : 1;
+#define GO_MT(NW, COLS, MT) hipLaunchKernelGGL((gemm_bf16_skinny16_kernel<NW, MODE, NORM, EMIT, COLS, MT>), grid, dim3(NW * WAVE), lds, stream, \
                                         X, W, Y, M, N, K, x.norm_w, x.eps, x.rows, x.ss_in, x.n_ss, x.emit_nw, x.emit_xw, x.emit_ss, \
                                         x.conv)
+#define GO(NW, COLS) do { \
+        if (mt == 1) GO_MT(NW, COLS, 1); \
+        else if constexpr (NW <= 8 && COLS <= 32 && NORM != NORM_INSIDE) GO_MT(NW, COLS, 2); \
+        else return -3; \
+    } while (0)
     if constexpr (MODE == OUT_CONV) {
         // eight channels a workgroup (three half tiles); the waves split K as always, at most eight of them:
         // sixteen would leave a wave 128 registers, too few for three tiles' operands of two chunks
@@ -1169,6 +1241,7 @@ int launch_skinny16(const void* X, const bf16_t* W, void* Y, int M, int N, int K
         } else return -3;
     }
 #undef GO
+#undef GO_MT
     return launch_status();
 }
 
@@ -1259,7 +1332,7 @@ template <int MODE, int AROUND = TILED_PLAIN>
 int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, float* ws, hipStream_t stream,
                 const TiledExtra& ex = TiledExtra()) {
     if constexpr (AROUND == TILED_PLAIN) {
-        if (M <= 16) return launch_skinny16<MODE, NORM_NONE, false>(X, W, Y, M, N, K, Skinny16Extra(), stream);
+        if (few_rows_kernel(M, N, K)) return launch_skinny16<MODE, NORM_NONE, false>(X, W, Y, M, N, K, Skinny16Extra(), stream);
         if (M <= 64) return launch_skinny64<MODE, NORM_NONE, false>(X, W, Y, M, N, K, ws, FinishExtra(), stream);
     }
     {
@@ -1343,7 +1416,7 @@ TUFF_EXPORT int tuff_gemm_bf16_emit_layout(int M, int N, int K, int* tiles, int*
         return 0;
     }
     *tiles = plan_skinny(M, N, K, 16, true).tiles;
-    *rows = M <= 16 ? 16 : 64;
+    *rows = M <= 16 ? 16 : 64;                          // (17 to 32 rows: the kernel for few rows, with tiles of 64 rows)
     return 0;
 }
 
@@ -1358,7 +1431,7 @@ TUFF_EXPORT int tuff_gemm_bf16_scaled_supported(int M, int N, int K) {
 // emit: for tuff_gemm_bf16_accum_emit.
 TUFF_EXPORT int tuff_gemm_bf16_workspace(int M, int N, int K, int emit, long long* ws_floats) {
     *ws_floats = 0;
-    if (M <= 16 || N <= 0) return 0;
+    if (N <= 0 || few_rows_kernel(M, N, K)) return 0;
     *ws_floats = M <= 64 ? plan_skinny(M, N, K, 16, emit != 0).ws_floats : plan_tiled(M, N, K).ws_floats;
     return 0;
 }
@@ -1407,7 +1480,7 @@ TUFF_EXPORT int tuff_gemm_bf16_accum_emit(const void* X, const void* W, float* Y
         t.emit_nw = next_norm_w; t.emit_xw = (bf16_t*)xw; t.emit_ss = ss;
         return launch_mode<OUT_F32_ACCUM, TILED_EMIT>((const bf16_t*)X, (const bf16_t*)W, Y, M, N, K, ws, stream, t);
     }
-    if (M <= 16) {
+    if (few_rows_kernel(M, N, K)) {
         Skinny16Extra x;
         x.emit_nw = next_norm_w; x.emit_xw = (bf16_t*)xw; x.emit_ss = ss;
         return launch_skinny16<OUT_F32_ACCUM, NORM_NONE, true>(X, (const bf16_t*)W, Y, M, N, K, x, stream);
@@ -1439,7 +1512,7 @@ TUFF_EXPORT int tuff_gemm_bf16_scaled(const void* XW, const float* ss, int n_ss,
         }
         return -3;
     }
-    if (M <= 16) {
+    if (few_rows_kernel(M, N, K)) {
         Skinny16Extra x;
         x.ss_in = ss; x.n_ss = n_ss; x.eps = eps;
         return launch_skinny16_mode<NORM_SCALED>(XW, (const bf16_t*)W, Y, M, N, K, mode, x, stream);
@@ -1464,7 +1537,7 @@ TUFF_EXPORT int tuff_gemm_bf16_conv64(const void* X, const float* ss, int n_ss, 
                                       int M, int d, int K, const void* taps, int taps_dt, int n_taps, float* state,
                                       const int* state_slot, float* ws, hipStream_t stream) {
     if (M <= 0 || d <= 0) return 0;
-    if (K % 8 != 0 || M <= 16 || M > 64 || d % 16 != 0 || n_taps < 2 || n_taps - 1 > CONV_MAX_TAPS) return -2;
+    if (K % 8 != 0 || M <= SKINNY_ROWS || M > 64 || d % 16 != 0 || n_taps < 2 || n_taps - 1 > CONV_MAX_TAPS) return -2;
     ConvTail cv;
     cv.taps_w = taps; cv.taps_dt = taps_dt; cv.taps = n_taps; cv.state = state; cv.state_slot = state_slot;
     FinishExtra x;
@@ -1481,7 +1554,8 @@ TUFF_EXPORT int tuff_gemm_bf16_conv(const void* X, int norm_kind, const float* n
                                     const void* taps, int taps_dt, int n_taps, float* state, const int* state_slot,
                                     hipStream_t stream) {
     if (M <= 0 || d <= 0) return 0;
-    if (K % 8 != 0 || M > 16 || d % 16 != 0 || n_taps < 2 || n_taps - 1 > CONV_MAX_TAPS) return -2;
+    if (K % 8 != 0 || M > SKINNY_ROWS || d % 16 != 0 || n_taps < 2 || n_taps - 1 > CONV_MAX_TAPS) return -2;
+    if (norm_kind == 1 && M > 16) return -2;
     Skinny16Extra x;
     x.conv.taps_w = taps; x.conv.taps_dt = taps_dt; x.conv.taps = n_taps; x.conv.state = state; x.conv.state_slot = state_slot;
     const bf16_t* w = (const bf16_t*)W;

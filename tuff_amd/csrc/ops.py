@@ -364,7 +364,7 @@ def gemm_emit_layout(M: int, N: int, K: int) -> Optional[tuple]:
     with N outputs and inner size K, or None where such a product cannot leave them (more than 64 rows
     and an inner size that is no multiple of 64, a product cut along K, a last block of columns that is
     not whole)."""
-    key = (M if M > EMIT_MAX_ROWS else M <= 16, N, K)
+    key = (M if M > 16 else 0, N, K)                   # (which kernel takes 17 to 64 rows depends on all three)
     if key not in _emit_layouts:
         t, r = _c_int(0), _c_int(0)
         _check(load("gemm_bf16").tuff_gemm_bf16_emit_layout(M, N, K, ctypes.byref(t), ctypes.byref(r)), "gemm_emit_layout")
@@ -433,7 +433,7 @@ def gemm_scaled(xw: torch.Tensor, ss: torch.Tensor, eps: float, w, out: torch.Te
                                                    None if ws is None else ws.data_ptr(), _stream()), "gemm_bf16_scaled")
 
 
-CONV_MAX_ROWS = 16                            # gemm_conv: one token a row
+CONV_MAX_ROWS = 32                            # gemm_conv: one token a row (the norm inside: at most NORMED_MAX_ROWS)
 
 
 def conv_group_rows(w_in: torch.Tensor) -> torch.Tensor:
@@ -450,7 +450,7 @@ def conv_group_rows(w_in: torch.Tensor) -> torch.Tensor:
 def gemm_conv(x: torch.Tensor, w, out: torch.Tensor, *, conv_w: torch.Tensor, state: torch.Tensor, state_slot: torch.Tensor,
               norm_w: Optional[torch.Tensor] = None, eps: float = 0.0, ss: Optional[torch.Tensor] = None) -> None:
     """Input projection and gated short convolution of single tokens (row r is request r's token, at
-    most 16 rows) in one kernel: out [M, d] bfloat16 = C * conv(B * X) with (B, C, X) = x @ w.T, and
+    most 32 rows) in one kernel: out [M, d] bfloat16 = C * conv(B * X) with (B, C, X) = x @ w.T, and
     the rows' states shifted.  w: conv_group_rows() of the projection, tiled.  x: bfloat16 [M, K]; or
     the float32 residual stream with norm_w and eps (the RMSNorm runs inside); or bf16(x * norm weight)
     with ss and eps as gemm_accum_emit leaves them."""
@@ -468,13 +468,14 @@ def gemm_conv(x: torch.Tensor, w, out: torch.Tensor, *, conv_w: torch.Tensor, st
     kind, nw_ptr, ss_ptr, n_ss = 0, None, None, 0
     if ss is not None:
         _gpu("x", x, torch.bfloat16)
-        _gpu("ss", ss, torch.float32, (None, 16))
+        _gpu("ss", ss, torch.float32, (None, 16 if M <= 16 else 64))
         kind, ss_ptr, n_ss = 2, ss.data_ptr(), ss.shape[0]
     elif norm_w is not None:
         _gpu("x", x, torch.float32)
         _gpu("norm_w", norm_w, torch.float32, (K,))
-        if K > NORMED_MAX_K:
-            raise KernelError(f"gemm_conv: the norm inside needs an inner size up to {NORMED_MAX_K}, got {K}")
+        if K > NORMED_MAX_K or M > NORMED_MAX_ROWS:
+            raise KernelError(f"gemm_conv: the norm inside needs an inner size up to {NORMED_MAX_K} and at most "
+                              f"{NORMED_MAX_ROWS} rows, got {K} and {M}")
         kind, nw_ptr = 1, norm_w.data_ptr()
     else:
         _gpu("x", x, torch.bfloat16)
@@ -488,7 +489,7 @@ CONV64_MAX_ROWS = 64                          # gemm_conv64: one token a row
 
 def gemm_conv64(x: torch.Tensor, w, out: torch.Tensor, *, conv_w: torch.Tensor, state: torch.Tensor, state_slot: torch.Tensor,
                 eps: float = 0.0, ss: Optional[torch.Tensor] = None) -> None:
-    """gemm_conv for 17 to 64 rows, in two kernels (the projection's partial tiles; the kernel that adds
+    """gemm_conv for 33 to 64 rows, in two kernels (the projection's partial tiles; the kernel that adds
     them and runs the convolution), without the projected rows ever being written.  w: the projection
     [3 d, K] as the checkpoint has it (B | C | X), tiled.  x: bfloat16 [M, K], or bf16(x * norm weight)
     with ss [tiles][64] and eps as gemm_accum_emit leaves them for these rows."""
@@ -501,8 +502,8 @@ def gemm_conv64(x: torch.Tensor, w, out: torch.Tensor, *, conv_w: torch.Tensor, 
     _gpu("conv_w", conv_w, shape=(d, taps))
     _gpu("state", state, torch.float32, (None, taps - 1, d))
     _gpu("state_slot", state_slot, torch.int32, (M,))
-    if not 16 < M <= CONV64_MAX_ROWS or K % 8 or d % 16 or not 2 <= taps <= 17:
-        raise KernelError(f"gemm_conv64: 17 to {CONV64_MAX_ROWS} rows, an inner size that is a multiple of 8, a width that is "
+    if not CONV_MAX_ROWS < M <= CONV64_MAX_ROWS or K % 8 or d % 16 or not 2 <= taps <= 17:
+        raise KernelError(f"gemm_conv64: {CONV_MAX_ROWS + 1} to {CONV64_MAX_ROWS} rows, an inner size that is a multiple of 8, a width that is "
                           f"a multiple of 16 and 2 to 17 taps; got {M} rows, inner size {K}, width {d}, {taps} taps")
     ss_ptr, n_ss = None, 0
     if ss is not None:

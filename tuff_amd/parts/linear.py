@@ -81,8 +81,8 @@ class Linear:
 
     def forward_conv(self, x, *, conv_w, state, state_slot) -> Optional[torch.Tensor]:
         """x as for forward(), one token a row.  Returns C * conv(B * X) [T, out / 3] in bfloat16 with the
-        states shifted, or None where this needs the separate kernels (nothing is touched then).  Up to 16
-        rows: one kernel, from the regrouped weight; 17 to 64 rows: the kernel that adds the projection's
+        states shifted, or None where this needs the separate kernels (nothing is touched then).  Up to 32
+        rows: one kernel, from the regrouped weight; 33 to 64 rows: the kernel that adds the projection's
         partial tiles runs the convolution."""
         from .norm import PendingNorm
         if self.weight_grouped is None:
@@ -95,7 +95,7 @@ class Linear:
         if pending is not None:
             if pending.pre is not None:
                 x, kw = pending.pre[0], dict(ss=pending.pre[1], eps=pending.norm.eps)
-            elif T <= ops.CONV_MAX_ROWS and pending.rows is None and self.in_features <= ops.NORMED_MAX_K:
+            elif T <= ops.NORMED_MAX_ROWS and pending.rows is None and self.in_features <= ops.NORMED_MAX_K:
                 x, kw = pending.x, dict(norm_w=pending.norm.weight_f32, eps=pending.norm.eps)
             else:
                 x = pending.tensor()
