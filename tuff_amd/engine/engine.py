@@ -111,7 +111,9 @@ class Engine:
     # ------------------------------------------------------------------------ step
     def step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Runs one batch.  Returns float32 logits [wanted, vocab] on the device, in the order
-        of the entries and of their `want` lists, or None if nothing is wanted.
+        of the entries and of their `want` lists, or None if nothing is wanted.  The tensor may be the
+        step function's own buffer (a recorded step writes its logits to the same place at every replay):
+        it holds this step's logits until the next step; a caller that keeps them copies them.
         Raises OutOfPages (and leaves every request as it was) if the pool is too small.
         device_tokens: for a caller that starts a step before it has seen the last one's tokens.
         Either an int32 tensor on the device with one id per token of the step, or a triple
