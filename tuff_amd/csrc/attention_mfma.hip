@@ -90,7 +90,7 @@ constexpr int UNIT = 64;                   // keys a unit: two steps of 32
 constexpr int UNITS = PART / UNIT;
 
 // NW: waves a workgroup (1: the wave walks the partition's four units; 4: a unit a wave, merged through LDS).
-template <int HDP, int NB, int NW, bool FUSED>
+template <int HDP, int NB, int NW, bool FUSED, bool STREAM_V>
 __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
     float* __restrict__ ws_o, float* __restrict__ ws_ml,
@@ -213,8 +213,8 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
     };
     // A page's V^T rows are 2 * page_size bytes: with pages of 16 positions a step of 32 keys reads whole rows and
     // never comes back to them; with larger pages it reads a part of each row's cache lines and the steps after it
-    // read the rest, so those loads are ordinary ones (a line asked for as streaming does not wait for them).
-    const bool stream_v = page_size <= 16;
+    // read the rest, so those loads are ordinary ones (a line asked for as streaming does not wait for them):
+    // STREAM_V is page_size <= 16.
     auto v_frag = [&](const Tile& t, int db) {
         const int dim = db * 16 + n16;
         bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
         const int off0 = (g / 2) ? t.off0[1] : t.off0[0];
         if (!live || dim >= hd) return z;
         const bf16x8* at = (const bf16x8*)(v_cache + base + (long long)dim * page_size + off0 + (g % 2) * 8);
-        return stream_v ? __builtin_nontemporal_load(at) : *at;
+        if constexpr (STREAM_V) return __builtin_nontemporal_load(at); else return *at;
     };
     auto load_tile = [&](int key0, Tile& t) {
 #pragma unroll
@@ -653,22 +653,29 @@ int few_waves = 2048;
 // round it is not.
 int kv_fast_waves = 6144;
 
-template <int HDP, int NB, bool FUSED>
+template <int HDP, int NB, bool FUSED, bool STREAM_V = true>
 void launch_partition(dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* kc, bf16_t* vc, float* ws_o,
                       float* ws_ml, const int* bt, int max_blocks, const int2* blk, const int4* req_info,
                       int H, int Hkv, int hd, int ps, int window, float scale, int n_parts, const FusedQKV& fq) {
+    if constexpr (STREAM_V) {
+        if (ps > 16) {
+            launch_partition<HDP, NB, FUSED, false>(grid, stream, q, kc, vc, ws_o, ws_ml, bt, max_blocks, blk, req_info, H, Hkv, hd,
+                                                    ps, window, scale, n_parts, fq);
+            return;
+        }
+    }
     const long long waves = (long long)grid.x * grid.y * grid.z;
     const int kv_fast = waves >= kv_fast_waves ? 1 : 0;
     if (kv_fast) grid = dim3(grid.x * grid.z, grid.y, 1);
     if constexpr (HDP * NB <= 128) {
         // the fused form prepares its queries in every wave: four waves pay for that four times
         if (waves < (FUSED ? few_waves / 2 : few_waves)) {
-            hipLaunchKernelGGL((attn_partition_kernel<HDP, NB, UNITS, FUSED>), grid, dim3(UNITS * WAVE), 0, stream, q, kc, vc, ws_o,
+            hipLaunchKernelGGL((attn_partition_kernel<HDP, NB, UNITS, FUSED, STREAM_V>), grid, dim3(UNITS * WAVE), 0, stream, q, kc, vc, ws_o,
                                ws_ml, bt, max_blocks, blk, req_info, H, Hkv, hd, ps, window, scale, n_parts, fq, kv_fast);
             return;
         }
     }
-    hipLaunchKernelGGL((attn_partition_kernel<HDP, NB, 1, FUSED>), grid, dim3(WAVE), 0, stream, q, kc, vc, ws_o, ws_ml, bt,
+    hipLaunchKernelGGL((attn_partition_kernel<HDP, NB, 1, FUSED, STREAM_V>), grid, dim3(WAVE), 0, stream, q, kc, vc, ws_o, ws_ml, bt,
                        max_blocks, blk, req_info, H, Hkv, hd, ps, window, scale, n_parts, fq, kv_fast);
 }
 }  // namespace
