@@ -42,6 +42,9 @@ def test_groups_by_window_and_shared_page_numbering():
     assert lay.group_of_entry == {0: 0, 2: 0, 3: 1, 4: 1}
     assert lay.bytes_per_token(2) == 2 * 2 * (2 * 16 + 4 * 8 + 2 * 16 + 64)
     assert lay.state_bytes_per_request() == 2 * 8 * 4
+    # values of a width of their own: a token costs keys + values, not twice the keys
+    assert PagedKV(2, 16).v_dim == 16 and PagedKV(2, 16, None, 40).v_dim == 40
+    assert CacheLayout.from_specs({0: PagedKV(2, 16, value_dim=40)}).bytes_per_token(2) == 2 * 2 * (16 + 40)
     with pytest.raises(CacheError, match="unknown cache declaration"):
         CacheLayout.from_specs({0: "ring buffer"})
 

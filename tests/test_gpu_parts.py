@@ -413,6 +413,106 @@ def test_toy_mixer_with_several_cache_entries(gpu):
         registry.unregister_architecture("ToySeveralForCausalLM")
 
 
+def test_toy_mixer_with_keys_narrower_than_values(gpu):
+    """A mixer whose keys are 8 wide and whose values are the model's width, in one PagedKV entry with
+    a window: the pool is laid out by the declaration ([pages, heads, page, 8] and [pages, heads, 24,
+    page]), pages behind the window go back, and the framework's own attention refuses such a cache by
+    its shape.  Whole, token by token and mixed with few pages, against a plain loop."""
+    from tuff_amd.config.base import ModelConfig
+    from tuff_amd.csrc import ops
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.models import registry
+    from tuff_amd.models.decoder import DecoderModel
+    from tuff_amd.parts.base import MIXERS, Mixer, PagedKV, WeightDecl
+    from tuff_amd.parts.block import PreNormBlock
+    from tuff_amd.parts.ffn import SwiGLU
+    from tuff_amd.parts.norm import RMSNorm
+    from tuff_amd.weights.random_init import random_weights
+    d, dk, V, eps, window = 24, 8, 83, 1e-5, 20
+    shapes = {}
+
+    class NarrowKeys(Mixer):
+        def __init__(self, d, dk, window, name):
+            self.d, self.dk, self.window, self.name = d, dk, window, name
+
+        def weight_decls(self):
+            return [WeightDecl(self.name + ".q", (self.dk, self.d)), WeightDecl(self.name + ".k", (self.dk, self.d))]
+
+        def cache_spec(self):
+            return PagedKV(1, self.dk, self.window, value_dim=self.d)
+
+        def bind(self, weights, rt):
+            self.rt, self.wq, self.wk = rt, weights[self.name + ".q"].float(), weights[self.name + ".k"].float()
+
+        def forward(self, h, ctx, cache, residual, write_cache=True):
+            shapes["k"], shapes["v"] = tuple(cache.k.shape[1:]), tuple(cache.v.shape[1:])
+            ps, g = cache.page_size, ctx.groups[cache.group]
+            hf = h.float()
+            q, k = hf @ self.wq.T, hf @ self.wk.T
+            assert write_cache
+            slot = g.slot_mapping.long()
+            cache.k[slot // ps, 0, slot % ps] = k.to(cache.k.dtype)
+            cache.v[slot // ps, 0, :, slot % ps] = hf.to(cache.v.dtype)
+            pos, req = ctx.positions.tolist(), ctx.req_of_token.tolist()
+            for t in range(ctx.T):
+                lo = max(0, pos[t] - self.window + 1)
+                at = torch.arange(lo, pos[t] + 1, device=h.device)
+                page = g.block_table[req[t]].long()[at // ps]
+                assert int(page.min()) >= 0                        # no page of the window was given back
+                keys, vals = cache.k[page, 0, at % ps].float(), cache.v[page, 0, :, at % ps].float()
+                p = torch.softmax(keys @ q[t] / self.dk ** 0.5, 0)
+                residual[t] += p @ vals
+
+    @dataclasses.dataclass
+    class Cfg(ModelConfig):
+        architecture: ClassVar[str] = "ToyNarrowKeysForCausalLM"
+        vocab_size: int
+
+    def build(cfg):
+        blocks = [PreNormBlock(RMSNorm(d, eps, "n1"), MIXERS.get("narrow_keys")(d, dk, window, "mix"), RMSNorm(d, eps, "n2"),
+                               SwiGLU(d, 40, names={"gate": "g", "up": "u", "down": "d"}))]
+        return DecoderModel(vocab_size=cfg.vocab_size, hidden_size=d, embedding=WeightDecl("emb", (cfg.vocab_size, d)),
+                            blocks=blocks, final_norm=RMSNorm(d, eps, "fn"))
+
+    MIXERS.register("narrow_keys", NarrowKeys)
+    registry.register_architecture("ToyNarrowKeysForCausalLM", Cfg, build)
+    try:
+        model = registry.build_model(registry.config_from_dict({"architectures": ["ToyNarrowKeysForCausalLM"], "vocab_size": V}))
+        assert model.cache_specs == {0: PagedKV(1, dk, window, d)}
+        w32 = random_weights(model.weight_decls(), 6, torch.float32, "cpu")
+        eng = Engine(model, {k: v.to(gpu) for k, v in w32.items()}, dtype="float32", max_tokens=192, poison_cache=True)
+        assert eng.layout.bytes_per_token(4) == 4 * (dk + d)
+        reqs = {"a": util.rand_tokens(70, V, 1), "b": util.rand_tokens(45, V, 2), "c": util.rand_tokens(52, V, 3)}
+        whole = util.run_plan(eng, util.plan_whole(reqs))
+        ps = eng.manager.page_size
+        assert shapes == {"k": (1, ps, dk), "v": (1, d, ps)}
+        single = util.run_plan(eng, util.plan_tail(reqs, 100))
+        mixed = util.run_plan(eng, util.plan_mixed(reqs, seed=7, decode_tail=6))
+        view = eng.storage.views[0]
+        with pytest.raises(ops.KernelError, match="v_cache"):
+            ops.attention_general(torch.zeros(1, dk, device=gpu), view.k, view.v, torch.zeros(1, dk, device=gpu),
+                                  block_table=torch.zeros(1, 1, dtype=torch.int32, device=gpu),
+                                  req_of_token=torch.zeros(1, dtype=torch.int32, device=gpu),
+                                  positions=torch.zeros(1, dtype=torch.int32, device=gpu), H=1, Hkv=1, hd=dk, page_size=ps)
+        w = {k: v.double() for k, v in w32.items()}
+        for rid, toks in reqs.items():
+            x = w["emb"][toks]
+            h = plain.rms_norm(x, w["n1"], eps)
+            q, k = h @ w["mix.q"].T, h @ w["mix.k"].T
+            n = h.shape[0]
+            i = torch.arange(n)
+            seen = (i[None, :] <= i[:, None]) & (i[None, :] > i[:, None] - window)
+            score = (q @ k.T / dk ** 0.5).masked_fill(~seen, float("-inf"))
+            x = x + torch.softmax(score, -1) @ h
+            x = x + plain.swiglu(plain.rms_norm(x, w["n2"], eps), w["g"], w["u"], w["d"])
+            want = plain.rms_norm(x, w["fn"], eps) @ w["emb"].T
+            for got in (whole, single, mixed):
+                util.assert_close_f32(got[rid], want, rid)
+    finally:
+        MIXERS.unregister("narrow_keys")
+        registry.unregister_architecture("ToyNarrowKeysForCausalLM")
+
+
 # ------------------------------------------------------- run order and cache groups as data
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_layer_run_twice_a_shared_cache_and_a_window_group(gpu, dtype):

@@ -97,7 +97,7 @@ class CacheLayout:
         return CacheLayout(paged, states, windows, group_of)
 
     def bytes_per_token(self, elem_size: int) -> int:
-        return sum(2 * s.num_kv_heads * s.head_dim * elem_size for s in self.paged.values())
+        return sum(s.num_kv_heads * (s.head_dim + s.v_dim) * elem_size for s in self.paged.values())
 
     def state_bytes_per_request(self) -> int:
         return sum(s.nbytes() for s in self.states.values())

@@ -28,10 +28,17 @@ class WeightDecl:
 @dataclasses.dataclass(frozen=True)
 class PagedKV:
     """Keys and values that grow by one entry a token, kept in pages.  `window`: only the
-    last `window` positions are ever read (None: all)."""
+    last `window` positions are ever read (None: all).  `value_dim`: the width of a value where
+    it is not the keys' (None: head_dim); the framework's own attention kernels take equal
+    widths only and refuse others by the cache's shape."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_dim: Optional[int] = None
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclasses.dataclass(frozen=True)
