@@ -264,9 +264,9 @@ class Engine:
                 torch.cuda.synchronize()                    # its last replay may still be under way
                 self._graphs.pop(next(iter(self._graphs)))
             g = _RecordedStep(p, self.device, width * self.page_size)
-            self._graphs[key] = g
             g.refresh(p, device_tokens)
             logits = self.model.forward(g.ctx, self.storage.views)
+            self._graphs[key] = g                           # only a shape whose eager step went through
             try:
                 g.record(lambda: self.model.forward(g.ctx, self.storage.views))
             except Exception as e:                         # noqa: BLE001 - recording is an optimisation
