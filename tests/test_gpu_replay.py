@@ -246,7 +246,6 @@ def test_steps_with_portions_recorded_in_sections_equal_eager_steps(gpu, name, d
     what an engine that records nothing gives; so do the tokens decoded afterwards out of the cache
     and the conv states those steps left."""
     from tuff_amd.engine.engine import Engine
-    monkeypatch.setattr(Engine, "SECTIONS_MIN_TOKENS", 40)
     V = util.CONFIGS[name][0]["vocab_size"]
     reqs = {k: util.rand_tokens(n, V, 10 + i) for i, (k, n) in enumerate(
         [("a", 300), ("b", 220), ("c", 130), ("d", 90), ("e", 75)])}
@@ -295,7 +294,6 @@ def test_recordings_are_dropped_and_made_again(gpu, monkeypatch):
     """Room for one recording of each kind: sizes that take turns push each other out and are recorded
     again, and every step still equals the eager one."""
     from tuff_amd.engine.engine import Engine
-    monkeypatch.setattr(Engine, "SECTIONS_MIN_TOKENS", 40)
     monkeypatch.setattr(Engine, "MAX_SECTIONED", 1)
     monkeypatch.setattr(Engine, "MAX_GRAPHS", 1)
     V = util.TINY_A["vocab_size"]
@@ -325,6 +323,35 @@ def test_recordings_are_dropped_and_made_again(gpu, monkeypatch):
     # a size is recorded when it has come three times: in the first round its third and fourth step replay, later all four
     assert eng.section_replays == 2 * 2 + 2 * 2 * 4 and len(eng._sectioned) == 1 and len(eng._graphs) == 1
     assert eng.graph_replays == 3 * 2 * 1
+    for rid in reqs:
+        mask = ~torch.isnan(want[rid][:, 0])
+        assert torch.equal(got[rid][mask], want[rid][mask]), rid
+
+
+def test_sizes_that_push_each_other_out_are_recorded_less_and_less_often(gpu, monkeypatch):
+    """Three sizes take turns, one step each, with room for one recording: a recording is pushed out before
+    it is used again, so the engine asks for more and more returns of a size before it records it; the
+    steps still equal the eager ones."""
+    from tuff_amd.engine.engine import Engine
+    monkeypatch.setattr(Engine, "MAX_SECTIONED", 1)
+    V = util.TINY_A["vocab_size"]
+    reqs = {k: util.rand_tokens(2200, V, 40 + i) for i, k in enumerate("ab")}
+    steps, fed = [], {k: 0 for k in reqs}
+    def portion(rid, n):
+        t = reqs[rid][fed[rid]:fed[rid] + n]
+        fed[rid] += n
+        assert len(t) == n
+        return {"id": rid, "tokens": t, "want": [n - 1]}
+    for rnd in range(14):
+        for n in (40, 50, 60):
+            steps.append({"step": len(steps), "entries": [portion("a", n - 10), portion("b", 10)], "end": []})
+    steps[-1]["end"] = ["a", "b"]
+    eager = make_engine("A", "bfloat16", max_tokens=4480, use_graphs=False)
+    want = util.run_plan(eager, steps)
+    eng = make_engine("A", "bfloat16", max_tokens=4480)
+    got = util.run_plan(eng, steps)
+    # recorded at every step from the third round on it would be 36 times
+    assert 3 <= eng.section_recordings <= 8 and eng.section_replays > eng.section_recordings
     for rid in reqs:
         mask = ~torch.isnan(want[rid][:, 0])
         assert torch.equal(got[rid][mask], want[rid][mask]), rid

@@ -71,7 +71,9 @@ class Engine:
         self.record_portions = self.use_graphs and model.records_portions()
         self._sectioned: dict = {}
         self._sectioned_seen: dict = {}
+        self._record_at = self.SECTIONS_RECORD_AT
         self.section_replays = 0
+        self.section_recordings = 0
 
     # ---------------------------------------------------------------- construction
     @classmethod
@@ -203,8 +205,8 @@ class Engine:
             ops.scatter_i32(tokens, device_tokens[0], device_tokens[1])
 
     # ------------------------------------------------------- steps recorded in sections
-    SECTIONS_MIN_TOKENS = 128        # below, the products choose their kernels by more than the number of rows
-    SECTIONS_RECORD_AT = 3           # a number of tokens is recorded when it comes for this time
+    SECTIONS_MIN_TOKENS = 2          # every step with a portion may be recorded (a step of 64 tokens: 1.57 ms of launches, 1.22 ms replayed)
+    SECTIONS_RECORD_AT = 3           # a number of tokens is recorded when it comes for this time (more, once sizes push each other out)
     MAX_SECTIONED = 4
 
     def _portion_step(self, ctx, device_tokens=None) -> Optional[torch.Tensor]:
@@ -219,12 +221,18 @@ class Engine:
             if len(self._sectioned_seen) > 256 and key not in self._sectioned_seen:
                 self._sectioned_seen.clear()                # sizes that came once or twice and never again
             seen = self._sectioned_seen[key] = self._sectioned_seen.get(key, 0) + 1
-            if seen < self.SECTIONS_RECORD_AT:
+            if seen < self._record_at:
                 self._place_device_tokens(ctx.tokens, device_tokens)
                 return self.model.forward(ctx, self.storage.views)
             if len(self._sectioned) >= self.MAX_SECTIONED:
                 torch.cuda.synchronize()                    # its last replay may still be under way
-                self._sectioned.pop(next(iter(self._sectioned)))
+                old_key = next(iter(self._sectioned))
+                if self._sectioned.pop(old_key).replays <= 1:
+                    # More sizes take turns than recordings are kept: this one was pushed out before it was
+                    # used again.  Recording costs about two eager steps, so sizes now have to come more often.
+                    self._record_at = min(2 * self._record_at, 1 << 16)
+                    self._sectioned_seen[old_key] = 0
+            self.section_recordings += 1
             rec = _SectionedStep(ctx.T, self.manager.num_slots, self.device)
             try:
                 rec.record(ctx, lambda c: self.model.forward(c, self.storage.views))
@@ -299,6 +307,7 @@ class _SectionedStep:
         self.copied = torch.cuda.Event()
         self.pool = torch.cuda.graph_pool_handle()
         self.program: list = []                # graphs and functions of a context, in order
+        self.replays = 0
         self._graph = None
         self._capture = None
 
@@ -360,6 +369,7 @@ class _SectionedStep:
 
     def replay(self, ctx):
         out = None
+        self.replays += 1
         for piece in self.program:
             if isinstance(piece, torch.cuda.CUDAGraph):
                 piece.replay()
