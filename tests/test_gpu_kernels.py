@@ -47,7 +47,9 @@ def test_gemm_f32(gpu, M, N, K):
                                    # the same with K a multiple of 64: operands go straight into LDS
                                    (1100, 8200, 192), (1030, 8190, 128), (1100, 4001, 256), (257, 129, 512), (100, 40, 64),
                                    # few blocks and a short K: blocks of 64 x 64, ragged in M and N
-                                   (200, 1000, 1536), (65, 70, 3072), (500, 1536, 1536), (130, 2049, 320)])
+                                   (200, 1000, 1536), (65, 70, 3072), (500, 1536, 1536), (130, 2049, 320),
+                                   # 17 to 64 rows, a wide output and a short K: blocks of 64 x 64 of the tiled kernel
+                                   (17, 9216, 128), (40, 16390, 2048), (64, 24576, 192), (33, 10240, 3072)])
 def test_gemm_bf16(gpu, M, N, K):
     from tuff_amd.csrc import ops
     x, w = _r(M, K, seed=4, dtype=torch.bfloat16), _r(N, K, seed=5, dtype=torch.bfloat16)
@@ -77,7 +79,8 @@ def test_gemm_bf16(gpu, M, N, K):
 @pytest.mark.parametrize("M,N,K", [(1, 32, 64), (8, 512, 240), (16, 6144, 2048), (5, 200, 96), (64, 384, 256),
                                    (40, 2050, 2048), (24, 2050, 2048), (32, 16384, 2048), (300, 130, 136), (2048, 512, 128), (1100, 8200, 72),
                                    (200, 384, 1024), (72, 4100, 2048),
-                                   (1030, 8202, 136), (1100, 4002, 200), (1030, 8202, 128), (1100, 4002, 192), (120, 13826, 1536)])
+                                   (1030, 8202, 136), (1100, 4002, 200), (1030, 8202, 128), (1100, 4002, 192), (120, 13826, 1536),
+                                   (17, 16384, 2048), (64, 13824, 1536), (25, 12290, 640)])
 def test_gemm_bf16_swiglu_epilogue(gpu, M, N, K):
     """Rows of w are gate and up rows interleaved; the output is silu(gate) * up."""
     from tuff_amd.csrc import ops
@@ -128,7 +131,9 @@ def test_gemm_with_the_norm_inside(gpu, M, N, K, use_rows):
 
 @pytest.mark.parametrize("M,d,K1,N2", [(1, 64, 192, 512), (8, 2048, 8192, 6144), (16, 240, 328, 777 * 2), (5, 96, 96, 40),
                                        (17, 96, 96, 40), (32, 2048, 8192, 6144), (24, 240, 328, 777 * 2), (40, 2048, 8192, 6144), (64, 240, 328, 777 * 2), (33, 64, 192, 512),
-                                       (64, 2048, 2048, 65536)])
+                                       (64, 2048, 2048, 65536),
+                                       # the product that follows is wide with a short K: the tiled kernel reads these row sums
+                                       (17, 192, 96, 9216), (40, 2048, 2048, 16384), (64, 1536, 512, 13824), (25, 128, 64, 10242)])
 def test_gemm_that_prepares_the_next_norm(gpu, M, d, K1, N2):
     """residual += a @ w1.T leaves bf16(residual * norm weight) and per-tile row sums of squares;
     the next product scales its rows by them: together rmsnorm(residual) @ w2.T."""

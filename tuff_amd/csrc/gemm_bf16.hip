@@ -132,6 +132,7 @@ __device__ __forceinline__ void store_quad(void* Y, long long row, long long col
 // waves that share rows add theirs in the order of their columns).
 struct TiledExtra {
     const float* ss_in = nullptr; int n_ss = 0; float eps = 0.f;
+    int ss_rows = 0;                      // rows of a group of sums in ss_in (0: M; 64 where a product of at most 64 rows left them)
     const float* emit_nw = nullptr; bf16_t* emit_xw = nullptr; float* emit_ss = nullptr;
 };
 enum : int { TILED_PLAIN = 0, TILED_SCALED = 1, TILED_EMIT = 2 };
@@ -401,6 +402,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_dma_kernel(
     if constexpr (AROUND == TILED_SCALED) {
         // while the first operands are on their way: the scale of each of the block's rows, its groups' sums in order
         // (a product cut along K leaves that to the kernel that adds the slices)
+        const int ss_rows = ex.ss_rows ? ex.ss_rows : M;
         for (int r = tid; r < BM && gridDim.z == 1; r += 64 * NW) {
             const long long row = m0 + r;
             float t = 0.f;
@@ -410,7 +412,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_dma_kernel(
                 for (int j0 = 0; j0 < ex.n_ss; j0 += 16) {
                     float v[16];
 #pragma unroll
-                    for (int u = 0; u < 16; ++u) v[u] = j0 + u < ex.n_ss ? ex.ss_in[(long long)(j0 + u) * M + row] : 0.f;
+                    for (int u = 0; u < 16; ++u) v[u] = j0 + u < ex.n_ss ? ex.ss_in[(long long)(j0 + u) * ss_rows + row] : 0.f;
 #pragma unroll
                     for (int u = 0; u < 16; ++u) t += v[u];
                 }
@@ -1112,18 +1114,29 @@ struct SkinnyPlan { int tiles, waves, slices, chunks_per_slice, cols; long long 
 
 constexpr int SKINNY_ROWS = 32;     // the most rows of the kernel whose waves split K inside the workgroup (two row tiles)
 
+// 17 to 64 rows and a wide output with a short K (gate and up of a feed-forward): the tiled product with one
+// block of 64 x 64 for every 64 columns gives every CU a workgroup without slices of K, so no second kernel
+// adds partial tiles, and its time is that of streaming W whatever the rows.  Measured against the two ways
+// for few rows, SwiGLU epilogue, 17 to 64 rows: 16,384 x 2,048 18 to 22 us -> 15.5 to 16.5, 13,824 x 1,536 14 to
+// 17 -> 11.5, 9,216 x 1,536 12 to 14 -> 11, 24,576 x 2,048 26 to 28.5 -> 24 to 27; no gain at 6,144 and 8,192
+// columns nor at 32,768.
+int wide64_min_n = 9216, wide64_max_n = 24576, wide64_min_m = 17;      // measurements may move them
+bool wide64_shape(int N, int K) { return N >= wide64_min_n && N <= wide64_max_n && K % TBK == 0 && K / TBK <= 48; }
+bool rows64_tiled(int M, int N, int K) { return M >= wide64_min_m && M <= 64 && wide64_shape(N, K); }
+
 // Whether a product of M rows goes through that kernel (else, up to 64 rows: K cut over workgroups and a
 // second kernel that adds the slices).  Up to 16 rows always.  17 to 32 rows: every workgroup reads all M
 // rows of X again, M / (its columns) times the bytes of its share of W, and has half the waves; measured
 // on the shapes of a 1.2B model (against the two kernels of the other way, at 32 rows): 2,048 columns
 // 14.8 us against 11.9, 3,072 columns 8.8 against 10.7, a conv's input projection with the convolution
 // 12.5 against 15.2, 16,384 columns 21.7 against 21.3, 65,536 columns 67.7 against 52.2; at 17 rows
-// it wins everywhere.  So: narrow outputs up to 20 rows, medium ones up to 32, wide ones up to 24.
+// it wins everywhere.  So: narrow outputs up to 20 rows, medium ones up to 32, wide ones up to 24 (where the
+// tiled product does not take them, above).
 bool few_rows_kernel(int M, int N, int K, bool conv = false) {
-    (void)K;
     if (M <= 16) return true;
     if (M > SKINNY_ROWS) return false;
     if (conv) return true;
+    if (rows64_tiled(M, N, K)) return false;
     return N <= 2048 ? M <= 20 : N <= 8192 ? true : M <= 24;
 }
 
@@ -1333,7 +1346,7 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
                 const TiledExtra& ex = TiledExtra()) {
     if constexpr (AROUND == TILED_PLAIN) {
         if (few_rows_kernel(M, N, K)) return launch_skinny16<MODE, NORM_NONE, false>(X, W, Y, M, N, K, Skinny16Extra(), stream);
-        if (M <= 64) return launch_skinny64<MODE, NORM_NONE, false>(X, W, Y, M, N, K, ws, FinishExtra(), stream);
+        if (M <= 64 && !rows64_tiled(M, N, K)) return launch_skinny64<MODE, NORM_NONE, false>(X, W, Y, M, N, K, ws, FinishExtra(), stream);
     }
     {
         // Large blocks where they give most CUs one.  Of the small ones a CU holds two if there are
@@ -1341,7 +1354,8 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
         // the operands of four steps under way.  Where even the small blocks are fewer than half the
         // CUs (few rows, narrow output), blocks of 64 x 64 take over if K is short, else K is cut into
         // slices, a block a slice.
-        const TiledPlan t = plan_tiled(M, N, K);
+        TiledPlan t = plan_tiled(M, N, K);
+        if (rows64_tiled(M, N, K)) { t.shape = 3; t.slices = 1; t.steps_per_slice = ceil_div(K, TBK); t.ws_floats = 0; }
         if (t.slices > 1 && !ws) return -4;
 #define TILED(TM, TN, WM, WN, AHEAD) do { \
             auto kern = gemm_bf16_tiled_kernel<TM, TN, WM, WN, AHEAD, MODE>; \
@@ -1396,6 +1410,16 @@ int launch_mode(const bf16_t* X, const bf16_t* W, void* Y, int M, int N, int K, 
 }
 }  // namespace
 
+// For measurements: for how many columns and from how many rows on a product of at most 64 rows with a short K
+// takes blocks of 64 x 64 instead of slices of K.  Returns the least number of columns before.
+TUFF_EXPORT int tuff_gemm_bf16_wide64(int min_n, int max_n, int min_m) {
+    const int old = wide64_min_n;
+    if (min_n > 0) wide64_min_n = min_n;
+    if (max_n > 0) wide64_max_n = max_n;
+    if (min_m > 0) wide64_min_m = min_m;
+    return old;
+}
+
 // For measurements: forces the block shape of every product of more than 64 rows whose K is a multiple
 // of 64 (0: 256 x 256, 1: 128 x 128 two a CU, 2: 128 x 128 one a CU, 3: 64 x 64, 4: 256 x 192; -1: by size).
 // Returns the value before.
@@ -1432,6 +1456,7 @@ TUFF_EXPORT int tuff_gemm_bf16_scaled_supported(int M, int N, int K) {
 TUFF_EXPORT int tuff_gemm_bf16_workspace(int M, int N, int K, int emit, long long* ws_floats) {
     *ws_floats = 0;
     if (N <= 0 || few_rows_kernel(M, N, K)) return 0;
+    // (a wide product of few rows that the tiled kernel takes needs none, but only some of its epilogues go that way)
     *ws_floats = M <= 64 ? plan_skinny(M, N, K, 16, emit != 0).ws_floats : plan_tiled(M, N, K).ws_floats;
     return 0;
 }
@@ -1498,11 +1523,11 @@ TUFF_EXPORT int tuff_gemm_bf16_scaled(const void* XW, const float* ss, int n_ss,
                                       int M, int N, int K, int mode, float* ws, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (K % 8 != 0 || n_ss < 1) return -2;
-    if (M > 64) {
-        // ss [n_ss][M]; bfloat16 and SwiGLU outputs (what reads a norm in a layer)
+    if (M > 64 || (rows64_tiled(M, N, K) && (mode == OUT_BF16 || mode == OUT_SWIGLU))) {
+        // ss [n_ss][M] ([n_ss][64] from a product of at most 64 rows); bfloat16 and SwiGLU outputs (what reads a norm in a layer)
         if (!tiled_scaled_ok(M, N, K)) return -2;
         TiledExtra t;
-        t.ss_in = ss; t.n_ss = n_ss; t.eps = eps;
+        t.ss_in = ss; t.n_ss = n_ss; t.eps = eps; t.ss_rows = M > 64 ? 0 : 64;
         const bf16_t* x = (const bf16_t*)XW;
         const bf16_t* w = (const bf16_t*)W;
         if (mode == OUT_BF16) return launch_mode<OUT_BF16, TILED_SCALED>(x, w, Y, M, N, K, ws, stream, t);
