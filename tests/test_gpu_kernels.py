@@ -1260,6 +1260,12 @@ def test_sample_top_k_ties_and_uniform_logits(gpu):
     assert out.cpu().tolist() == [0, 249, 499]           # equal values are ordered by index
     ops.sample(l.to(gpu), out, temps=ones, top_ks=torch.full((3,), 10, dtype=torch.int32, device=gpu), uniforms=u)
     assert out.cpu().tolist() == [0, 4, 9]
+    # zeros of either sign are equal values too
+    l[:, 1::3] = -0.0
+    ops.sample(l.to(gpu), out, temps=ones, uniforms=u)
+    assert out.cpu().tolist() == [0, 249, 499]
+    ops.sample(l.to(gpu), out, temps=ones, top_ks=torch.full((3,), 10, dtype=torch.int32, device=gpu), uniforms=u)
+    assert out.cpu().tolist() == [0, 4, 9]
 
 
 def test_repeat_penalty(gpu):

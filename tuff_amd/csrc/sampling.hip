@@ -23,6 +23,7 @@ typedef unsigned long long u64;
 
 __device__ __forceinline__ uint32_t order_key(float f) {
     const uint32_t u = __float_as_uint(f);
+    if (u == 0x80000000u) return 0x80000000u;          // -0 and +0 compare equal: one key, so that the index decides
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
