@@ -398,26 +398,45 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_dma_kernel(
         constexpr int st = decltype(s)::value;
         if (kt_begin + st < kt_end) issue(st, kt_begin + st);
     });
+    // TILED_SCALED: the sum of squares of each of the block's rows, in SS_PARTS parts: thread (part, row) adds the groups
+    // part, part + SS_PARTS, ... in that order, sixteen loads at a time (one after the other would be as many trips to
+    // memory: a product of few rows leaves 256 groups for 2,048 columns); behind the first barrier of the loop the parts
+    // of a row are added in their order and the row's scale is left for the epilogue.  (Up to sixteen groups, as the
+    // tiled products of a prompt leave them: one thread a row, the scale at once.)
+    constexpr int SS_PARTS = (64 * NW) / BM >= 4 ? 4 : (64 * NW) / BM >= 2 ? 2 : 1;
+    __shared__ float row_ss[AROUND == TILED_SCALED ? SS_PARTS : 1][AROUND == TILED_SCALED ? BM : 1];
     __shared__ float row_scale[AROUND == TILED_SCALED ? BM : 1];
     if constexpr (AROUND == TILED_SCALED) {
-        // while the first operands are on their way: the scale of each of the block's rows, its groups' sums in order
-        // (a product cut along K leaves that to the kernel that adds the slices)
+        // while the first operands are on their way (a product cut along K leaves the scales to the kernel that adds the slices)
         const int ss_rows = ex.ss_rows ? ex.ss_rows : M;
-        for (int r = tid; r < BM && gridDim.z == 1; r += 64 * NW) {
+        if (ex.n_ss <= 16) {
+            // one trip to memory a row: the scale at once
+            if (tid < BM && gridDim.z == 1) {
+                const long long row = m0 + tid;
+                float v[16], t = 0.f;
+#pragma unroll
+                for (int u = 0; u < 16; ++u) v[u] = (row < M && u < ex.n_ss) ? ex.ss_in[(long long)u * ss_rows + row] : 0.f;
+#pragma unroll
+                for (int u = 0; u < 16; ++u) t += v[u];
+                row_scale[tid] = 1.0f / sqrtf(t / (float)K + ex.eps);
+            }
+        } else if (tid < SS_PARTS * BM && gridDim.z == 1) {
+            const int r = tid % BM, part = tid / BM;
             const long long row = m0 + r;
             float t = 0.f;
             if (row < M) {
-                // sixteen groups' sums are asked for together (one after the other would be as many trips to
-                // memory), then added in their order
-                for (int j0 = 0; j0 < ex.n_ss; j0 += 16) {
+                for (int j0 = part; j0 < ex.n_ss; j0 += 16 * SS_PARTS) {
                     float v[16];
 #pragma unroll
-                    for (int u = 0; u < 16; ++u) v[u] = j0 + u < ex.n_ss ? ex.ss_in[(long long)(j0 + u) * ss_rows + row] : 0.f;
+                    for (int u = 0; u < 16; ++u) {
+                        const int j = j0 + u * SS_PARTS;
+                        v[u] = j < ex.n_ss ? ex.ss_in[(long long)j * ss_rows + row] : 0.f;
+                    }
 #pragma unroll
                     for (int u = 0; u < 16; ++u) t += v[u];
                 }
             }
-            row_scale[r] = 1.0f / sqrtf(t / (float)K + ex.eps);
+            row_ss[part][r] = t;
         }
         // read in the epilogue, behind the barriers of the loop (every wave waits for its LDS writes before each)
     }
@@ -434,6 +453,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_dma_kernel(
                 });
                 __builtin_amdgcn_s_barrier();
                 if (kt + STAGES - 1 < kt_end) issue((buf + STAGES - 1) % STAGES, kt + STAGES - 1);
+                if constexpr (AROUND == TILED_SCALED) {
+                    if (kt == kt_begin && ex.n_ss > 16 && tid < BM && gridDim.z == 1) {
+                        float t = row_ss[0][tid];
+#pragma unroll
+                        for (int q = 1; q < SS_PARTS; ++q) t += row_ss[q][tid];
+                        row_scale[tid] = 1.0f / sqrtf(t / (float)K + ex.eps);
+                    }
+                }
                 read_half(S0(), buf, S0());
                 mult(S1());                                            // the second half of the step before (zeros at first)
                 spread();
@@ -453,6 +480,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_dma_kernel(
             for (int j = 0; j < TN; ++j)
                 store_quad<OUT_F32>(mine, m0 + wm + i * 16 + r16, n0 + wn + j * 16 + g * 4, M, N, acc[i][j]);
         return;
+    }
+    if constexpr (AROUND == TILED_SCALED) {
+        if (kt_end - kt_begin < 2) __syncthreads();        // a single step: no barrier has followed the scales yet
     }
     if constexpr (AROUND == TILED_EMIT) {
         // whole blocks of columns only (the host sees to it): Y += acc, the next norm's operand, the row's sum of squares
