@@ -712,7 +712,10 @@ def test_attention_of_single_tokens_does_not_depend_on_the_order_of_its_workgrou
         torch.cuda.synchronize()
         return out.float().cpu(), c["kc"].float().cpu()
 
+    for fn in (lib.tuff_attention_stage_k_waves, lib.tuff_attention_few_waves):
+        fn.argtypes, fn.restype = [ctypes.c_int], ctypes.c_int
     before = lib.tuff_attention_kv_fast_waves(-1)
+    staged, few = lib.tuff_attention_stage_k_waves(-1), lib.tuff_attention_few_waves(-1)
     try:
         for fused in (False, True):
             lib.tuff_attention_kv_fast_waves(1 << 30)
@@ -722,8 +725,66 @@ def test_attention_of_single_tokens_does_not_depend_on_the_order_of_its_workgrou
             assert torch.isfinite(o_part).all()
             assert torch.equal(o_part, o_kv), f"fused={fused}"
             assert torch.equal(torch.nan_to_num(k_part, nan=1e9), torch.nan_to_num(k_kv, nan=1e9))
+            # ... and as the largest launches run: one wave a partition, the keys through LDS
+            lib.tuff_attention_few_waves(0)
+            lib.tuff_attention_stage_k_waves(0)
+            o_lds, k_lds = run(fused)
+            lib.tuff_attention_stage_k_waves(1 << 30)
+            o_one, _ = run(fused)
+            lib.tuff_attention_few_waves(few)
+            assert torch.equal(o_lds, o_one) and torch.equal(o_lds, o_part), f"fused={fused}: keys through LDS"
+            assert torch.equal(torch.nan_to_num(k_part, nan=1e9), torch.nan_to_num(k_lds, nan=1e9))
     finally:
         lib.tuff_attention_kv_fast_waves(before)
+        lib.tuff_attention_stage_k_waves(staged)
+        lib.tuff_attention_few_waves(few)
+
+
+@pytest.mark.parametrize("H,Hkv,hd,ps", [(32, 8, 64, 16), (6, 3, 64, 64), (4, 2, 40, 16), (3, 1, 48, 32), (8, 2, 56, 16)])
+def test_attention_of_single_tokens_with_keys_through_lds_or_not(gpu, H, Hkv, hd, ps):
+    """Large launches ask for the keys of heads of up to 64 channels as they lie in memory and put them into the
+    operands' order through LDS, small ones read them in that order at once: the same bits either way (forced both
+    ways here), and close to the plain attention."""
+    import ctypes
+    from tuff_amd.csrc import ops
+    lens = [700, 1, 257, 256, 33, 1025, 64, 17, 300]
+    R = len(lens)
+    lib = ops.load("attention_mfma")
+    lib.tuff_attention_stage_k_waves.argtypes = [ctypes.c_int]
+    lib.tuff_attention_stage_k_waves.restype = ctypes.c_int
+    lib.tuff_attention_few_waves.argtypes = [ctypes.c_int]
+    lib.tuff_attention_few_waves.restype = ctypes.c_int
+    case = _paged_case(gpu, torch.bfloat16, H, Hkv, hd, ps, lens, 0)
+    kc, vc, table, req, pos, q, Ks, Vs = case
+    # the last token of every request
+    last = [int(torch.nonzero((req == i) & (pos == lens[i] - 1))[0]) for i in range(R)]
+    q1 = q[last].contiguous().to(gpu)
+    info = torch.tensor([[i, 1, lens[i] - 1, lens[i]] for i in range(R)], dtype=torch.int32, device=gpu)
+    positions = torch.tensor([n - 1 for n in lens], dtype=torch.int32, device=gpu)
+    outs = []
+    before = lib.tuff_attention_stage_k_waves(-1)
+    few = lib.tuff_attention_few_waves(0)                 # one wave a partition, as large launches have it
+    try:
+        for waves in (1 << 30, 0):
+            lib.tuff_attention_stage_k_waves(waves)
+            out = torch.full((R, H * hd), float("nan"), dtype=torch.bfloat16, device=gpu)
+            ops.attention_mfma(q1, kc.to(gpu), vc.to(gpu), out, blocks=None, nb=1, hd=hd, block_table=table.to(gpu), req_info=info,
+                               positions=positions, H=H, Hkv=Hkv, page_size=ps, max_ctx_len=max(lens))
+            torch.cuda.synchronize()
+            outs.append(out.float().cpu())
+    finally:
+        lib.tuff_attention_stage_k_waves(before)
+        lib.tuff_attention_few_waves(few)
+    assert torch.isfinite(outs[0]).all() and torch.equal(outs[0], outs[1])
+    G = H // Hkv
+    for i in range(R):
+        K, V = Ks[i][:lens[i]], Vs[i][:lens[i]]                           # [n, Hkv, hd] of the request, float64
+        qi = q[last[i]].double().view(H, hd)
+        for h in range(H):
+            p = torch.softmax(K[:, h // G] @ qi[h] / hd ** 0.5, 0)
+            want = p @ V[:, h // G]
+            got = outs[1][i].view(H, hd)[h].double()
+            assert (got - want).abs().max() <= 2 ** -6 * max(float(want.abs().max()), 0.05), (i, h)
 
 
 @pytest.mark.parametrize("H,Hkv,hd,ps", [(4, 2, 16, 16), (4, 1, 24, 16), (3, 3, 80, 16), (2, 1, 256, 32),

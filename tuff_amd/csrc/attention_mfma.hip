@@ -90,7 +90,7 @@ constexpr int UNIT = 64;                   // keys a unit: two steps of 32
 constexpr int UNITS = PART / UNIT;
 
 // NW: waves a workgroup (1: the wave walks the partition's four units; 4: a unit a wave, merged through LDS).
-template <int HDP, int NB, int NW, bool FUSED, bool STREAM_V>
+template <int HDP, int NB, int NW, bool FUSED, bool STREAM_V, bool STAGE_K = false>
 __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
     float* __restrict__ ws_o, float* __restrict__ ws_ml,
@@ -192,6 +192,27 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
     // into registers a step ahead of their use (where the head size leaves room for it); large
     // tiles (head size x columns) load as they go.
     constexpr bool AHEAD = HDP * NB <= 256;
+    // STAGE_K (heads of up to 64 channels): a step's keys are asked for as they lie in memory, 1 KB an instruction (the
+    // 16 keys of a half are one run of 16 hd elements), and go through LDS into the order of the matrix operands.  Asked
+    // for in that order at once, an instruction touches half of each of sixteen lines and every line is asked for twice:
+    // with several rounds of waves on the chip the memory side is what bounds the kernel, and whole lines are 3 to 7 %
+    // faster (16,384 workgroups; nothing at 6,144); with one round the trip through LDS only adds to each wave's chain
+    // (3 to 7 % slower), so the launch chooses.
+    static_assert(!STAGE_K || (HDP == 64 && HDP * NB <= 256 && NW == 1), "staged keys: heads of up to 64, one wave a partition");
+    constexpr bool STAGE = STAGE_K;
+    __shared__ __attribute__((aligned(16))) bf16_t k_stage[STAGE ? NW : 1][STAGE ? 32 * 64 : 8];
+    // where the 16-byte piece `chunk` of key `key` of the step lies in the wave's 4 KB: rows of 128 bytes, the pieces of
+    // a row exchanged so that the sixteen rows an operand read takes its pieces from fall into different banks
+    auto stage_at = [&](int key, int chunk) { return key * 64 + ((chunk ^ (((key >> 1) & 1) | (((key >> 3) & 3) << 1))) * 8); };
+    const int row_pieces = hd / 8;                                   // 16-byte pieces of a key
+    int stage_to[2][2];                                              // where this lane's four pieces of a step go (-1: no piece)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int piece = 64 * i + lane;
+            stage_to[h][i] = (STAGE && piece < 16 * row_pieces) ? stage_at(16 * h + piece / row_pieces, piece % row_pieces) : -1;
+        }
     struct Tile {
         bf16x8 kf[2][AHEAD ? KC : 1];
         bf16x8 vx[AHEAD ? DB : 1];
@@ -234,7 +255,20 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
             t.off0[h] = hs % page_size;
             t.base[h] = (page * Hkv + kvh) * (long long)page_size * hd;
         }
-        if constexpr (AHEAD) {
+        if constexpr (STAGE) {
+            // kf[h][i]: pieces 64 i + lane of half h, as they lie in memory
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const int piece = 64 * i + lane;
+                    bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+                    t.kf[h][i] = (t.live[h] && stage_to[h][i] >= 0)
+                        ? __builtin_nontemporal_load((const bf16x8*)(k_cache + t.base[h] + (long long)t.off0[h] * hd + piece * 8)) : z;
+                }
+#pragma unroll
+            for (int db = 0; db < DB; ++db) t.vx[db] = v_frag(t, db);
+        } else if constexpr (AHEAD) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -317,6 +351,16 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
     auto compute = [&](int key0, const Tile& t) {
         // ---- S^T = K Q^T, twice 16 keys
         f32x4 s[2][NB];
+        bf16_t* stage = k_stage[STAGE ? wave : 0];
+        if constexpr (STAGE) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    if (stage_to[h][i] >= 0) *(bf16x8*)(stage + stage_to[h][i]) = t.kf[h][i];
+                }
+            __builtin_amdgcn_wave_barrier();       // the wave's LDS accesses run in the order of the program
+        }
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
@@ -324,7 +368,11 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
 #pragma unroll
             for (int kc = 0; kc < KC; ++kc) {
                 bf16x8 kf;
-                if constexpr (AHEAD) kf = t.kf[kb][kc]; else kf = k_frag(t, kb, kc);
+                if constexpr (STAGE) {
+                    bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+                    const int chunk = kc * 4 + g;
+                    kf = chunk < row_pieces ? *(const bf16x8*)(stage + stage_at(8 * (n16 / 4) + 4 * kb + n16 % 4, chunk)) : z;
+                } else if constexpr (AHEAD) kf = t.kf[kb][kc]; else kf = k_frag(t, kb, kc);
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) s[kb][nb] = mfma32(kf, qf[nb][kc], s[kb][nb]);
             }
@@ -652,6 +700,8 @@ int few_waves = 2048;
 // several rounds of waves on the chip (it holds about 3,000 of them) that is 7 to 11 % faster, with one
 // round it is not.
 int kv_fast_waves = 6144;
+// From how many workgroups on the keys of heads of up to 64 channels go through LDS (STAGE_K of the kernel).
+int stage_k_waves = 8192;
 
 template <int HDP, int NB, bool FUSED, bool STREAM_V = true>
 void launch_partition(dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* kc, bf16_t* vc, float* ws_o,
@@ -671,6 +721,13 @@ void launch_partition(dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* kc
         // the fused form prepares its queries in every wave: four waves pay for that four times
         if (waves < (FUSED ? few_waves / 2 : few_waves)) {
             hipLaunchKernelGGL((attn_partition_kernel<HDP, NB, UNITS, FUSED, STREAM_V>), grid, dim3(UNITS * WAVE), 0, stream, q, kc, vc, ws_o,
+                               ws_ml, bt, max_blocks, blk, req_info, H, Hkv, hd, ps, window, scale, n_parts, fq, kv_fast);
+            return;
+        }
+    }
+    if constexpr (HDP == 64 && HDP * NB <= 256) {
+        if (waves >= stage_k_waves) {
+            hipLaunchKernelGGL((attn_partition_kernel<HDP, NB, 1, FUSED, STREAM_V, true>), grid, dim3(WAVE), 0, stream, q, kc, vc, ws_o,
                                ws_ml, bt, max_blocks, blk, req_info, H, Hkv, hd, ps, window, scale, n_parts, fq, kv_fast);
             return;
         }
@@ -744,6 +801,14 @@ TUFF_EXPORT int tuff_attention_few_waves(int n) {
 
 // From how many workgroups on the kv head changes fastest in the order of the workgroups.  For
 // measurements and tests; the result does not depend on it.  Returns the value before.
+// From how many workgroups on keys are asked for in whole lines and go through LDS.  For measurements and tests; the
+// result does not depend on it.  Returns the value before.
+TUFF_EXPORT int tuff_attention_stage_k_waves(int n) {
+    const int old = stage_k_waves;
+    if (n >= 0) stage_k_waves = n;
+    return old;
+}
+
 TUFF_EXPORT int tuff_attention_kv_fast_waves(int n) {
     const int old = kv_fast_waves;
     if (n >= 0) kv_fast_waves = n;
