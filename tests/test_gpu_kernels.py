@@ -583,6 +583,24 @@ def test_attention_mfma(gpu, H, Hkv, hd, ps, window):
         _check_step(case, reqs, got, H, hd, window, nb)
 
 
+@pytest.mark.parametrize("H,Hkv,hd,ps", [(8, 2, 64, 96), (4, 1, 64, 112), (6, 3, 32, 144), (4, 2, 128, 96), (4, 4, 64, 272)])
+@pytest.mark.parametrize("window", [0, 300])
+def test_attention_mfma_on_pages_that_do_not_divide_a_partition(gpu, H, Hkv, hd, ps, window):
+    """Pages of 96, 112, 144 and 272 positions: a partition of 256 keys that starts inside a page touches one
+    page more than 256 / page size rounded up (the partition at key 256 of pages of 96: pages 2 to 5).
+    Contexts beyond 1,100 keys, every partition start among them; stale pages hold NaN."""
+    from tuff_amd.csrc import ops
+    reqs = [(1199, 1), (1150, 40), (0, 33), (255, 3), (511, 2), (767, 1), (1023, 2), (300, 1)]
+    case = _mixed_step_case(gpu, reqs, H, Hkv, hd, ps)
+    T = case["q"].shape[0]
+    blocks = torch.from_numpy(ops.query_blocks(case["q_len"], H // Hkv, 1)).to(gpu)
+    out = torch.full((T, H * hd), float("nan"), dtype=torch.bfloat16, device=gpu)
+    ops.attention_mfma(case["q"].to(gpu), case["kc"], case["vc"], out, block_table=case["table"],
+                       blocks=blocks, nb=1, req_info=case["req_info"], positions=case["positions"], H=H, Hkv=Hkv,
+                       hd=hd, page_size=ps, max_ctx_len=case["max_ctx_len"], window=window)
+    _check_step(case, reqs, out.cpu().double().reshape(T, H, hd), H, hd, window, ps)
+
+
 def _decode_case(gpu, R, H, Hkv, ps, lens, seed=0, nan_pool=True):
     """R requests with lens[r] tokens in the cache after this step; the step brings each one's last
     token as a projected row [q heads | k heads | v heads] of heads of 64.  Pages shuffled."""
@@ -609,7 +627,7 @@ def _decode_case(gpu, R, H, Hkv, ps, lens, seed=0, nan_pool=True):
                 req_info=i32([[r, 1, n - 1, n] for r, n in enumerate(lens)]), max_ctx_len=max(lens))
 
 
-@pytest.mark.parametrize("H,Hkv,ps", [(32, 8, 16), (6, 3, 64), (16, 1, 32)])
+@pytest.mark.parametrize("H,Hkv,ps", [(32, 8, 16), (6, 3, 64), (16, 1, 32), (8, 2, 96), (4, 1, 112)])
 @pytest.mark.parametrize("window", [0, 300])
 @pytest.mark.parametrize("norm_dt", [torch.float32, torch.bfloat16, None])
 def test_attention_decode_fused_equals_the_separate_kernels(gpu, H, Hkv, ps, window, norm_dt):
@@ -618,7 +636,7 @@ def test_attention_decode_fused_equals_the_separate_kernels(gpu, H, Hkv, ps, win
     kernel: the same cache and the same output, bit for bit; stale pages hold NaN."""
     from tuff_amd.csrc import ops
     hd, eps, base = 64, 1e-6, 1e6
-    lens = [700, 1, 257, 256, 33, 1025, 64]
+    lens = [700, 1, 257, 256, 33, 1025, 64, 1290]
     R = len(lens)
     qw = kw = None
     if norm_dt is not None:

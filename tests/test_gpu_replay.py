@@ -75,6 +75,32 @@ def test_heads_of_64_and_other_page_sizes(gpu, page_size, dtype):
     check_plan("E", dtype, plan, reqs, page_size=page_size, max_tokens=peak, max_requests=4)
 
 
+@pytest.mark.parametrize("page_size", [96, 112])
+def test_pages_that_do_not_divide_a_partition_of_keys(gpu, page_size):
+    """Pages of 96 and 112 positions under a request of 1,200 tokens in bfloat16: the single-token attention cuts
+    the keys into partitions of 256, and a partition that starts inside a page touches one page more than
+    256 / page size rounded up.  A head in portions, then single tokens across the partition edge at 1,024
+    and beyond 1,100, beside a short request."""
+    V = util.CONFIGS["E"][0]["vocab_size"]
+    reqs = {"long": util.rand_tokens(1200, V, 77), "short": util.rand_tokens(140, V, 78)}
+    steps, at = [], {"long": 0, "short": 0}
+
+    def step(parts):
+        entries = []
+        for rid, n in parts:
+            toks = reqs[rid][at[rid]:at[rid] + n]
+            at[rid] += len(toks)
+            if toks:
+                entries.append({"id": rid, "tokens": toks, "want": list(range(len(toks)))})
+        steps.append({"step": len(steps), "entries": entries, "end": []})
+    step([("long", 500)])
+    step([("long", 500), ("short", 100)])
+    while at["long"] < 1200:
+        step([("long", 1), ("short", 1)])
+    steps[-1]["end"] = ["long", "short"]
+    check_plan("E", "bfloat16", steps, reqs, page_size=page_size, max_tokens=16 * page_size)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name,n_req", [("A+", 20), ("E", 37), ("B+", 64)])
 def test_many_requests_decode_together(gpu, name, n_req, dtype):

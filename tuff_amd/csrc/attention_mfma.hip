@@ -89,6 +89,13 @@ __device__ __forceinline__ float merged(float a, float ca, float b, float cb) { 
 constexpr int UNIT = 64;                   // keys a unit: two steps of 32
 constexpr int UNITS = PART / UNIT;
 
+// How many pages the partition that starts at key_begin (a multiple of PART) touches: one lane of the
+// wave fetches each page's number.  A partition that starts inside a page (page sizes that do not divide
+// PART) touches one page more than PART / page_size rounded up.
+__host__ __device__ inline int partition_pages(int key_begin, int page_size) {
+    return (key_begin + PART - 1) / page_size - key_begin / page_size + 1;
+}
+
 // NW: waves a workgroup (1: the wave walks the partition's four units; 4: a unit a wave, merged through LDS).
 template <int HDP, int NB, int NW, bool FUSED, bool STREAM_V, bool STAGE_K = false>
 __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
@@ -118,7 +125,7 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
     const int key_begin = part * PART;
     const int first_page = key_begin / page_size;
     int my_page = -1;                      // lane i: the page of the partition's i-th block of page_size keys
-    if (lane < (PART + page_size - 1) / page_size && first_page + lane < max_blocks) my_page = table[first_page + lane];
+    if (lane < partition_pages(key_begin, page_size) && first_page + lane < max_blocks) my_page = table[first_page + lane];
 
     // the block's range of keys
     const int last_col = min(ncols, col0 + NB * 16) - 1;
@@ -789,6 +796,13 @@ static int launch_attention(const void* q, const void* k_cache, const void* v_ca
     if (rc) return rc;
     return launch_merge((const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, n_tokens, H, hd, window, n_parts, PART,
                         stream);
+}
+
+// The number of lanes of a wave that fetch page numbers for partition `part` with pages of page_size
+// positions (what the kernel computes; host arithmetic, for checks).
+TUFF_EXPORT int tuff_attention_partition_pages(int part, int page_size) {
+    if (part < 0 || page_size <= 0 || (long long)part * PART + PART > 0x7fffffffll) return -2;
+    return partition_pages(part * PART, page_size);
 }
 
 // Below how many workgroups a step's partitions get four waves each (0: never).  For measurements and
