@@ -77,6 +77,94 @@ def test_random_folder_loads_back_and_is_reproducible(tmp_path):
     assert torch.equal(t1, t2)
 
 
+def test_the_generator_is_the_specified_one(monkeypatch):
+    """Every element against the numpy restatement of the generator's text (tests/plain/random_plain.py, which
+    shares no code with it): the float64 deviates bit for bit, the float32 values, the bfloat16 bits; the same
+    whether a tensor is made whole or in pieces; and against the library's ln, cos and root to 1e-14."""
+    import math
+    import numpy as np
+    from plain import random_plain
+    from tuff_amd.parts.base import WeightDecl
+    name, seed, n = "model.layers.3.feed_forward.w1.weight", 5, 70001
+    z = random_init.normal_deviates(random_init.tensor_key(seed, name), 0, n).numpy()
+    zp = random_plain.deviates(seed, name, n)
+    assert np.array_equal(z.view(np.uint64), zp.view(np.uint64))
+    # against the formula with the library's functions, from the text's integers
+    key, G = random_init.tensor_key(seed, name), random_init.GOLDEN
+    for i in (0, 1, 2, 999, 70000):
+        a, b = random_init._mix_int(key + (2 * i + 1) * G), random_init._mix_int(key + (2 * i + 2) * G)
+        u1, u2 = ((a >> 11) + 1) * 2.0 ** -53, (b >> 11) * 2.0 ** -53
+        assert abs(z[i] - math.sqrt(-2 * math.log(u1)) * math.cos(2 * math.pi * u2)) < 1e-14
+    # the extremes of the uniform draws: nothing non-finite, the root of zero is harmless
+    assert abs(z.mean()) < 0.02 and abs(z.std() - 1) < 0.01 and abs((z ** 4).mean() - 3) < 0.15 and np.abs(z).max() > 3.5
+    for init, shape in (("normal", (37, 53)), ("norm", (97,))):
+        d = WeightDecl("some.weight", shape, init)
+        want32 = random_plain.tensor_f32(9, "some.weight", shape, init)
+        assert np.array_equal(random_init.random_tensor(d, 9, torch.float32).numpy().view(np.uint32), want32.view(np.uint32))
+        got16 = random_init.random_tensor(d, 9, torch.bfloat16)
+        assert np.array_equal(got16.view(torch.int16).numpy().view(np.uint16), random_plain.to_bfloat16_bits(want32))
+        monkeypatch.setitem(random_init.CHUNK, "cpu", 11)             # in pieces of 11 elements: the same tensor
+        assert torch.equal(random_init.random_tensor(d, 9, torch.bfloat16), got16)
+        monkeypatch.setitem(random_init.CHUNK, "cpu", 1 << 21)
+    # another seed, another name: other values
+    d1, d2 = WeightDecl("a.weight", (64,), "normal"), WeightDecl("b.weight", (64,), "normal")
+    assert not torch.equal(random_init.random_tensor(d1, 1, torch.float32), random_init.random_tensor(d2, 1, torch.float32))
+    assert not torch.equal(random_init.random_tensor(d1, 1, torch.float32), random_init.random_tensor(d1, 2, torch.float32))
+
+
+@pytest.mark.parametrize("stored", [torch.bfloat16, torch.float32])
+def test_a_seed_is_one_model_whichever_entry_point_makes_it(tmp_path, stored):
+    """random_weights() (what Engine.from_config and `tuff --random` use) and write_random_model() read back
+    (what the C interface's tuff_model_write_random and the tests' folders use): the same bits."""
+    cfg, model, decls = model_and_decls("B")
+    folder = random_init.write_random_model(cfg, str(tmp_path / "m"), seed=4, dtype=stored, device="cpu")
+    for run in (torch.bfloat16, torch.float32):
+        made = random_init.random_weights(decls, 4, run, "cpu", stored_dtype=stored)
+        read = loader.load_weights(folder, decls, run, "cpu")
+        assert set(made) == set(read)
+        for k in made:
+            assert made[k].dtype == read[k].dtype and torch.equal(made[k], read[k]), k
+
+
+def test_a_checkpoint_in_several_files(tmp_path):
+    """model.safetensors.index.json names the file of every tensor: the same weights as from one file."""
+    cfg, model, decls = model_and_decls("A")
+    folder = random_init.write_random_model(cfg, str(tmp_path / "m"), seed=0)
+    whole = loader.load_weights(folder, decls, torch.bfloat16, "cpu")
+    st = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+    names = st.names()
+    parts = {"model-00001-of-00002.safetensors": names[::2], "model-00002-of-00002.safetensors": names[1::2]}
+    for fn, ns in parts.items():
+        write_safetensors(os.path.join(folder, fn), [(n, st.shape(n), st.dtype(n)) for n in ns], st.read)
+    with open(os.path.join(folder, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {}, "weight_map": {n: fn for fn, ns in parts.items() for n in ns}}, f)
+    os.unlink(os.path.join(folder, "model.safetensors"))
+    sharded = loader.load_weights(folder, decls, torch.bfloat16, "cpu")
+    assert all(torch.equal(whole[k], sharded[k]) for k in whole)
+    # an index that names a tensor its file does not hold, or a file outside the folder
+    with open(os.path.join(folder, "model.safetensors.index.json"), "w") as f:
+        json.dump({"weight_map": {n: "model-00001-of-00002.safetensors" for n in names}}, f)
+    with pytest.raises(loader.WeightsError):
+        loader.load_weights(folder, decls, torch.bfloat16, "cpu")
+    with open(os.path.join(folder, "model.safetensors.index.json"), "w") as f:
+        json.dump({"weight_map": {names[0]: "../x.safetensors"}}, f)
+    with pytest.raises(loader.WeightsError):
+        loader.load_weights(folder, decls, torch.bfloat16, "cpu")
+
+
+def test_tensors_the_model_does_not_know_are_a_warning_listed_once(tmp_path):
+    cfg, model, decls = model_and_decls("A")
+    folder = random_init.write_random_model(cfg, str(tmp_path / "m"), seed=0)
+    before = loader.load_weights(folder, decls, torch.bfloat16, "cpu")
+    _rewrite(folder, lambda t: t.update({"model.layers.9.extra.weight": torch.zeros(2), "rotary.inv_freq": torch.zeros(8)}))
+    with pytest.warns(loader.UnexpectedTensorsWarning) as rec:
+        after = loader.load_weights(folder, decls, torch.bfloat16, "cpu")
+    assert len(rec) == 1 and rec[0].message.names == ["model.layers.9.extra.weight", "rotary.inv_freq"]
+    assert set(after) == set(before) and all(torch.equal(before[k], after[k]) for k in before)
+    with pytest.raises(loader.WeightsError, match=r"unexpected tensors \(2\)"):
+        loader.load_weights(folder, decls, torch.bfloat16, "cpu", strict=True)
+
+
 def test_types_are_kept_as_stored(tmp_path):
     cfg, model, decls = model_and_decls("A")
     folder = random_init.write_random_model(cfg, str(tmp_path / "f32"), seed=0, dtype=torch.float32)
@@ -129,7 +217,10 @@ def test_tied_and_untied_heads(tmp_path):
     folder = random_init.write_random_model(cfg, str(tmp_path / "tied"), seed=0)
     _rewrite(folder, lambda t: t.update({"lm_head.weight": torch.zeros(512, 64, dtype=torch.bfloat16)}))
     with pytest.raises(loader.WeightsError, match="unexpected tensors"):
-        loader.load_weights(folder, decls, torch.bfloat16, "cpu")
+        loader.load_weights(folder, decls, torch.bfloat16, "cpu", strict=True)
+    with pytest.warns(loader.UnexpectedTensorsWarning, match="lm_head.weight"):    # a tied model reads no head of its own
+        w = loader.load_weights(folder, decls, torch.bfloat16, "cpu")
+    assert "lm_head.weight" not in w
     cfg, model, decls = model_and_decls("B")                                 # untied
     folder = random_init.write_random_model(cfg, str(tmp_path / "untied"), seed=0)
     _rewrite(folder, lambda t: t.pop("lm_head.weight"))
