@@ -10,7 +10,7 @@ for p in (ROOT, os.path.dirname(os.path.abspath(__file__))):
 
 
 def pytest_configure(config):
-    config.addinivalue_line("markers", "gpu: needs a gfx950 GPU (run on the GPU box)")
+    config.addinivalue_line("markers", "gpu: needs a gfx950 GPU")
 
 
 @pytest.fixture(scope="session")

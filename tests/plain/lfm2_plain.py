@@ -6,6 +6,19 @@ shares neither loader, nor layers, nor cache with the engine under test.
 
 Everything runs on the CPU in the dtype of the tensors handed in (float64 by
 default).
+
+`rnd`: where given, a function applied to every activation that an engine with
+bfloat16 activations holds in bfloat16 between two of its operations: the normed
+operand of every projection, a projection's output (q, k, v; B, C, X), the normed
+and rotated q and k (the cache holds such keys) and v, the softmax weights as the
+second product takes them, the attention's output, the gated conv output and the
+SwiGLU product.  The residual stream, the sums inside every product, the norms'
+statistics, the softmax and the conv's own sums stay as they are.  With
+rnd = "round to bfloat16 and back" in float64 arithmetic this is a model of the
+rounding noise that any such engine has, however it orders its sums: the
+tests' yardstick for an engine's bfloat16 error, in the manner of the reference's
+tolerance gate, which measures its engine against another runtime's error
+(tools/lfm25_gate.py:117-144).
 """
 from __future__ import annotations
 
@@ -41,8 +54,16 @@ def rope_neox(x: torch.Tensor, pos: torch.Tensor, base: float) -> torch.Tensor:
     return torch.cat([x0 * c - x1 * s, x0 * s + x1 * c], dim=-1)
 
 
+def _same(t):
+    return t
+
+
+def to_bfloat16_and_back(t: torch.Tensor) -> torch.Tensor:
+    return t.to(torch.bfloat16).to(t.dtype)
+
+
 def short_conv(h: torch.Tensor, w_in: torch.Tensor, w_conv: torch.Tensor,
-               w_out: torch.Tensor) -> torch.Tensor:
+               w_out: torch.Tensor, rnd=_same) -> torch.Tensor:
     """Gated short convolution over a whole sequence that starts with empty history.
 
     bcx = W_in h; B, C, X = thirds of bcx; u = B*X;
@@ -53,18 +74,18 @@ def short_conv(h: torch.Tensor, w_in: torch.Tensor, w_conv: torch.Tensor,
     """
     T, d = h.shape
     K = w_conv.shape[1]
-    bcx = h @ w_in.T
+    bcx = rnd(h @ w_in.T)
     b, c, xx = bcx[:, :d], bcx[:, d:2 * d], bcx[:, 2 * d:]
     u = b * xx
     hist = torch.cat([torch.zeros(K - 1, d, dtype=h.dtype), u], dim=0)   # row i = time i-(K-1)
     y = torch.zeros_like(u)
     for k in range(K):
         y = y + hist[k:k + T] * w_conv[:, k]
-    return (c * y) @ w_out.T
+    return rnd(c * y) @ w_out.T
 
 
 def attention(h: torch.Tensor, wq, wk, wv, wo, q_norm_w, k_norm_w, *, n_head: int,
-              n_kv: int, eps: float, base: float, pos0: int = 0) -> torch.Tensor:
+              n_kv: int, eps: float, base: float, pos0: int = 0, rnd=_same) -> torch.Tensor:
     """Causal GQA attention with per-head RMSNorm on q and k, then rotation.
 
     q head i reads kv head i // (n_head // n_kv); scores scaled by 1/sqrt(hd);
@@ -74,11 +95,11 @@ def attention(h: torch.Tensor, wq, wk, wv, wo, q_norm_w, k_norm_w, *, n_head: in
     T, _ = h.shape
     hd = wq.shape[0] // n_head
     pos = torch.arange(pos0, pos0 + T)
-    q = (h @ wq.T).reshape(T, n_head, hd)
-    k = (h @ wk.T).reshape(T, n_kv, hd)
-    v = (h @ wv.T).reshape(T, n_kv, hd)
-    q = rope_neox(rms_norm(q, q_norm_w, eps), pos, base)
-    k = rope_neox(rms_norm(k, k_norm_w, eps), pos, base)
+    q = rnd(h @ wq.T).reshape(T, n_head, hd)
+    k = rnd(h @ wk.T).reshape(T, n_kv, hd)
+    v = rnd(h @ wv.T).reshape(T, n_kv, hd)
+    q = rnd(rope_neox(rms_norm(q, q_norm_w, eps), pos, base))
+    k = rnd(rope_neox(rms_norm(k, k_norm_w, eps), pos, base))
     g = n_head // n_kv
     k = k.repeat_interleave(g, dim=1)
     v = v.repeat_interleave(g, dim=1)
@@ -86,19 +107,19 @@ def attention(h: torch.Tensor, wq, wk, wv, wo, q_norm_w, k_norm_w, *, n_head: in
     mask = torch.ones(T, T, dtype=torch.bool).tril()
     s = s.masked_fill(~mask, float("-inf"))
     s = torch.exp(s - s.max(-1, keepdim=True).values)
-    s = s / s.sum(-1, keepdim=True)
-    o = torch.einsum("hts,shd->thd", s, v).reshape(T, n_head * hd)
-    return o @ wo.T
+    total = s.sum(-1, keepdim=True)
+    o = torch.einsum("hts,shd->thd", rnd(s), v) / total.permute(1, 0, 2)
+    return rnd(o.reshape(T, n_head * hd)) @ wo.T
 
 
-def swiglu(h: torch.Tensor, w_gate, w_up, w_down) -> torch.Tensor:
+def swiglu(h: torch.Tensor, w_gate, w_up, w_down, rnd=_same) -> torch.Tensor:
     """W_down (g / (1 + exp(-g)) * u) with g = W_gate h, u = W_up h.
 
     tools/lfm25_fp64_ref.py:159-161; src/lfm25_gpu.cu:614-617.
     """
     g = h @ w_gate.T
     u = h @ w_up.T
-    return (g / (1.0 + torch.exp(-g)) * u) @ w_down.T
+    return rnd(g / (1.0 + torch.exp(-g)) * u) @ w_down.T
 
 
 # --------------------------------------------------------------------------- model
@@ -135,7 +156,7 @@ def layer_is_conv(cfg: dict, i: int) -> bool:
     return cfg["layer_types"][i] == "conv"
 
 
-def forward_logits(cfg: dict, w: dict, tokens, dtype=torch.float64) -> torch.Tensor:
+def forward_logits(cfg: dict, w: dict, tokens, dtype=torch.float64, rnd=_same) -> torch.Tensor:
     """Logits [T, vocab] of one whole sequence starting at position 0.
 
     Pre-norm decoder, two residual sub-blocks a layer: x += mixer(norm(x));
@@ -150,22 +171,22 @@ def forward_logits(cfg: dict, w: dict, tokens, dtype=torch.float64) -> torch.Ten
     x = w["model.embed_tokens.weight"][tok].to(dtype)
     for i in range(int(cfg["num_hidden_layers"])):
         p = f"model.layers.{i}."
-        h = rms_norm(x, w[p + "operator_norm.weight"], eps)
+        h = rnd(rms_norm(x, w[p + "operator_norm.weight"], eps))
         if layer_is_conv(cfg, i):
             conv_w = w[p + "conv.conv.weight"]
             conv_w = conv_w.reshape(conv_w.shape[0], conv_w.shape[-1])
-            o = short_conv(h, w[p + "conv.in_proj.weight"], conv_w, w[p + "conv.out_proj.weight"])
+            o = short_conv(h, w[p + "conv.in_proj.weight"], conv_w, w[p + "conv.out_proj.weight"], rnd=rnd)
         else:
             o = attention(h, w[p + "self_attn.q_proj.weight"], w[p + "self_attn.k_proj.weight"],
                           w[p + "self_attn.v_proj.weight"], w[p + "self_attn.out_proj.weight"],
                           w[p + "self_attn.q_layernorm.weight"], w[p + "self_attn.k_layernorm.weight"],
-                          n_head=n_head, n_kv=n_kv, eps=eps, base=base)
+                          n_head=n_head, n_kv=n_kv, eps=eps, base=base, rnd=rnd)
         x = x + o
-        h = rms_norm(x, w[p + "ffn_norm.weight"], eps)
+        h = rnd(rms_norm(x, w[p + "ffn_norm.weight"], eps))
         x = x + swiglu(h, w[p + "feed_forward.w1.weight"], w[p + "feed_forward.w3.weight"],
-                       w[p + "feed_forward.w2.weight"])
+                       w[p + "feed_forward.w2.weight"], rnd=rnd)
     head = w["lm_head.weight"] if "lm_head.weight" in w else w["model.embed_tokens.weight"]
-    return rms_norm(x, w["model.embedding_norm.weight"], eps) @ head.T
+    return rnd(rms_norm(x, w["model.embedding_norm.weight"], eps)) @ head.T
 
 
 def greedy_generate(cfg: dict, w: dict, prompt, n_new: int, dtype=torch.float64):

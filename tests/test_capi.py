@@ -89,7 +89,7 @@ def test_c_program_steps_generates_and_schedules(gpu, client, tmp_path, dtype):
 
     # the step function's logits at every position against the plain implementation
     got = torch.from_numpy(np.fromfile(logits_file, dtype="<f4").reshape(len(prompt), V).copy())
-    util.assert_close(dtype, got, util.plain_logits(name, prompt, stored), "C step")
+    util.assert_close(dtype, got, util.expected(name, prompt, stored), "C step")
 
     # generation and the scheduler calls against the Python entry point in this process
     llm = LLM(folder, dtype=dtype, max_num_seqs=4, ctx_size=512)

@@ -48,3 +48,23 @@ def test_the_scratch_copy_holds_sources_only(scratch):
         assert not [f for f in files if f.endswith((".so", ".pyc"))], folder
     assert os.path.islink(os.path.join(scratch, "tuff_amd", "csrc", "_lib")) or \
         not os.path.isdir(os.path.join(util.ROOT, "tuff_amd", "csrc", "_lib"))
+
+
+def test_the_frozen_vectors_are_well_formed():
+    """tests/golden/*.json: one file a configuration, a sha256 and a first choice for every row of every fixed
+    request, the fingerprint of the environment that made them, and the configurations that were byte-identical."""
+    import json
+    import golden
+    for name in golden.NAMES:
+        with open(golden.path_of(name)) as f:
+            g = json.load(f)
+        assert g["format"] == golden.FORMAT and g["configuration"] == name and g["dtype"] == "float32"
+        reqs = golden.requests_for(name)
+        assert set(g["requests"]) == set(reqs)
+        for rid, toks in reqs.items():
+            r = g["requests"][rid]
+            assert r["tokens"] == len(toks) == len(r["row_sha256"]) == len(r["top1"])
+            assert all(len(h) == 64 and int(h, 16) >= 0 for h in r["row_sha256"])
+        assert set(g["environment"]["fingerprint"]) == {"gpu_arch", "hipcc"}
+        assert len(g["provenance"]["configurations_verified_identical"]) == len(golden.configurations()) and g["provenance"]["reason"]
+        assert len(g["model"]["safetensors_sha256"]) == 64

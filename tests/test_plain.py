@@ -131,6 +131,67 @@ def test_attention_reduces_to_library_attention():
     assert torch.allclose(normed, o2.transpose(0, 1).reshape(T, d) @ wo.T)
 
 
+def test_the_per_head_norm_of_q_and_k_uses_the_models_eps():
+    """src/lfm25_engine.c:395 hands the model's one eps to the kernel that norms q and k per head
+    (src/lfm25_gpu.cu:420-452: rsqrtf(total_sq / head_dim + eps)), and tools/lfm25_fp64_ref.py:131-132 uses the same
+    rms() closure as for the layers' norms.  Configuration G has norm_eps = 0.5, far above a head's mean square, so
+    another eps for the heads (1e-5, 1e-6, none) changes the scores many times over.  By hand, without the plain
+    implementation's functions: one normed element of q, and the whole first layer's attention for two tokens."""
+    cfg, w = util.plain_model("G")
+    eps, H, base = cfg["norm_eps"], cfg["num_attention_heads"], cfg["rope_theta"]
+    assert eps == 0.5 and cfg["layer_types"][0] == "full_attention" and cfg["num_key_value_heads"] == H
+    hd = cfg["hidden_size"] // H
+    toks = [3, 77]
+    x = w["model.embed_tokens.weight"][toks]                                         # [2, d]
+    nw = w["model.layers.0.operator_norm.weight"]
+    h = torch.stack([x[t] / math.sqrt(float((x[t] ** 2).sum()) / x.shape[1] + eps) * nw for t in range(2)])
+    p = "model.layers.0.self_attn."
+    q, k, v = h @ w[p + "q_proj.weight"].T, h @ w[p + "k_proj.weight"].T, h @ w[p + "v_proj.weight"].T
+    qn, kn = w[p + "q_layernorm.weight"], w[p + "k_layernorm.weight"]
+    head, j = 2, 5
+    qh = q[1, head * hd:(head + 1) * hd]
+    ms = float((qh ** 2).sum()) / hd
+    assert ms < eps / 5                                                              # eps decides the size
+    want_q = float(qh[j]) / math.sqrt(ms + eps) * float(qn[j])
+    got_q = plain.rms_norm(q.reshape(2, H, hd), qn, eps)[1, head, j]
+    assert math.isclose(float(got_q), want_q, rel_tol=1e-12)
+    # token 1's attention output in every head, by hand: norm with eps, rotate the halves, two scores, softmax
+    def normed_rotated(vec, weight, pos):
+        out = torch.empty_like(vec)
+        for a in range(H):
+            hv = vec[a * hd:(a + 1) * hd]
+            hv = hv / math.sqrt(float((hv ** 2).sum()) / hd + eps) * weight
+            for i in range(hd // 2):
+                ang = pos * base ** (-2.0 * i / hd)
+                out[a * hd + i] = hv[i] * math.cos(ang) - hv[i + hd // 2] * math.sin(ang)
+                out[a * hd + i + hd // 2] = hv[i] * math.sin(ang) + hv[i + hd // 2] * math.cos(ang)
+        return out
+    q1, k0, k1 = normed_rotated(q[1], qn, 1), normed_rotated(k[0], kn, 0), normed_rotated(k[1], kn, 1)
+    o = torch.empty(H * hd, dtype=torch.float64)
+    for a in range(H):
+        sl = slice(a * hd, (a + 1) * hd)
+        s0, s1 = float(q1[sl] @ k0[sl]) / math.sqrt(hd), float(q1[sl] @ k1[sl]) / math.sqrt(hd)
+        p0 = 1.0 / (1.0 + math.exp(s1 - s0))
+        o[sl] = p0 * v[0, sl] + (1 - p0) * v[1, sl]
+    want = o @ w[p + "out_proj.weight"].T
+    got = plain.attention(h, w[p + "q_proj.weight"], w[p + "k_proj.weight"], w[p + "v_proj.weight"], w[p + "out_proj.weight"],
+                          qn, kn, n_head=H, n_kv=H, eps=eps, base=base)[1]
+    assert torch.allclose(got, want, rtol=1e-10, atol=1e-14)
+    # ... and the whole model hands that eps on: with the layers' outputs after the first mixer zeroed, the logits
+    # of token 1 are head(norm(x + attention)) with the attention computed above
+    w0 = dict(w)
+    for name in w:
+        if name.endswith("feed_forward.w2.weight") or (name.endswith("out_proj.weight") and ".layers.0." not in name):
+            w0[name] = torch.zeros_like(w[name])
+    x1 = x[1] + want
+    fin = x1 / math.sqrt(float((x1 ** 2).sum()) / x1.shape[0] + eps) * w["model.embedding_norm.weight"]
+    assert torch.allclose(plain.forward_logits(cfg, w0, toks)[1], fin @ w["lm_head.weight"].T, rtol=1e-10, atol=1e-14)
+    # the pin bites: the same with the heads normed by another eps is far off
+    other = plain.attention(h, w[p + "q_proj.weight"], w[p + "k_proj.weight"], w[p + "v_proj.weight"], w[p + "out_proj.weight"],
+                            qn, kn, n_head=H, n_kv=H, eps=1e-5, base=base)[1]
+    assert (other - want).abs().max() > 0.02 * want.abs().max()
+
+
 def test_attention_scale_is_one_over_root_of_the_head_size():
     # one head, no rotation effect at position 0 for the key: two tokens, scores by hand
     d = hd = 4

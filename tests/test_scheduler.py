@@ -241,6 +241,50 @@ def test_decoding_requests_take_turns_when_the_budget_is_smaller_than_their_numb
         assert r.output == expected_output([i, i + 1], 9)
 
 
+def test_decoding_requests_take_turns_also_when_every_step_is_decided_ahead():
+    """The serving loop decides step k+1 between advance() and commit() of step k, always with ahead=True: the
+    turn must move on there too, or the same requests run every step and the others starve until those end."""
+    ex = AheadExecutor(num_pages=256, page_size=1)                            # every token needs a page
+    sched = make(ex, max_batched_tokens=4, max_num_seqs=4)
+    reqs = [Request(k, [i, i + 1], SamplingParams(max_new_tokens=40)) for i, k in enumerate("abcd")]
+    for r in reqs:
+        sched.add(r)
+    while any(r.remaining() != 1 or r.status != "running" for r in reqs):     # all four decoding
+        batch = sched.schedule()
+        sched.update(batch, ex.step(batch))
+    sched.max_batched_tokens = 2
+    before = {r.id: len(r.output) for r in reqs}
+    batch = sched.schedule()
+    sampled = ex.step(batch)
+    seen = [{s.request.id for s in batch}]
+    for _ in range(7):                                                        # seven more steps, each decided ahead
+        sched.advance(batch)
+        nxt = sched.schedule(ahead=True)
+        assert nxt and len(nxt) == 2
+        for s in nxt:
+            if PLACEHOLDER in s.tokens:
+                s.tokens = [sampled[s.request.id]]
+        nxt_sampled = ex.step(nxt)
+        sched.commit(batch, sampled)
+        seen.append({s.request.id for s in nxt})
+        batch, sampled = nxt, nxt_sampled
+    sched.advance(batch)
+    sched.commit(batch, sampled)
+    counts = {k: sum(k in b for b in seen) for k in "abcd"}
+    assert set(counts.values()) == {4}, counts                               # 16 tokens, four each
+    assert {r.id: len(r.output) - before[r.id] for r in reqs} == {k: 4 for k in "abcd"}
+    # a refused ahead call leaves the turn where it was
+    turn = sched._decode_turn
+    pool = ex.manager.groups[0].pool
+    pool._free, kept = [], pool._free                                        # no page left: the call is refused
+    assert sched.schedule(ahead=True) is None and sched._decode_turn == turn
+    pool._free = kept
+    sched.max_batched_tokens = 4
+    run(sched, ex)
+    for i, r in enumerate(reqs):
+        assert r.output == expected_output([i, i + 1], 40)
+
+
 def test_waiting_request_is_not_admitted_into_a_full_pool():
     ex = FakeExecutor(num_pages=6, page_size=4)
     sched = make(ex, max_batched_tokens=64)
@@ -472,3 +516,98 @@ def test_random_scenarios_ahead_equal_plain(seed):
         assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == pages and ex.manager.free_slots == 4
         assert sorted(r.id for r in sched.finished) == list(range(len(spec)))
     assert outs["plain"] == outs["ahead"]
+
+
+# ------------------------------------------------------- a step that fails midway
+class _Out:
+    """Stands in for the sampler's output tensor on the device."""
+
+    def __init__(self, values):
+        self.values, self.shape = list(values), (len(values),)
+
+
+class _Pending:
+    def __init__(self, values):
+        self.out = _Out(values)
+
+    def tokens(self):
+        return list(self.out.values)
+
+
+class _FakeSampler:
+    def launch(self, logits, samplers):
+        assert len(logits) == len(samplers)
+        return _Pending(logits)
+
+    def needs_history(self, sampler):
+        return False
+
+
+class _FakeEngine:
+    """Engine.step over the fake executor: resolves tokens that are still 'on the device', checks the order of
+    what it is fed, and fails midway at the call it is told to, as a refused launch would."""
+
+    def __init__(self, ex, fail_at_call):
+        self.ex, self.fail_at_call, self.calls = ex, fail_at_call, 0
+
+    def step(self, entries, device_tokens=None):
+        from tuff_amd.engine.engine import StepFailed
+        self.calls += 1
+        flat = [t for e in entries for t in e.tokens]
+        if device_tokens is not None:
+            if isinstance(device_tokens, _Out):
+                flat = list(device_tokens.values)
+            else:
+                out, places, sources = device_tokens
+                for p, q in zip(places, sources):
+                    flat[p] = out.values[q]
+        if self.calls == self.fail_at_call:
+            raise StepFailed([e.req_id for e in entries], RuntimeError("launch refused")) from RuntimeError("launch refused")
+        logits, at = [], 0
+        for e in entries:
+            toks = flat[at:at + len(e.tokens)]
+            at += len(e.tokens)
+            assert self.ex.manager.length(e.req_id) == len(self.ex.fed[e.req_id])
+            self.ex.manager.extend(e.req_id, len(toks))
+            self.ex.fed[e.req_id] += toks
+            for _ in e.want:
+                logits.append(next_token(self.ex.fed[e.req_id]))
+        self.ex.manager.check()
+        return logits
+
+
+@pytest.mark.parametrize("run_ahead", [True, False])
+@pytest.mark.parametrize("fail_at_call", [1, 2, 4, 7])
+def test_the_run_loop_ends_the_requests_of_a_step_that_failed_midway(fail_at_call, run_ahead):
+    """Engine.step raises StepFailed after some kernels ran: what the step's requests hold is gone.  The loop ends
+    exactly those requests with the reason, their pages and slots come back, nothing that was drawn and not yet
+    seen is left in their output, and the other requests go on to the right tokens when the loop is called again."""
+    import types
+    from tuff_amd.engine.engine import StepFailed
+    from tuff_amd.engine.llm import Loop
+    ex = AheadExecutor(num_pages=64, page_size=4)
+    sched = make(ex, max_batched_tokens=3, max_num_seqs=4)                    # no step holds all four requests
+    reqs = [Request(k, [i, i + 1, i + 2], SamplingParams(max_new_tokens=6)) for i, k in enumerate("abcd")]
+    for r in reqs:
+        sched.add(r)
+    llm = types.SimpleNamespace(engine=_FakeEngine(ex, fail_at_call), sampler=_FakeSampler(), run_ahead=run_ahead)
+    loop = Loop(llm, sched)
+    failures = []
+    for _ in range(200):
+        try:
+            if loop.step() is None:
+                break
+        except StepFailed as e:
+            failures.append(e)
+    assert len(failures) == 1 and not sched.has_unfinished()
+    hit = set(failures[0].requests)
+    assert hit and hit < set("abcd")
+    for i, r in enumerate(reqs):
+        assert r.status == "finished" and PLACEHOLDER not in r.output
+        if r.id in hit:
+            assert r.finish_reason.startswith("error: launch refused")
+            assert r.output == expected_output([i, i + 1, i + 2], 6)[:len(r.output)]       # what it got before is right
+        else:
+            assert r.finish_reason == "length" and r.output == expected_output([i, i + 1, i + 2], 6)
+    ex.manager.check()
+    assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == 64

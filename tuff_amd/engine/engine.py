@@ -44,6 +44,18 @@ def require_gpu(device="cuda:0") -> torch.device:
     return torch.device(device)
 
 
+class StepFailed(RuntimeError):
+    """A step failed after its kernels had begun to run (a launch that was refused, an error in a part).
+    `.requests`: the ids of the step's requests; what they hold is no longer consistent (a fixed-size state has
+    moved on for some layers, pages that a window had passed are gone) and the engine refuses further steps of
+    them: end() them.  Requests that were not in the step are untouched."""
+
+    def __init__(self, requests, cause):
+        self.requests = list(requests)
+        super().__init__(f"the step failed midway ({type(cause).__name__}: {cause}); its requests "
+                         f"{self.requests} must be ended")
+
+
 class Engine:
     def __init__(self, model, weights: dict, *, dtype, device="cuda:0", page_size: int = 16,
                  max_tokens: int = 8192, max_requests: int = 8, num_pages=None, poison_cache: bool = False,
@@ -64,6 +76,7 @@ class Engine:
         self.manager = CacheManager(self.layout, self.page_size, num_pages, int(max_requests))
         self.storage = CacheStorage(self.manager, self.dtype, self.device, poison=poison_cache)
         self.steps = 0
+        self._broken: set = set()            # requests of a step that failed midway: no further steps, only end()
         # steps of single decoded tokens are recorded into graphs, one per (batch size, table width)
         self.use_graphs = bool(use_graphs) and model.graph_safe()
         self._graphs: dict = {}
@@ -72,6 +85,7 @@ class Engine:
         self._sectioned: dict = {}
         self._sectioned_seen: dict = {}
         self._record_at = self.SECTIONS_RECORD_AT
+        self._calm_replays = 0
         self.section_replays = 0
         self.section_recordings = 0
 
@@ -103,6 +117,7 @@ class Engine:
 
     def end(self, req_id: Hashable) -> None:
         self.manager.release(req_id)
+        self._broken.discard(req_id)
 
     def is_live(self, req_id) -> bool:
         return req_id in self.manager
@@ -133,6 +148,9 @@ class Engine:
         for e in entries:                     # refuse bad input before anything is changed
             if e.req_id not in self.manager:
                 raise ValueError(f"request {e.req_id!r} is not live: call begin() first")
+            if e.req_id in self._broken:
+                raise ValueError(f"request {e.req_id!r} was in a step that failed midway: what it holds is not "
+                                 f"consistent any more, end() it")
             if min(e.tokens) < 0 or max(e.tokens) >= V:
                 raise ValueError(f"request {e.req_id!r}: token id outside [0, {V})")
             if any((not 0 <= w < len(e.tokens)) for w in e.want):
@@ -156,16 +174,20 @@ class Engine:
                 for e in done:
                     self.manager.truncate(e.req_id, self.manager.length(e.req_id) - len(e.tokens))
                 raise
-        self.steps += 1
         try:
-            return self._run(entries, device_tokens)
-        except Exception:
-            # A launch that was refused.  The book-keeping goes back to before the step; paged entries are then
-            # as before (what was written lies beyond every request's length).  A fixed-size state of a layer
-            # that did run has moved on, so the caller should end the step's requests rather than go on with them.
+            out = self._run(entries, device_tokens)
+        except Exception as exc:
+            # A launch that was refused, or an error in a part, after some kernels ran.  The book-keeping goes back
+            # to before the step so that pages and lengths stay sound, but the requests' contents do not: a
+            # fixed-size state of a layer that did run has moved on, and pages that fell out of a window when the
+            # step was accounted are gone (freed, and filled with NaN under poison_cache).  So the step's requests
+            # are refused from now on; all the caller can do with them is end().
             for e in done:
                 self.manager.truncate(e.req_id, self.manager.length(e.req_id) - len(e.tokens))
-            raise
+                self._broken.add(e.req_id)
+            raise StepFailed([e.req_id for e in done], exc) from exc
+        self.steps += 1
+        return out
 
     def _run(self, entries, device_tokens):
         if self.use_graphs and all(len(e.tokens) == 1 for e in entries):
@@ -208,6 +230,8 @@ class Engine:
     SECTIONS_MIN_TOKENS = 2          # every step with a portion may be recorded (a step of 64 tokens: 1.57 ms of launches, 1.22 ms replayed)
     SECTIONS_RECORD_AT = 3           # a number of tokens is recorded when it comes for this time (more, once sizes push each other out)
     MAX_SECTIONED = 4
+    SECTIONS_CALM_REPLAYS = 64       # so many replays without a recording pushed out unused: the threshold halves again
+    SECTIONS_SEEN_KEPT = 256         # sizes whose counts are kept (the least recently seen go first)
 
     def _portion_step(self, ctx, device_tokens=None) -> Optional[torch.Tensor]:
         """A step with prompt portions.  What its kernels' launches depend on outside of the
@@ -218,9 +242,10 @@ class Engine:
         key = self.model.recording_key(ctx)
         rec = self._sectioned.get(key)
         if rec is None:
-            if len(self._sectioned_seen) > 256 and key not in self._sectioned_seen:
-                self._sectioned_seen.clear()                # sizes that came once or twice and never again
-            seen = self._sectioned_seen[key] = self._sectioned_seen.get(key, 0) + 1
+            seen = self._sectioned_seen.pop(key, 0) + 1    # (taken out and put back: the most recently seen is last)
+            self._sectioned_seen[key] = seen
+            while len(self._sectioned_seen) > self.SECTIONS_SEEN_KEPT:
+                self._sectioned_seen.pop(next(iter(self._sectioned_seen)))      # came once or twice, long ago
             if seen < self._record_at:
                 self._place_device_tokens(ctx.tokens, device_tokens)
                 return self.model.forward(ctx, self.storage.views)
@@ -232,6 +257,7 @@ class Engine:
                     # used again.  Recording costs about two eager steps, so sizes now have to come more often.
                     self._record_at = min(2 * self._record_at, 1 << 16)
                     self._sectioned_seen[old_key] = 0
+                    self._calm_replays = 0
             self.section_recordings += 1
             rec = _SectionedStep(ctx.T, self.manager.num_slots, self.device)
             try:
@@ -250,6 +276,13 @@ class Engine:
         merged = rec.refresh(ctx)
         self._place_device_tokens(merged.tokens, device_tokens)
         self.section_replays += 1
+        # A phase of many sizes (ragged tails of prompts) raises the threshold; once the sizes that come are replayed
+        # again and again without one being pushed out unused, it comes down, or a later steady stream of another
+        # size would never be recorded.
+        self._calm_replays += 1
+        if self._calm_replays >= self.SECTIONS_CALM_REPLAYS and self._record_at > self.SECTIONS_RECORD_AT:
+            self._record_at = max(self.SECTIONS_RECORD_AT, self._record_at // 2)
+            self._calm_replays = 0
         return rec.replay(merged)
 
     # --------------------------------------------------------------- recorded decode

@@ -17,7 +17,7 @@ import torch
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .batch import StepEntry
-from .engine import Engine
+from .engine import Engine, StepFailed
 from .scheduler import PLACEHOLDER, Request, Scheduler
 
 
@@ -133,6 +133,12 @@ class Loop:
         pending = self.llm.sampler.launch(logits, [r.sampler for r in sampling]) if sampling else None
         return sampling, pending
 
+    def _end_requests_of(self, failed: StepFailed) -> None:
+        """What the requests of a step that failed midway hold is gone: they end here, with the reason, and give
+        back their pages and slots.  The scheduler's other requests go on if the caller calls again."""
+        for rid in failed.requests:
+            self.sched.abort(rid, reason=f"error: {failed.__cause__}")
+
     def step(self):
         """Runs one step and accounts for it.  Returns (the Scheduled entries whose requests were
         still live, {request id: token drawn}), or None when nothing is left to do."""
@@ -145,20 +151,31 @@ class Loop:
                 if sched.has_unfinished():
                     raise RuntimeError("the scheduler made no progress: no request fits the cache")
                 return None
-            sampling, pending = self._start(batch)
+            try:
+                sampling, pending = self._start(batch)
+            except StepFailed as e:
+                self._end_requests_of(e)
+                raise
         else:
             batch, sampling, pending = self.under_way
             self.under_way = None
         live = sched.advance(batch)
+        failed = None
         if self.llm.run_ahead and not any(sampler.needs_history(r.sampler) for r in sampling):
             nxt = sched.schedule(ahead=True)
             if nxt:
-                self.under_way = (nxt,) + self._start(nxt, (sampling, pending))
-                self.ahead_steps += 1
+                try:
+                    self.under_way = (nxt,) + self._start(nxt, (sampling, pending))
+                    self.ahead_steps += 1
+                except StepFailed as e:
+                    failed = e                             # this step's own tokens are still accounted for below
         sampled = {}
         if pending is not None:
             sampled = {r.id: t for r, t in zip(sampling, pending.tokens())}
         sched.commit(batch, sampled)
+        if failed is not None:
+            self._end_requests_of(failed)                  # after commit(): their last tokens are in place
+            raise failed
         self.steps += 1
         self.tokens += sum(len(s.tokens) for s in live)
         return live, {s.request.id: sampled[s.request.id] for s in live if s.samples}

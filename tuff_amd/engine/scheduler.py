@@ -92,6 +92,7 @@ class Scheduler:
         self.finished: list[Request] = []
         self.num_preemptions = 0
         self._decode_turn = 0                     # where the decoding requests' turns go on (budget < requests)
+        self._turn_pending = 0                    # by how much the step being decided moves the turn on
 
     # ------------------------------------------------------------------- requests
     def add(self, req: Request) -> None:
@@ -124,18 +125,27 @@ class Scheduler:
     def has_unfinished(self) -> bool:
         return bool(self.waiting or self.running)
 
-    def abort(self, req_id) -> None:
+    def abort(self, req_id, reason: str = "aborted") -> None:
+        """Ends a request wherever it is and gives back what it holds.  A token that was drawn and not yet seen
+        (a PLACEHOLDER at the end of its output) is dropped."""
         for r in list(self.running):
             if r.id == req_id:
                 self.running.remove(r)
                 self._end(r.id)
-                self._finish(r, "aborted")
+                self._drop_placeholders(r)
+                self._finish(r, reason)
                 return
         for r in list(self.waiting):
             if r.id == req_id:
                 self.waiting.remove(r)
-                self._finish(r, "aborted")
+                self._drop_placeholders(r)
+                self._finish(r, reason)
                 return
+
+    @staticmethod
+    def _drop_placeholders(req: Request) -> None:
+        while req.output and req.output[-1] == PLACEHOLDER:
+            req.output.pop()
 
     def _finish(self, req: Request, reason: str) -> None:
         req.status, req.finish_reason = FINISHED, reason
@@ -192,8 +202,14 @@ class Scheduler:
         is not admitted again in it."""
         preempted_now: set[int] = set()
         while True:
+            self._turn_pending = 0
             out = self._schedule_once(ahead, preempted_now)
             if out is None or out or not self.running or ahead:
+                if out:
+                    # the turn moves on when a step is really handed out, also one decided ahead (a serving loop
+                    # that always decides ahead would otherwise run the same requests every step); a refused
+                    # ahead call (None) changes nothing
+                    self._decode_turn += self._turn_pending
                 return out
             # running requests and none can take a token: make room
             victim = self.running[-1]
@@ -219,8 +235,7 @@ class Scheduler:
             # the one before stopped
             turn = self._decode_turn % n_decoding
             order = order[turn:n_decoding] + order[:turn] + order[n_decoding:]
-            if not ahead:
-                self._decode_turn += budget
+            self._turn_pending = budget
         for req in order:
             if req not in self.running or budget == 0:       # preempted meanwhile / nothing left
                 continue

@@ -162,10 +162,16 @@ class DecoderModel:
                 block.forward(x, ctx, self._views_of(i, cache_views), run.writes)
         # which rows are wanted is a fact of the step, not of its shape: the head runs outside of what is recorded
         # (a recorder keeps the function and hands back what it returns at each replay)
+        # What the last block left for the final norm is taken here, where the step's kernels are issued (or
+        # recorded: the tensors are then the recording's own, and every replay's head finds them as the eager
+        # step's head does), not inside the function that runs later.
+        pre = None
+        if head_fused and all_rows and hasattr(self.final_norm, "take_announced"):
+            pre = self.final_norm.take_announced(x)
         out: list = []
 
         def head(c):
-            out[:] = [self._head(x, c)]
+            out[:] = [self._head(x, c, pre)]
             return out[0]
 
         ctx.run_eagerly(head)
@@ -197,13 +203,14 @@ class DecoderModel:
                       or all_rows and ctx.n_logits <= ops.EMIT_MAX_ROWS))
         return fused, all_rows
 
-    def _head(self, x, ctx) -> Optional[torch.Tensor]:
-        logits = self._head_product(x, ctx)
+    def _head(self, x, ctx, pre=None) -> Optional[torch.Tensor]:
+        logits = self._head_product(x, ctx, pre)
         if logits is not None and (self.logit_scale != 1.0 or self.logit_softcap is not None):
             ops.scale_cap(logits, self.logit_scale, self.logit_softcap or 0.0)
         return logits
 
-    def _head_product(self, x, ctx) -> Optional[torch.Tensor]:
+    def _head_product(self, x, ctx, pre=None) -> Optional[torch.Tensor]:
+        """pre: (xw, ss), the final norm's operand and row sums as the last block's product left them, or None."""
         if ctx.n_logits == 0:
             return None
         rt = self.rt
@@ -211,9 +218,8 @@ class DecoderModel:
         logits = torch.empty(ctx.n_logits, self.vocab_size, dtype=torch.float32, device=rt.device)
         if head_fused:
             fn = self.final_norm
-            p = fn.pending(x, None if all_rows else ctx.logit_rows)
-            if p.pre is not None:
-                ops.gemm_scaled(p.pre[0], p.pre[1], fn.eps, self.head, logits)
+            if pre is not None and all_rows:
+                ops.gemm_scaled(pre[0], pre[1], fn.eps, self.head, logits)
                 return logits
             if ctx.n_logits <= ops.NORMED_MAX_ROWS and self.hidden_size <= ops.NORMED_MAX_K:
                 ops.gemm_normed(x, fn.weight_f32, fn.eps, self.head, logits, rows=ctx.logit_rows)

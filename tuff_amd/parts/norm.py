@@ -56,12 +56,13 @@ class RMSNorm(Norm):
 
     def pending(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> PendingNorm:
         """The norm of x as a PendingNorm, for consumers that say they accept one."""
-        pre, self._ready = None, getattr(self, "_ready", None)
-        if self._ready is not None:
-            if self._ready[0] is x and rows is None:
-                pre = self._ready[1:]
-            self._ready = None
-        return PendingNorm(self, x, rows, pre)
+        pre = self.take_announced(x)
+        return PendingNorm(self, x, rows, pre if rows is None else None)
+
+    def take_announced(self, x: torch.Tensor):
+        """(xw, ss) if the product that last added into x announced them, else None; either way nothing stays."""
+        ready, self._ready = getattr(self, "_ready", None), None
+        return ready[1:] if ready is not None and ready[0] is x else None
 
     def announce_operand(self, x: torch.Tensor, xw: torch.Tensor, ss: torch.Tensor) -> None:
         """Called by the product that has just added into x and, in the same kernel, written
