@@ -49,10 +49,9 @@ def shape_config(layers: int):
 
 
 def matmul_params(model) -> int:
-    """Elements of all projection matrices of the layers (not embedding, head or norms)."""
-    skip = {model.embedding_decl.name} | ({model.head_decl.name} if model.head_decl else set())
-    return sum(d.shape[0] * d.shape[1] for d in model.weight_decls()
-               if len(d.shape) == 2 and d.name not in skip and d.init == "normal" and d.shape[1] > 16)
+    """Elements of all projection matrices of the layers (what the parts' Linear declare; not embedding,
+    head, norms or conv taps)."""
+    return sum(d.shape[0] * d.shape[1] for d in model.weight_decls() if d.role == "projection")
 
 
 def prefill_flops(cfg, model, T: int, n_logits: int = 1) -> float:

@@ -261,10 +261,55 @@ def test_command_line(gpu, tmp_path):
         p6.stderr
     ts = [float(m.split("(t=")[1].rstrip(")")) for m in marks]
     assert ts == sorted(ts) and all(" s (t=" in m for m in marks)
+    # bfloat16 (the default type), configuration B, whose greedy continuation is not one token repeated: the tokens of
+    # the plain model up to its first near-tie, and teacher-forced on them the logits within the rounding model's noise
+    folder16 = util.model_folder("B", "bfloat16")
+    prompt16 = util.rand_tokens(11, util.TINY_B["vocab_size"], 5)
+    ids16 = ",".join(map(str, prompt16))
+    want16, margins16 = plain_generate("B", prompt16, 12, "bfloat16")
+    p7 = _tuff("--model", folder16, "--prompt-ids", ids16, "--dump-tokens", "-n", "12")
+    assert p7.returncode == 0, p7.stderr
+    got16 = [int(x) for x in p7.stdout.split()]
+    assert len(got16) == 12 and agree_up_to_near_ties(got16, want16, margins16, 2e-2) >= 1
+    ref.write_text("\n".join(map(str, want16)))
+    p8 = _tuff("--model", folder16, "--prompt-ids", ids16, "--teacher-force", str(ref), "--dump-logits", str(out),
+               "--tf-batch", "5", "-n", "12", "--dtype", "bf16")
+    assert p8.returncode in (0, 1), p8.stderr                 # 1: a first choice differs at a near-tie
+    raw = out.read_bytes()
+    n16, V16 = np.frombuffer(raw[8:16], dtype="<u4")
+    assert (n16, V16) == (12, util.TINY_B["vocab_size"])
+    rows16 = torch.from_numpy(np.frombuffer(raw[16:], dtype="<f4").reshape(12, V16).copy())
+    util.assert_close("bfloat16", rows16, util.expected("B", prompt16 + want16[:-1], "bfloat16")[slice(len(prompt16) - 1, None)],
+                      "teacher-forced logits, bfloat16")
     assert _tuff("--model", folder).returncode == 2
     assert _tuff("--model", folder, "--prompt-ids", ids, "-n", "5000").returncode == 2
     assert _tuff("--model", str(tmp_path), "--prompt-ids", ids).returncode == 1
     assert _tuff("--model", folder, "--inspect").returncode == 0
+
+
+def test_gpu_time_by_kernel_class(gpu):
+    """TUFF_TRACE=1: every entry point of the kernel libraries is timed with events and the run ends with a table of
+    calls and GPU time by kernel class (the reference's TUFF_TRACE report, src/cupti_profiler.cu:115-181); the
+    tokens are the same as without."""
+    folder = util.model_folder("E", "bfloat16")
+    ids = ",".join(map(str, util.rand_tokens(20, util.TINY_E["vocab_size"], 3)))
+    plain_run = _tuff("--model", folder, "--prompt-ids", ids, "--dump-tokens", "-n", "6")
+    env = dict(os.environ, TUFF_TRACE="1")
+    p = subprocess.run([sys.executable, os.path.join(util.ROOT, "bin", "tuff"), "--model", folder, "--prompt-ids", ids,
+                        "--dump-tokens", "-n", "6"], capture_output=True, text=True, timeout=300, env=env)
+    assert p.returncode == 0, p.stderr
+    assert p.stdout == plain_run.stdout and "GPU TIME BY KERNEL CLASS" not in plain_run.stderr
+    assert "GPU TIME BY KERNEL CLASS" in p.stderr
+    rows = {}
+    for line in p.stderr.splitlines():
+        cells = [c.strip() for c in line.split("|")]
+        if len(cells) == 7 and cells[0].startswith("tuff_"):
+            rows[cells[0]] = (int(cells[1]), float(cells[2]))
+    # one prompt step and five steps of a single token through 2 attention layers, a head each step
+    assert rows["tuff_attention_decode_fused"][0] == 10 and rows["tuff_attention_prefill"][0] == 2
+    assert rows["tuff_embed_rows"][0] == 6 and all(ms > 0 for _, ms in rows.values())
+    shares = [float(l.split("|")[6].strip().rstrip("%")) for l in p.stderr.splitlines() if l.startswith("tuff_") and l.count("|") == 6]
+    assert abs(sum(shares) - 100) < 1.5
 
 
 def test_command_line_jobs(gpu, tmp_path):

@@ -1330,6 +1330,68 @@ def test_sample_matches_the_plain_sampler(gpu, params):
     assert len(differ) <= 1
 
 
+def _exact_draw(logits_row, params, u):
+    """The reference's sampling order (src/sampler.c:115-230) with every sum in float64: the candidates in (value
+    descending, index ascending) order and the rank of the first whose cumulative probability reaches the draw."""
+    import numpy as np
+    l = logits_row.numpy().astype(np.float32)
+    scaled = (l - l.max()) * (np.float32(1.0) / np.float32(params["temp"]))          # float32, as both samplers form it
+    keep = np.nonzero(scaled >= (np.float32(math.log(params["min_p"])) if 0 < params.get("min_p", 0) < 1 else np.float32(-1e30)))[0]
+    order = keep[np.lexsort((keep, -scaled[keep].astype(np.float64)))]
+    if params.get("top_k", 0) > 0:
+        order = order[:params["top_k"]]
+    mass = np.exp(scaled[order].astype(np.float64))
+    cum = np.cumsum(mass)
+    active = len(order)
+    if 0 < params.get("top_p", 1.0) < 1:
+        active = int(np.searchsorted(cum, np.float64(np.float32(params["top_p"])) * cum[-1], side="left")) + 1
+    rank = int(np.searchsorted(cum[:active], np.float64(np.float32(u)) * cum[active - 1], side="left"))
+    return order, min(rank, active - 1), mass / cum[-1]
+
+
+def test_sample_at_a_border_of_the_cumulative_sums_is_the_exact_answer(gpu):
+    """A vocabulary of 47,098 at temperature 1 with top_p 0.95 and min_p 0.02 (a case that a search over seeds
+    found): the kernel's pick and the plain float32 sampler's lie 32 candidates apart.  The reference's sampler adds
+    its float32 probabilities one after the other (src/sampler.c:185-226), so after 44,000 terms its running sum is
+    off by up to 44,000 roundings and the candidate at which it reaches the draw is uncertain by that much
+    probability; the kernel adds 40-bit fixed-point probabilities exactly.  So: the kernel's pick is the float64
+    answer (to one candidate: its exp is float32), and the plain sampler's pick is as far from it as its rounding
+    explains and no further."""
+    import random
+    from plain.sampler_plain import PlainSampler
+    from tuff_amd.csrc import ops
+    seed, row = 9633, 0
+    rng = random.Random(seed)                                  # the search's own generation, step by step
+    V = rng.choice([rng.randint(1, 40), rng.randint(41, 3000), rng.randint(3001, 70000)])
+    R = rng.randint(1, 12)
+    kind = rng.random()
+    logits = torch.randn(R, V, generator=torch.Generator().manual_seed(seed)) * rng.choice([0.1, 1.0, 3.0, 10.0])
+    if kind < 0.3:
+        logits = (logits * 2).round() / 2
+    elif kind < 0.4:
+        logits[:, ::3] = -1e30
+    params = dict(temp=rng.choice([0.0, 0.3, 0.8, 1.0, 1.7]), top_k=rng.choice([0, 0, 1, 5, 40, 5000]),
+                  top_p=rng.choice([1.0, 1.0, 0.95, 0.5, 0.1]), min_p=rng.choice([0.0, 0.0, 0.02, 0.3]))
+    assert V == 47098 and params == dict(temp=1.0, top_k=0, top_p=0.95, min_p=0.02)
+    plain_s = PlainSampler(seed=seed + 1, **params)
+    probe = PlainSampler(seed=seed + 1, **params)
+    u = float(probe.rng.uniform())
+    want = plain_s.sample(logits[row].numpy())
+    out = torch.empty(1, dtype=torch.int32, device=gpu)
+    f = lambda key, dt: torch.full((1,), params[key], dtype=dt, device=gpu)
+    ops.sample(logits[row:row + 1].to(gpu), out, temps=f("temp", torch.float32), top_ks=f("top_k", torch.int32),
+               top_ps=f("top_p", torch.float32), min_ps=f("min_p", torch.float32),
+               uniforms=torch.tensor([u], dtype=torch.float32, device=gpu))
+    got = int(out[0])
+    order, exact, prob = _exact_draw(logits[row], params, u)
+    rank = {int(t): i for i, t in enumerate(order)}
+    assert abs(rank[got] - exact) <= 1, (rank[got], exact)
+    assert got != want                                          # the case is one where the two samplers differ ...
+    a, b = sorted((rank[got], rank[want]))
+    between = float(prob[a:b + 1].sum())
+    assert between <= len(order) * 2.0 ** -24, (between, len(order))   # ... by no more than sequential float32 sums explain
+
+
 def test_sample_top_k_ties_and_uniform_logits(gpu):
     from tuff_amd.csrc import ops
     V = 500

@@ -32,7 +32,9 @@ def _ids_from(text_or_path: str) -> list[int]:
 def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="tuff", description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter,
                                  epilog="Environment: TUFF_TIMING=1 prints one line per phase (configuration, model load, "
-                                        "prefill, warm-up, decode) with its seconds on standard error.")
+                                        "prefill, warm-up, decode) with its seconds on standard error.  TUFF_TRACE=1 "
+                                        "times every class of kernels with events (no recorded graphs meanwhile) and "
+                                        "prints a table of GPU time by kernel class at the end of the run.")
     ap.add_argument("--model", help="model folder (config.json + model.safetensors)")
     ap.add_argument("--random", metavar="CONFIG_JSON", help="random weights for this config.json instead of --model")
     ap.add_argument("--prompt", "-p", help="prompt text (needs tokenizer.json in the model folder)")
@@ -80,8 +82,11 @@ def _inspect(cfg, model, out=sys.stdout) -> None:
     n = model.num_parameters()
     print(f"parameters: {n} ({2 * n / 2**20:.1f} MiB in bfloat16)", file=out)
     for i, b in enumerate(model.blocks):
-        spec = b.mixer.cache_spec()
-        print(f"  layer {i}: {type(b.mixer).__name__} + {type(b.ffn).__name__ if b.ffn else '-'}  cache: {spec}", file=out)
+        # a block of another arrangement may have neither a mixer nor a feed-forward of these names
+        mixer, ffn = getattr(b, "mixer", None), getattr(b, "ffn", None)
+        inside = " + ".join(type(p).__name__ for p in (mixer, ffn) if p is not None) or type(b).__name__
+        spec = mixer.cache_spec() if hasattr(mixer, "cache_spec") else None
+        print(f"  layer {i}: {inside}  cache: {spec}", file=out)
     print(f"run order: {[r.block for r in model.schedule]}", file=out)
 
 
@@ -288,6 +293,9 @@ def _run(argv: list, loaded: dict) -> int:
         print(f"tuff: prompt ({len(ids)}) + -n ({n_predict}) does not fit -c {ctx}", file=sys.stderr)
         return 2
 
+    from .csrc import ops
+    if ops.TRACE:
+        ops.trace_reset()                                    # the model's loading is not part of the run
     try:
         if args.teacher_force or args.dump_logits:
             rc = _teacher_force(args, eng, ids, n_predict, chunk)
@@ -304,6 +312,9 @@ def _run(argv: list, loaded: dict) -> int:
     except Exception as e:                                   # noqa: BLE001
         print(f"tuff: {type(e).__name__}: {e}", file=sys.stderr)
         return 3
+    finally:
+        if ops.TRACE:
+            ops.trace_report(sys.stderr)
 
 
 def _timed(args, llm, ids, params, tm) -> int:

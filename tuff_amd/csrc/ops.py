@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import math
+import os
 from typing import Optional
 
 import torch
@@ -106,6 +107,75 @@ _SIGNATURES = {
 
 _libs: dict[str, ctypes.CDLL] = {}
 
+# TUFF_TRACE=1: GPU time by kernel class.  Every entry point of the kernel libraries is timed with a pair of
+# events around its launches (an entry point is a class of kernels: the attention of single tokens is its
+# partition kernel and its merge), and trace_report() prints calls, total, mean, least and most per class, in the
+# manner of the reference's TUFF_TRACE report (src/cupti_profiler.cu:115-181, switched on at src/main.c:1787-1789).
+# Events cannot be recorded into a graph, so an engine records no steps while this is on, and the step's time is
+# that of its launches one by one.
+TRACE = os.environ.get("TUFF_TRACE", "")[:1] == "1"
+_trace_open: list = []                   # (class, start event, end event) not yet read
+_trace_stats: dict = {}                  # class -> [calls, total ms, least ms, most ms]
+
+
+def _trace_fold(everything: bool) -> None:
+    """Reads the events that have completed (all of them after a synchronisation) into the statistics."""
+    if everything:
+        torch.cuda.synchronize()
+    keep = []
+    for name, a, b in _trace_open:
+        if not everything and not b.query():
+            keep.append((name, a, b))
+            continue
+        ms = a.elapsed_time(b)
+        st = _trace_stats.setdefault(name, [0, 0.0, float("inf"), 0.0])
+        st[0] += 1
+        st[1] += ms
+        st[2] = min(st[2], ms)
+        st[3] = max(st[3], ms)
+    _trace_open[:] = keep
+
+
+def _traced(name: str, fn):
+    def call(*args):
+        if torch.cuda.is_current_stream_capturing():
+            return fn(*args)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        rc = fn(*args)
+        b.record()
+        _trace_open.append((name, a, b))
+        if len(_trace_open) >= 4096:
+            _trace_fold(False)
+        return rc
+    return call
+
+
+def trace_reset() -> None:
+    _trace_fold(True)
+    _trace_stats.clear()
+
+
+def trace_stats() -> dict:
+    """{kernel class: (calls, total ms, least ms, most ms)} since the last trace_reset()."""
+    _trace_fold(True)
+    return {k: tuple(v) for k, v in _trace_stats.items()}
+
+
+def trace_report(out) -> None:
+    stats = sorted(trace_stats().items(), key=lambda kv: -kv[1][1])
+    total = sum(v[1] for _, v in stats)
+    line = "=" * 104
+    print(f"\n{line}\n{'GPU TIME BY KERNEL CLASS (TUFF_TRACE)':^104}\n{line}", file=out)
+    print(f"Total GPU time in kernel classes: {total:.3f} ms\n", file=out)
+    print(f"{'Kernel class (entry point)':<44} | {'Calls':>7} | {'Total(ms)':>10} | {'Avg(us)':>9} | {'Min(us)':>9} | "
+          f"{'Max(us)':>9} | {'GPU Time%':>9}", file=out)
+    print("-" * 104, file=out)
+    for name, (calls, ms, lo, hi) in stats:
+        print(f"{name:<44} | {calls:>7} | {ms:>10.3f} | {1e3 * ms / calls:>9.2f} | {1e3 * lo:>9.2f} | {1e3 * hi:>9.2f} | "
+              f"{100 * ms / total if total else 0:>8.1f}%", file=out)
+    print(line, file=out)
+
 
 def load(module: str) -> ctypes.CDLL:
     """The loaded library of a kernel module; compiled at first use if it is not built yet."""
@@ -117,6 +187,8 @@ def load(module: str) -> ctypes.CDLL:
             fn = getattr(lib, name)
             fn.argtypes = argtypes
             fn.restype = _c_int
+            if TRACE and argtypes and argtypes[-1] is _c_void_p:        # (the last argument is the stream: it launches)
+                setattr(lib, name, _traced(name, fn))
         _libs[module] = lib
     return lib
 

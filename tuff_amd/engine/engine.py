@@ -78,7 +78,8 @@ class Engine:
         self.steps = 0
         self._broken: set = set()            # requests of a step that failed midway: no further steps, only end()
         # steps of single decoded tokens are recorded into graphs, one per (batch size, table width)
-        self.use_graphs = bool(use_graphs) and model.graph_safe()
+        # (nothing is recorded while the kernel classes are being timed: events cannot go into a graph)
+        self.use_graphs = bool(use_graphs) and model.graph_safe() and not ops.TRACE
         self._graphs: dict = {}
         self.graph_replays = 0
         self.record_portions = self.use_graphs and model.records_portions()

@@ -23,6 +23,7 @@ class WeightDecl:
     init: str = "normal"            # random-weights mode: "normal" N(0, 0.02) | "norm" 1 + N(0, 0.01)
     alt_shapes: tuple = ()          # shapes that are accepted and reshaped to `shape`
     aliases: tuple = ()             # other names the same tensor may have
+    role: str = ""                  # "projection": the matrix of a Linear (every token is multiplied by it)
 
 
 @dataclasses.dataclass(frozen=True)

@@ -42,7 +42,7 @@ class Linear:
         self.bias = None              # bound: float32 [out]
 
     def weight_decls(self) -> list[WeightDecl]:
-        decls = [WeightDecl(n, (o, self.in_features), "normal", aliases=a)
+        decls = [WeightDecl(n, (o, self.in_features), "normal", aliases=a, role="projection")
                  for n, o, a in zip(self.names, self.outs, self.aliases)]
         if self.bias_names is not None:
             decls += [WeightDecl(n, (o,), "normal") for n, o in zip(self.bias_names, self.outs)]

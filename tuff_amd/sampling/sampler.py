@@ -4,6 +4,14 @@ Per request: greedy if temp <= 0 (the penalty is not applied then, as in the ref
 fast path, src/sampler.c:102-113); else repetition penalty -> min-p -> top-k -> top-p -> draw
 with the request's own xorshift128+ generator.  The uniform is drawn on the host, one per
 stochastic row, so a request's stream does not depend on what else is in the batch.
+
+Not the reference's arithmetic at the borders of the cumulative sums: the reference adds its float32
+probabilities one after the other (src/sampler.c:185-226), so its running sum carries up to one rounding a
+term and the candidate at which it reaches top_p, or the draw, is uncertain by that much probability (at a
+vocabulary of 47,000 to 65,000: candidates 20 to 100 places apart, all of them of tiny probability).  The kernel
+adds 40-bit fixed-point probabilities exactly, whatever the order, and picks what float64 sums pick.  The same
+seed and logits can therefore give another token than the reference's sampler where the draw falls that close to
+a border; with small vocabularies or sharp distributions they agree.
 """
 from __future__ import annotations
 
