@@ -266,9 +266,22 @@ SCENARIOS = {
 }
 
 
-def run_scenario(name: str, dtype: str, runs: int = 3) -> dict:
+def scenario_lengths(sc: dict) -> list:
     import math
     import random
+    rng = random.Random(sc["seed"])
+    kind, lo, hi = sc["prompts"]
+    if kind == "uniform":
+        return [rng.randint(lo, hi) for _ in range(sc["requests"])]
+    return [int(math.exp(rng.uniform(math.log(lo), math.log(hi)))) for _ in range(sc["requests"])]
+
+
+def scenario_pages(sc: dict) -> int:
+    return sum(-(-(n + sc["new_tokens"]) // 16) for n in scenario_lengths(sc)) + 64
+
+
+def run_scenario(name: str, dtype: str, runs: int = 3, eng=None) -> dict:
+    """eng: an engine of the scenario's shape and seed with room for it (else one is made)."""
     import torch
     from tuff_amd.engine.engine import Engine
     from tuff_amd.engine.llm import LLM
@@ -276,15 +289,11 @@ def run_scenario(name: str, dtype: str, runs: int = 3) -> dict:
     from tuff_amd.sampling.params import SamplingParams
     sc = SCENARIOS[name]
     cfg = config_from_dict(sc["config"])
-    rng = random.Random(sc["seed"])
-    kind, lo, hi = sc["prompts"]
-    if kind == "uniform":
-        lens = [rng.randint(lo, hi) for _ in range(sc["requests"])]
-    else:
-        lens = [int(math.exp(rng.uniform(math.log(lo), math.log(hi)))) for _ in range(sc["requests"])]
+    lens = scenario_lengths(sc)
     new = sc["new_tokens"]
-    pages = sum(-(-(n + new) // 16) for n in lens) + 64
-    eng = Engine.from_config(cfg, sc["seed"], dtype=dtype, page_size=16, num_pages=pages, max_requests=sc["at_a_time"])
+    if eng is None:
+        eng = Engine.from_config(cfg, sc["seed"], dtype=dtype, page_size=16, num_pages=scenario_pages(sc),
+                                 max_requests=sc["at_a_time"])
     llm = LLM(engine=eng, max_num_seqs=sc["at_a_time"], max_batched_tokens=sc["budget"],
               ctx_size=cfg.max_position_embeddings, ignore_eos=True)
     g = torch.Generator().manual_seed(SEED)
@@ -313,6 +322,72 @@ def run_scenario(name: str, dtype: str, runs: int = 3) -> dict:
                        "steps": st["steps"], "preemptions": st["preemptions"]}}
 
 
+# Other shapes of the architecture, measured after the benchmark's own: decode at batch 8 and 64 at the benchmark's
+# context, the 2,048-token prefill, and the shape's serving scenario on the same engine.
+OTHER_SHAPES = {"2.6b": "lfm2-2.6b", "700m": "lfm2-700m-long"}           # key in `points` -> scenario whose config it is
+FAR_BATCH, FAR_CONTEXT = 64, 32768                                         # attention is nine tenths of what this step reads
+NEAR_CONTEXT = 256                                                         # ... and next to nothing of this one's
+
+
+def describe_shape(cfg, model) -> str:
+    return (f"{cfg.num_hidden_layers} layers (attention at {','.join(str(i) for i in cfg.full_attn_idxs)}), hidden {cfg.hidden_size}, "
+            f"{cfg.num_attention_heads}/{cfg.num_key_value_heads} heads of {cfg.head_dim}, ffn {cfg.ffn_dim}, vocab {cfg.vocab_size}, "
+            f"conv_L_cache {cfg.conv_L_cache}, {model.num_parameters()} parameters")
+
+
+class Measured:
+    """One engine of one shape and the points measured on it."""
+
+    def __init__(self, cfg, seed: int, dtype: str, max_b: int, context: int, pages: int = 0, max_requests: int = 0):
+        from tuff_amd.engine.engine import Engine
+        from tuff_amd.engine.llm import LLM
+        self.cfg, self.dtype, self.max_b, self.context, self.page = cfg, dtype, max_b, context, 16
+        need = max(max_b * (-(-context // self.page)), PREFILL_STREAM * (PREFILL_TOKENS // self.page)) + PREFILL_TOKENS // self.page + 8
+        self.eng = Engine.from_config(cfg, seed, dtype=dtype, page_size=self.page, num_pages=max(need, pages),
+                                      max_requests=max(max_b, PREFILL_STREAM, max_requests) + 1)
+        self.model = self.eng.model
+        self.llm = LLM(engine=self.eng, max_num_seqs=max_b, max_batched_tokens=2048, ctx_size=context, ignore_eos=True)
+
+    def tokens_of_room(self) -> int:
+        return self.eng.manager.groups[0].pool.num_pages * self.page if self.eng.manager.groups else 0
+
+    def decode_point(self, batch: int, steps: int, warmup: int, seed: int, runs: int, context: int = 0) -> dict:
+        from tuff_amd.engine.llm import LLM
+        context = context or self.context
+        llm = self.llm
+        if context != self.context:
+            llm = LLM(engine=self.eng, max_num_seqs=self.max_b, max_batched_tokens=2048, ctx_size=context, ignore_eos=True)
+        secs, ctx_mean = [], 0.0
+        for run in range(runs):
+            s_, ctx_mean = run_decode(llm, self.cfg, batch, context, steps, warmup, seed + 1000 * run)
+            secs.append(s_)
+        rate, spread = mean_spread([batch * steps / s_ for s_ in secs])
+        step_s = sum(secs) / len(secs) / steps
+        gbs = decode_bytes(self.cfg, self.model, self.eng, batch, ctx_mean) / step_s / 1e9
+        return {"tok_s": rate, "spread": spread, "ms": 1e3 * step_s, "GBs": gbs}
+
+    def prefill(self, runs: int, warmup: int) -> dict:
+        flops = prefill_flops(self.cfg, self.model, PREFILL_TOKENS)
+        return prefill_record(run_prefill(self.llm, self.cfg, PREFILL_TOKENS, runs=runs, warmup=warmup), flops, self.dtype)
+
+
+def put(points: dict, key: str, pt: dict, spread: bool = False) -> None:
+    points[key] = round(pt["tok_s"], 1)
+    if spread:
+        points[key + "_spread"] = round(pt["spread"], 1)
+    points[key + "_ms_per_step"] = round(pt["ms"], 4)
+    points[key + "_roofline_frac"] = round(pt["GBs"] / HBM_PEAK_GBS, 4)
+
+
+def guarded(points: dict, key: str, fn) -> None:
+    """A point beside the benchmark must not lose it: what fails is recorded in words."""
+    try:
+        fn()
+    except Exception as e:                                    # noqa: BLE001
+        points[key] = None
+        points[key + "_error"] = f"{type(e).__name__}: {e}"[:200]
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -321,11 +396,13 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=8192)
     ap.add_argument("--no-long-points", dest="long_points", action="store_false",
-                    help="skip decode at batch 8, context 32768 and at batch 1, context 131072")
+                    help="skip the points further out: contexts of 256, 32768 and 131072, the long prompt")
+    ap.add_argument("--no-other-shapes", dest="other_shapes", action="store_false",
+                    help="skip the 2.6B and 700M shapes (decode at batch 8 and 64, prefill, their serving scenarios)")
     ap.add_argument("--layers", type=int, default=SHAPE["num_hidden_layers"],
                     help="fewer layers than the shape has (sizes of a layer stay)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
-    ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    ap.add_argument("--no-points", action="store_true", help="skip everything but the decode step at --batch")
     ap.add_argument("--point-steps", type=int, default=96)
     ap.add_argument("--runs", type=int, default=3, help="runs a point (mean and spread over them)")
     ap.add_argument("--no-probe", dest="probe", action="store_false",
@@ -333,6 +410,9 @@ def main() -> int:
     ap.add_argument("--prefill-warmup", type=int, default=4, help="untimed prefill runs before the timed ones")
     ap.add_argument("--only-prefill", action="store_true",
                     help="measure the 2,048-token prefill alone (for profiling) and print its record")
+    ap.add_argument("--shape", default="1.2b", choices=["1.2b"] + sorted(OTHER_SHAPES),
+                    help="measure another shape of the architecture in the benchmark's place (for profiling; "
+                         "its points only, no other shapes after it)")
     ap.add_argument("--scenario", choices=sorted(SCENARIOS),
                     help="instead of the benchmark: a serving run through the scheduler on another shape")
     args = ap.parse_args()
@@ -348,94 +428,107 @@ def main() -> int:
         return 0
 
     import torch
-    from tuff_amd.engine.engine import Engine
-    from tuff_amd.engine.llm import LLM
+    from tuff_amd.models.registry import config_from_dict
 
-    cfg = shape_config(args.layers)
-    page = 16
+    cfg, seed, shape_name = shape_config(args.layers), SEED, "LFM2.5-1.2B"
+    if args.shape != "1.2b":
+        sc = SCENARIOS[OTHER_SHAPES[args.shape]]
+        cfg, seed, shape_name = config_from_dict(sc["config"]), sc["seed"], OTHER_SHAPES[args.shape].upper().replace("-LONG", "")
+        args.other_shapes = False
     max_b = args.batch if args.no_points else max(args.batch, 64)
-    pages = max(max_b * (-(-args.context // page)), PREFILL_STREAM * (PREFILL_TOKENS // page)) + PREFILL_TOKENS // page + 8
-    eng = Engine.from_config(cfg, SEED, dtype=args.dtype, page_size=page, num_pages=pages,
-                             max_requests=max(max_b, PREFILL_STREAM) + 1)
-    llm = LLM(engine=eng, max_num_seqs=max_b, max_batched_tokens=2048, ctx_size=args.context, ignore_eos=True)
-    model = eng.model
+    far = args.long_points and not args.no_points and args.dtype == "bf16"
+    m = Measured(cfg, seed, args.dtype, max_b, args.context,
+                 pages=(FAR_BATCH * FAR_CONTEXT // 16 + 64) if far else 0)
+    eng, model = m.eng, m.model
 
-    flops = prefill_flops(cfg, model, PREFILL_TOKENS)
     if args.only_prefill:
-        print(json.dumps({"prefill": prefill_record(run_prefill(llm, cfg, PREFILL_TOKENS, runs=args.runs, warmup=args.prefill_warmup), flops, args.dtype)}))
+        print(json.dumps({"prefill": m.prefill(args.runs, args.prefill_warmup)}))
         return 0
 
-    def decode_point(batch: int, steps: int, warmup: int, seed: int, context: int = 0, on=None) -> dict:
-        context = context or args.context
-        secs, ctx_mean = [], 0.0
-        for run in range(args.runs):
-            s_, ctx_mean = run_decode(on or llm, cfg, batch, context, steps, warmup, seed + 1000 * run)
-            secs.append(s_)
-        rates = [batch * steps / s_ for s_ in secs]
-        rate, spread = mean_spread(rates)
-        step_s = sum(secs) / len(secs) / steps
-        gbs = decode_bytes(cfg, model, eng, batch, ctx_mean) / step_s / 1e9
-        return {"tok_s": rate, "spread": spread, "ms": 1e3 * step_s, "GBs": gbs}
-
-    head = decode_point(args.batch, args.steps, args.warmup, SEED)
+    head = m.decode_point(args.batch, args.steps, args.warmup, seed, args.runs)
+    further = []
     out = {
-        "metric": f"decode tok/s at batch {args.batch}, context {args.context} (LFM2.5-1.2B shape)", "value": round(head["tok_s"], 1),
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} ({shape_name} shape)", "value": round(head["tok_s"], 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(head["ms"], 4),
         "runs": args.runs, "spread": round(head["spread"], 1),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
-        "data": "synthetic: seeded random weights (seed 2), uniform random token ids",
+        "data": f"synthetic: seeded random weights (seed {seed}), uniform random token ids",
         "config": {
-            "model": "LFM2.5-1.2B shape (Lfm2ForCausalLM)", "layers": cfg.num_hidden_layers,
-            "layers_of_shape": SHAPE["num_hidden_layers"],
+            "model": f"{shape_name} shape (Lfm2ForCausalLM)", "layers": cfg.num_hidden_layers,
+            "layers_of_shape": SHAPE["num_hidden_layers"] if args.shape == "1.2b" else cfg.num_hidden_layers,
             "attention_layers": ",".join(str(i) for i in cfg.full_attn_idxs), "hidden": cfg.hidden_size,
             "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
             "ffn": cfg.ffn_dim, "vocab": cfg.vocab_size, "conv_L_cache": cfg.conv_L_cache,
             "tied_embeddings": cfg.tie_word_embeddings, "global_batch": args.batch, "seq_len": args.context,
-            "prefill_tokens": PREFILL_TOKENS, "page_size": page, "parameters": model.num_parameters(),
-            "norm_eps": cfg.norm_eps, "rope_theta": cfg.rope_theta,
+            "parameters": model.num_parameters(),
+            "constants": f"norm_eps {cfg.norm_eps}, rope_theta {cfg.rope_theta}, page_size {m.page}, prefill_tokens {PREFILL_TOKENS}",
             "parallelism": "single GPU"},
         "roofline": {"bound": "hbm", "achieved": round(head["GBs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(head["GBs"] / HBM_PEAK_GBS, 4)},
     }
     if not args.no_points:
-        out["prefill"] = prefill_record(run_prefill(llm, cfg, PREFILL_TOKENS, runs=args.runs, warmup=args.prefill_warmup), flops, args.dtype)
+        out["prefill"] = m.prefill(args.runs, args.prefill_warmup)
         points = {}
         for b in (1, 64):
-            pt = decode_point(b, args.point_steps, 8, SEED + b)
-            points[f"decode_b{b}"] = round(pt["tok_s"], 1)
-            points[f"decode_b{b}_spread"] = round(pt["spread"], 1)
-            points[f"decode_b{b}_ms_per_step"] = round(pt["ms"], 4)
+            pt = m.decode_point(b, args.point_steps, 8, SEED + b, args.runs)
+            put(points, f"decode_b{b}", pt, spread=True)
             points[f"decode_b{b}_GBs"] = round(pt["GBs"], 1)
-            points[f"decode_b{b}_roofline_frac"] = round(pt["GBs"] / HBM_PEAK_GBS, 4)
-        if args.long_points and LONG_PROMPT <= max_b * args.context:
-            # a long prompt in portions: the attention over what earlier portions left is most of its work
-            try:
-                dt, spread = mean_spread(run_long_prompt(llm, cfg, LONG_PROMPT, args.runs))
+        if args.long_points:
+            room = m.tokens_of_room()
+
+            def long_prompt():
+                # a long prompt in portions: the attention over what earlier portions left is most of its work
+                dt, spread = mean_spread(run_long_prompt(m.llm, cfg, LONG_PROMPT, args.runs))
                 points[f"prompt_{LONG_PROMPT}_tok_s"] = round(LONG_PROMPT / dt, 1)
                 points[f"prompt_{LONG_PROMPT}_ms"] = round(dt * 1e3, 2)
                 points[f"prompt_{LONG_PROMPT}_spread_ms"] = round(spread * 1e3, 2)
-            except Exception as e:                            # noqa: BLE001 - a point beside the benchmark must not lose it
-                points[f"prompt_{LONG_PROMPT}_tok_s"] = None
-                points[f"prompt_{LONG_PROMPT}_error"] = f"{type(e).__name__}: {e}"[:200]
-        if args.long_points:
-            # the same model further out: the cache of the live requests is then most of what a step reads
-            for b, ctx in LONG_POINTS:
+            if LONG_PROMPT <= room:
+                guarded(points, f"prompt_{LONG_PROMPT}_tok_s", long_prompt)
+                further.append(f"a prompt of {LONG_PROMPT} in portions of {PREFILL_TOKENS}")
+            # the same model nearer and further out: at a context of 256 a step reads weights and next to no cache
+            # (the pure regime of few rows against a whole model), far out the cache is most of what it reads
+            for b, ctx, steps, runs in ([(1, NEAR_CONTEXT, 64, args.runs), (8, NEAR_CONTEXT, 64, args.runs)]
+                                        + [(b, ctx, 32, args.runs) for b, ctx in LONG_POINTS]
+                                        + ([(FAR_BATCH, FAR_CONTEXT, 24, 1)] if far else [])):
                 key = f"decode_b{b}_ctx{ctx}"
-                if b * ctx > max_b * args.context:
-                    continue                                  # the pool was made for max_b requests of --context
-                try:
-                    far = LLM(engine=eng, max_num_seqs=max_b, max_batched_tokens=2048, ctx_size=ctx, ignore_eos=True)
-                    pt = decode_point(b, 32, 4, SEED + ctx, context=ctx, on=far)
-                    points[key] = round(pt["tok_s"], 1)
-                    points[key + "_ms_per_step"] = round(pt["ms"], 4)
-                    points[key + "_roofline_frac"] = round(pt["GBs"] / HBM_PEAK_GBS, 4)
-                except Exception as e:                        # noqa: BLE001 - a point beside the benchmark must not lose it
-                    points[key] = None
-                    points[key + "_error"] = f"{type(e).__name__}: {e}"[:200]
+                if b * ctx > room or b > max_b:
+                    continue                                  # the pool was made for less
+                guarded(points, key, lambda: put(points, key, m.decode_point(b, steps, 4, SEED + ctx + b, runs, context=ctx)))
+                further.append(f"decode b{b} ctx {ctx}" + (" (1 run)" if runs == 1 and args.runs != 1 else ""))
         out["points"] = points
     if args.probe and args.dtype == "bf16":
-        del llm
+        del m.llm
         out["probe"] = probe(eng.device)
+    if args.other_shapes and not args.no_points and args.dtype == "bf16" and args.layers == SHAPE["num_hidden_layers"]:
+        del m, eng, model
+        torch.cuda.empty_cache()
+        for short, scenario in OTHER_SHAPES.items():
+            sc = SCENARIOS[scenario]
+            ocfg = config_from_dict(sc["config"])
+            points = out["points"]
+
+            def shape():
+                o = Measured(ocfg, sc["seed"], args.dtype, 64, args.context, pages=scenario_pages(sc),
+                             max_requests=sc["at_a_time"])
+                out["config"][f"shape_{short}"] = describe_shape(ocfg, o.model) + f", seed {sc['seed']}"
+                for b in (8, 64):
+                    put(points, f"{short}_decode_b{b}", o.decode_point(b, 48, 8, sc["seed"] + b, 2 if b == 8 else 1))
+                pre = o.prefill(2, args.prefill_warmup)
+                points[f"{short}_prefill_tok_s"], points[f"{short}_prefill_ms"], points[f"{short}_prefill_frac"] = \
+                    pre["value"], pre["ms"], pre["frac"]
+                r = run_scenario(scenario, "bfloat16", 2, eng=o.eng)
+                points[f"{short}_scenario_tok_s"], points[f"{short}_scenario_s"] = r["value"], r["seconds"]
+                points[f"{short}_scenario_generated_per_s"] = r["generated_per_s"]
+                del o
+                torch.cuda.empty_cache()
+            guarded(points, f"{short}_decode_b8", shape)
+            c = sc["config"]
+            kind, lo, hi = sc["prompts"]
+            further.append(f"{short} shape: decode b8 (2 runs) and b64 (1 run) ctx {args.context}, prefill {PREFILL_TOKENS} (2 runs), scenario of "
+                           f"{sc['requests']} requests with {kind} prompts of {lo} to {hi} tokens and {sc['new_tokens']} new each, "
+                           f"{sc['budget']} tokens a step (2 runs after one)")
+    if further:
+        out["config"]["further_points"] = "; ".join(further)
     print(json.dumps(out))
     return 0
 
