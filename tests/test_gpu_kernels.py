@@ -135,7 +135,9 @@ def test_gemm_with_the_norm_inside(gpu, M, N, K, use_rows):
                                        # the product that follows is wide with a short K: the tiled kernel reads these row sums
                                        (17, 192, 96, 9216), (40, 2048, 2048, 16384), (64, 1536, 512, 13824), (25, 128, 64, 10242),
                                        # ... and the residual stream itself is that wide
-                                       (20, 9216, 128, 512), (40, 10240, 64, 96)])
+                                       (20, 9216, 128, 512), (40, 10240, 64, 96),
+                                       # 33 to 64 rows of a medium-wide residual stream
+                                       (48, 2304, 512, 3072), (64, 4096, 256, 4096), (33, 2064, 96, 2100)])
 def test_gemm_that_prepares_the_next_norm(gpu, M, d, K1, N2):
     """residual += a @ w1.T leaves bf16(residual * norm weight) and per-tile row sums of squares;
     the next product scales its rows by them: together rmsnorm(residual) @ w2.T."""
