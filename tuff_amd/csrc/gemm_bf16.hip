@@ -641,6 +641,30 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
         }
     }
 
+    // OUT_CONV: likewise the rows of the state and the taps that the convolution reads (slot -> state: two trips to
+    // memory one after the other, which now run beside the product instead of behind it); the first CONV_AHEAD rows of the
+    // state, which is all of them up to a kernel length of CONV_AHEAD + 1, and the last tap.
+    constexpr int CONV_AHEAD = 4;
+    float st_ahead[CONV ? EPI_TILES : 1][CONV_AHEAD], tap_ahead[CONV ? EPI_TILES : 1][CONV_AHEAD + 1];
+    if constexpr (CONV) {
+#pragma unroll
+        for (int i = 0; i < EPI_TILES; ++i) {
+            const int mt = tid / 256 + i * EPI_GROUPS, t = tid % 256, l = t / 4;
+            const int row = mt * 16 + (l / 16) * 4 + t % 4, ch = (int)blockIdx.x * 8 + (l % 16), d = N / 3, Kc = cv.taps;
+#pragma unroll
+            for (int k = 0; k <= CONV_AHEAD; ++k) tap_ahead[i][k] = 0.f;
+#pragma unroll
+            for (int k = 0; k < CONV_AHEAD; ++k) st_ahead[i][k] = 0.f;
+            if (mt < MT && (l % 16) < 8 && row < M && ch < d) {
+                const float* st = cv.state + (long long)cv.state_slot[row] * (Kc - 1) * d;
+#pragma unroll
+                for (int k = 0; k < CONV_AHEAD; ++k)
+                    if (k < Kc - 1) { st_ahead[i][k] = st[(long long)k * d + ch]; tap_ahead[i][k] = cv.tap(ch, k); }
+                tap_ahead[i][CONV_AHEAD] = cv.tap(ch, Kc - 1);
+            }
+        }
+    }
+
     f32x4 acc[MT][TN];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -793,10 +817,11 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_bf16_skinny16_kernel(const voi
                 float sv[CONV_MAX_TAPS], wv[CONV_MAX_TAPS];
 #pragma unroll
                 for (int k = 0; k < CONV_MAX_TAPS; ++k) {
+                    if (k < CONV_AHEAD) { sv[k] = st_ahead[ei][k]; wv[k] = tap_ahead[ei][k]; continue; }   // (zero beyond Kc - 1)
                     sv[k] = k < Kc - 1 ? st[(long long)k * d + ch] : 0.f;
                     wv[k] = k < Kc - 1 ? cv.tap(ch, k) : 0.f;
                 }
-                const float w_last = cv.tap(ch, Kc - 1);
+                const float w_last = tap_ahead[ei][CONV_AHEAD];
                 const float u = bcx[0] * bcx[2];
                 float y = 0.f;
 #pragma unroll
