@@ -596,6 +596,85 @@ def test_layers_of_full_size_bfloat16_against_float32(gpu):
     assert (outs["bfloat16"].argmax(-1) == outs["float32"].argmax(-1))[clear].all()
 
 
+def test_decode_of_64_requests_at_8192_keys_against_float32(gpu):
+    """The benchmark's largest launches, whole: 64 requests with 8,191 tokens each in the cache bring one token.
+    The attention then runs 16,384 workgroups a layer (a wave a partition of 256 keys, the kv head changing fastest
+    in their order, keys through LDS) and the products take 64 rows.  Against the float32 path on the same cache:
+    the bfloat16 engine computes the prompts, its keys, values and conv states are copied (exactly) into a float32
+    engine, and both run the step.  With random weights 8,192 keys weigh about the same, and the attention adds a
+    thirtieth of what the feed-forwards put into the residual stream: a partition more or less would change nothing
+    one could see.  So one value in every partition of every request is made fifty times as large as the others
+    (each is then a third of its request's attention output), and the attention's output projection thirty-two times
+    as large (the attention then adds about what the stream holds)."""
+    import ctypes
+    import random
+    from tuff_amd.cache.storage import PagedKVView
+    from tuff_amd.csrc import ops
+    from tuff_amd.engine.batch import StepEntry
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.models.registry import build_model, config_from_dict
+    from tuff_amd.weights.random_init import random_weights
+    cfg = config_from_dict(util.FULL_SIZE_LAYERS)
+    R, ctx, ps = 64, 8192, 16
+    rng = random.Random(5)
+    kw = dict(page_size=ps, num_pages=R * ctx // ps + 8, max_requests=R)
+    engines = []
+    for dtype in (torch.bfloat16, torch.float32):
+        model = build_model(cfg)
+        weights = random_weights(model.weight_decls(), 7, dtype, gpu)
+        weights["model.layers.1.self_attn.out_proj.weight"] *= 32.0          # (a power of two: exact in either type)
+        engines.append(Engine(model, weights, dtype=dtype, **kw))
+    a, b = engines
+    lib = ops.load("attention_mfma")
+    lib.tuff_attention_stage_k_waves.argtypes, lib.tuff_attention_stage_k_waves.restype = [ctypes.c_int], ctypes.c_int
+    assert R * (ctx // ops.ATTN_PARTITION) * cfg.num_key_value_heads >= lib.tuff_attention_stage_k_waves(-1)
+    last = []
+    for r in range(R):
+        toks = util.rand_tokens(ctx, cfg.vocab_size, 900 + r)
+        a.begin(r)
+        b.begin(r)
+        for i in range(0, ctx - 1, 2048):
+            a.step([StepEntry(r, toks[i:min(i + 2048, ctx - 1)], [])])
+        b.manager.extend(r, ctx - 1)
+        assert a.manager.block_table(r, 0) == b.manager.block_table(r, 0)
+        last.append(toks[-1])
+    loud = []                                          # (page, offset) of one position in every partition of every request
+    for r in range(R):
+        table = a.manager.block_table(r, 0)
+        for part in range(ctx // ops.ATTN_PARTITION):
+            pos = min(part * ops.ATTN_PARTITION + rng.randrange(ops.ATTN_PARTITION), ctx - 2)
+            loud.append((table[pos // ps], pos % ps))
+    pages = torch.tensor([p for p, _ in loud], device=gpu)
+    offs = torch.tensor([o for _, o in loud], device=gpu)
+    for e, va in a.storage.views.items():
+        vb = b.storage.views[e]
+        if isinstance(va, PagedKVView):
+            va.v[pages, :, :, offs] *= 50.0
+            vb.k.copy_(va.k)
+            vb.v.copy_(va.v)
+        else:
+            vb.state.copy_(va.state)
+    entries = [StepEntry(r, [last[r]], [0]) for r in range(R)]
+    got = a.step(entries).float().cpu()
+    states_before = {e: vb.state.clone() for e, vb in b.storage.views.items() if not isinstance(vb, PagedKVView)}
+    want = b.step(entries).float().cpu()
+    assert torch.isfinite(want).all()
+    util.assert_close_bf16(got, want, "64 requests at 8,192 keys", rms=0.02)
+    # what a loud value is worth: without one of them (request 3, its partition 17) the float32 logits of that request
+    # move by far more than the tolerance, so a partition lost or taken twice would show
+    b.manager.truncate(3, ctx - 1)
+    page, off = loud[3 * (ctx // ops.ATTN_PARTITION) + 17]
+    for e, vb in b.storage.views.items():
+        if isinstance(vb, PagedKVView):
+            vb.v[page, :, :, off] /= 50.0
+        else:
+            vb.state.copy_(states_before[e])               # the conv states as they were before the step
+    again = b.step([entries[3]]).float().cpu()
+    other = again
+    spread = float(want[3].double().pow(2).mean().sqrt())
+    assert float((other[0].double() - want[3].double()).pow(2).mean().sqrt()) > 0.05 * spread
+
+
 def test_the_benchmarked_model(gpu):
     """The model bench.py times (16 layers of the 1.2B shape, random weights of its seed), three requests of 200, 64
     and 141 tokens: the float32 engine against the plain implementation in float64, the same bits whole, with the
