@@ -413,11 +413,13 @@ def test_toy_mixer_with_several_cache_entries(gpu):
         registry.unregister_architecture("ToySeveralForCausalLM")
 
 
-def test_toy_mixer_with_keys_narrower_than_values(gpu):
+@pytest.mark.parametrize("value_rows", [False, True])
+def test_toy_mixer_with_keys_narrower_than_values(gpu, value_rows):
     """A mixer whose keys are 8 wide and whose values are the model's width, in one PagedKV entry with
     a window: the pool is laid out by the declaration ([pages, heads, page, 8] and [pages, heads, 24,
-    page]), pages behind the window go back, and the framework's own attention refuses such a cache by
-    its shape.  Whole, token by token and mixed with few pages, against a plain loop."""
+    page], or with value_rows [pages, heads, page, 24]: values a row a position, as a mixer with kernels of
+    its own may want them), pages behind the window go back, and the framework's own attention refuses
+    such a cache by its shape.  Whole, token by token and mixed with few pages, against a plain loop."""
     from tuff_amd.config.base import ModelConfig
     from tuff_amd.csrc import ops
     from tuff_amd.engine.engine import Engine
@@ -439,7 +441,7 @@ def test_toy_mixer_with_keys_narrower_than_values(gpu):
             return [WeightDecl(self.name + ".q", (self.dk, self.d)), WeightDecl(self.name + ".k", (self.dk, self.d))]
 
         def cache_spec(self):
-            return PagedKV(1, self.dk, self.window, value_dim=self.d)
+            return PagedKV(1, self.dk, self.window, value_dim=self.d, value_rows=value_rows)
 
         def bind(self, weights, rt):
             self.rt, self.wq, self.wk = rt, weights[self.name + ".q"].float(), weights[self.name + ".k"].float()
@@ -452,14 +454,18 @@ def test_toy_mixer_with_keys_narrower_than_values(gpu):
             assert write_cache
             slot = g.slot_mapping.long()
             cache.k[slot // ps, 0, slot % ps] = k.to(cache.k.dtype)
-            cache.v[slot // ps, 0, :, slot % ps] = hf.to(cache.v.dtype)
+            if value_rows:
+                cache.v[slot // ps, 0, slot % ps] = hf.to(cache.v.dtype)
+            else:
+                cache.v[slot // ps, 0, :, slot % ps] = hf.to(cache.v.dtype)
             pos, req = ctx.positions.tolist(), ctx.req_of_token.tolist()
             for t in range(ctx.T):
                 lo = max(0, pos[t] - self.window + 1)
                 at = torch.arange(lo, pos[t] + 1, device=h.device)
                 page = g.block_table[req[t]].long()[at // ps]
                 assert int(page.min()) >= 0                        # no page of the window was given back
-                keys, vals = cache.k[page, 0, at % ps].float(), cache.v[page, 0, :, at % ps].float()
+                keys = cache.k[page, 0, at % ps].float()
+                vals = (cache.v[page, 0, at % ps] if value_rows else cache.v[page, 0, :, at % ps]).float()
                 p = torch.softmax(keys @ q[t] / self.dk ** 0.5, 0)
                 residual[t] += p @ vals
 
@@ -478,14 +484,14 @@ def test_toy_mixer_with_keys_narrower_than_values(gpu):
     registry.register_architecture("ToyNarrowKeysForCausalLM", Cfg, build)
     try:
         model = registry.build_model(registry.config_from_dict({"architectures": ["ToyNarrowKeysForCausalLM"], "vocab_size": V}))
-        assert model.cache_specs == {0: PagedKV(1, dk, window, d)}
+        assert model.cache_specs == {0: PagedKV(1, dk, window, d, value_rows)}
         w32 = random_weights(model.weight_decls(), 6, torch.float32, "cpu")
         eng = Engine(model, {k: v.to(gpu) for k, v in w32.items()}, dtype="float32", max_tokens=192, poison_cache=True)
         assert eng.layout.bytes_per_token(4) == 4 * (dk + d)
         reqs = {"a": util.rand_tokens(70, V, 1), "b": util.rand_tokens(45, V, 2), "c": util.rand_tokens(52, V, 3)}
         whole = util.run_plan(eng, util.plan_whole(reqs))
         ps = eng.manager.page_size
-        assert shapes == {"k": (1, ps, dk), "v": (1, d, ps)}
+        assert shapes == {"k": (1, ps, dk), "v": (1, ps, d) if value_rows else (1, d, ps)}
         single = util.run_plan(eng, util.plan_tail(reqs, 100))
         mixed = util.run_plan(eng, util.plan_mixed(reqs, seed=7, decode_tail=6))
         view = eng.storage.views[0]

@@ -2,7 +2,8 @@
 
 Per PagedKV entry: K as [num_pages, kv_heads, page_size, head_dim] and V transposed within the
 page, [num_pages, kv_heads, value_dim, page_size] (the matrix cores read both with the summed
-index contiguous; value_dim is head_dim unless the part declares another), in the compute dtype
+index contiguous; value_dim is head_dim unless the part declares another; a part that declares
+`value_rows` gets [num_pages, kv_heads, page_size, value_dim] instead), in the compute dtype
 (bfloat16 in serving, float32 in the 32-bit path; the reference keeps float32 rows
 [layer][kv_head][pos][hd], src/lfm25_gpu.cu:480-483).  Per FixedState entry: one
 tensor [num_slots, *shape] of the declared type (float32 unless the part says otherwise).  Pages are not cleared when they are handed out again: nothing
@@ -55,7 +56,7 @@ class CacheStorage:
             gi = layout.group_of_entry[e]
             n = manager.groups[gi].pool.num_pages
             shape = (n, spec.num_kv_heads, ps, spec.head_dim)
-            vshape = (n, spec.num_kv_heads, spec.v_dim, ps)
+            vshape = (n, spec.num_kv_heads, ps, spec.v_dim) if spec.value_rows else (n, spec.num_kv_heads, spec.v_dim, ps)
             if poison:
                 # stale reads show up as NaN in the logits
                 k = torch.full(shape, float("nan"), dtype=dtype, device=device)

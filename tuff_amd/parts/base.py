@@ -30,12 +30,16 @@ class WeightDecl:
 class PagedKV:
     """Keys and values that grow by one entry a token, kept in pages.  `window`: only the
     last `window` positions are ever read (None: all).  `value_dim`: the width of a value where
-    it is not the keys' (None: head_dim); the framework's own attention kernels take equal
-    widths only and refuse others by the cache's shape."""
+    it is not the keys' (None: head_dim).  `value_rows`: values lie as keys do, a row a position
+    ([page, kv_head, offset, value_dim]), instead of transposed within the page ([page, kv_head,
+    value_dim, offset], which is what the matrix cores of the framework's own attention kernels
+    read).  Those kernels take equal widths and transposed values only and refuse another cache by
+    its shape; a mixer with kernels of its own declares what suits them."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     value_dim: Optional[int] = None
+    value_rows: bool = False
 
     @property
     def v_dim(self) -> int:
