@@ -104,21 +104,50 @@ def plain_model(name: str, stored: str = "bfloat16"):
 class Expected:
     """What a request's logits should be: `want` from the plain implementation in float64, and `rounded`, the same
     with every activation that an engine holds in bfloat16 between its operations rounded to bfloat16 (the plain
-    implementation's `rnd`): the yardstick for an engine's bfloat16 error.  Rows are chosen from both at once."""
+    implementation's `rnd`): the yardstick for an engine's bfloat16 error.  `rounded` is a list: several
+    realizations of the same roundings (every value scaled by a constant before it is rounded and scaled back after,
+    which moves each value to another place between its two bfloat16 neighbours); the yardstick is their mean.
+    Rows are chosen from all at once."""
 
-    def __init__(self, want: torch.Tensor, rounded: torch.Tensor):
-        self.want, self.rounded = want, rounded
+    def __init__(self, want: torch.Tensor, rounded):
+        self.want = want
+        self.rounded = list(rounded) if isinstance(rounded, (list, tuple)) else [rounded]
         self.shape = want.shape
 
     def __getitem__(self, rows):
-        return Expected(self.want[rows], self.rounded[rows])
+        return Expected(self.want[rows], [r[rows] for r in self.rounded])
+
+    def yardstick(self) -> torch.Tensor:
+        """Per row: the rounding model's error (RMS over the vocabulary relative to the logits' spread), the mean
+        over its realizations."""
+        return torch.stack([row_errors(r, self.want) for r in self.rounded]).mean(0)
+
+
+# One realization of the rounding noise scatters by a fifth of its size over a request of 25 tokens where the
+# hidden size is 32 to 100 (few values are rounded at each place); the mean of three halves that.  Models with a wide
+# residual stream round thousands of values at each place and one realization is steady (and a forward costs more).
+REALIZATION_SCALES = (1.0, 1.3, 0.77)
+SMALL_HIDDEN = 512
+
+
+def rounding(scale: float):
+    from plain.lfm2_plain import to_bfloat16_and_back
+    if scale == 1.0:
+        return to_bfloat16_and_back
+    return lambda t: to_bfloat16_and_back(t * scale) / scale
+
+
+def rounded_logits(cfg: dict, w: dict, tokens) -> list:
+    from plain.lfm2_plain import forward_logits
+    scales = REALIZATION_SCALES if int(cfg["hidden_size"]) <= SMALL_HIDDEN else REALIZATION_SCALES[:1]
+    return [forward_logits(cfg, w, list(tokens), rnd=rounding(c)) for c in scales]
 
 
 @functools.lru_cache(maxsize=256)
-def _plain_logits(name: str, tokens: tuple, stored: str, rounded: bool) -> torch.Tensor:
-    from plain.lfm2_plain import forward_logits, to_bfloat16_and_back
+def _plain_logits(name: str, tokens: tuple, stored: str, rounded: bool):
+    from plain.lfm2_plain import forward_logits
     cfg, w = plain_model(name, stored)
-    return forward_logits(cfg, w, list(tokens), **(dict(rnd=to_bfloat16_and_back) if rounded else {}))
+    return tuple(rounded_logits(cfg, w, tokens)) if rounded else forward_logits(cfg, w, list(tokens))
 
 
 def plain_logits(name: str, tokens, stored: str = "bfloat16") -> torch.Tensor:
@@ -131,8 +160,8 @@ def expected(name: str, tokens, stored: str = "bfloat16") -> Expected:
 
 def expected_of(cfg: dict, w: dict, tokens) -> Expected:
     """The same for a model that is not one of CONFIGS (cfg and float64 tensors as read_model returns them)."""
-    from plain.lfm2_plain import forward_logits, to_bfloat16_and_back
-    return Expected(forward_logits(cfg, w, list(tokens)), forward_logits(cfg, w, list(tokens), rnd=to_bfloat16_and_back))
+    from plain.lfm2_plain import forward_logits
+    return Expected(forward_logits(cfg, w, list(tokens)), rounded_logits(cfg, w, tokens))
 
 
 def rand_tokens(n: int, vocab: int, seed: int) -> list[int]:
@@ -352,7 +381,7 @@ def assert_close_bf16(got: torch.Tensor, want, what: str = "", rms: float = 0.03
     assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
     assert torch.isfinite(got).all(), f"{what}: non-finite logits"
     if isinstance(want, Expected):
-        mine, yard = row_errors(got, want.want), row_errors(want.rounded, want.want)
+        mine, yard = row_errors(got, want.want), want.yardstick()
         ratio = float(mine.mean() / yard.mean())
         assert ratio <= BF16_MEAN_RATIO, (f"{what}: mean relative RMS error {float(mine.mean()):.5f} is {ratio:.2f} times "
                                           f"the rounding model's {float(yard.mean()):.5f} (> {BF16_MEAN_RATIO})")
