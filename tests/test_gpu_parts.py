@@ -622,6 +622,137 @@ def test_a_layer_run_twice_a_shared_cache_and_a_window_group(gpu, dtype):
         registry.unregister_architecture("ToyOrderForCausalLM")
 
 
+# ------------------------------------------- a position encoding that reads more than positions
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_position_encoding_over_two_axes_reads_what_comes_with_the_tokens(gpu, dtype):
+    """A rotary encoding defined here whose angle comes from two numbers a token (a row and a column, as of the
+    patches of an image), not from the token's place in the sequence: half of every head turns with the row, half
+    with the column.  It declares the input it reads (TokenInput), steps bring it in StepEntry.inputs, the step's
+    context hands it on; requests of a scheduler bring it as a function of the place.  Nothing in the framework's
+    files knows of it.  Whole, in portions and mixed against a plain loop; greedy generation through LLM.generate
+    (the generated tokens go on along a row) against the plain loop run again for every token."""
+    from tuff_amd.config.base import ModelConfig
+    from tuff_amd.engine.engine import Engine
+    from tuff_amd.engine.llm import LLM
+    from tuff_amd.models import registry
+    from tuff_amd.models.decoder import DecoderModel
+    from tuff_amd.parts.attention import AttentionMixer
+    from tuff_amd.parts.base import PositionEncoding, TokenInput, WeightDecl
+    from tuff_amd.parts.block import PreNormBlock
+    from tuff_amd.parts.ffn import SwiGLU
+    from tuff_amd.parts.norm import RMSNorm
+    from tuff_amd.sampling.params import SamplingParams
+    from tuff_amd.weights.random_init import random_weights
+    d, H, Hkv, hd, ffn, V, theta, eps, width = 48, 3, 1, 16, 80, 131, 100.0, 1e-5, 7
+
+    def turn(x, pos, half):
+        """x [T, heads, hd] with channels half*hd/2 .. of every head rotated by pos (half-split pairs), the rest as it is."""
+        lo = half * hd // 2
+        out = x.clone()
+        out[..., lo:lo + hd // 2] = plain.rope_neox(x[..., lo:lo + hd // 2], pos, theta)
+        return out
+
+    class GridRotary(PositionEncoding):
+        def token_inputs(self):
+            return [TokenInput("grid", cols=2)]
+
+        def apply_step(self, q, k, ctx):
+            grid = ctx.inputs["grid"].long()
+            for t, heads in ((q, H), (k, Hkv)):
+                x = t.view(t.shape[0], heads, hd)
+                for half in (0, 1):
+                    lo = half * hd // 2
+                    inv = theta ** (-2.0 * torch.arange(hd // 4, device=t.device, dtype=torch.float32) / (hd // 2))
+                    ang = grid[:, half].float()[:, None] * inv
+                    c, s_ = ang.cos()[:, None, :].to(t.dtype), ang.sin()[:, None, :].to(t.dtype)
+                    a, b = x[..., lo:lo + hd // 4].clone(), x[..., lo + hd // 4:lo + hd // 2].clone()
+                    x[..., lo:lo + hd // 4] = a * c - b * s_
+                    x[..., lo + hd // 4:lo + hd // 2] = b * c + a * s_
+
+    @dataclasses.dataclass
+    class GridConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyGridForCausalLM"
+        vocab_size: int
+
+    def build(cfg):
+        def block(i):
+            names = {k: f"l{i}.{k}" for k in ("q", "k", "v", "o", "q_norm", "k_norm")}
+            return PreNormBlock(RMSNorm(d, eps, f"l{i}.n1"),
+                                AttentionMixer(d, H, Hkv, hd, names=names, qk_norm_eps=eps, position=GridRotary()),
+                                RMSNorm(d, eps, f"l{i}.n2"),
+                                SwiGLU(d, ffn, names={"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"}))
+        return DecoderModel(vocab_size=cfg.vocab_size, hidden_size=d, embedding=WeightDecl("emb", (cfg.vocab_size, d)),
+                            blocks=[block(0), block(1)], final_norm=RMSNorm(d, eps, "fn"))
+
+    def grid_of(rid, start, n):
+        """Request rid's tokens lie row by row on a grid `width` wide that starts at row = its number."""
+        first = int(rid[1:])
+        place = torch.arange(start, start + n)
+        return {"grid": torch.stack([first + place // width, place % width], 1).numpy()}
+
+    registry.register_architecture("ToyGridForCausalLM", GridConfig, build)
+    try:
+        cfg = registry.config_from_dict({"architectures": ["ToyGridForCausalLM"], "vocab_size": V})
+        model = registry.build_model(cfg)
+        assert [t.name for t in model.token_inputs()] == ["grid"]
+        stored = torch.float32 if dtype == "float32" else torch.bfloat16
+        weights = random_weights(model.weight_decls(), 6, stored, "cpu", stored_dtype=stored)
+        w = {k: v.double() for k, v in weights.items()}
+
+        def logits_of(rid, toks):
+            T = len(toks)
+            g = torch.from_numpy(grid_of(rid, 0, T)["grid"])
+            x = w["emb"][toks]
+            for i in range(2):
+                h = plain.rms_norm(x, w[f"l{i}.n1"], eps)
+                q = plain.rms_norm((h @ w[f"l{i}.q"].T).reshape(T, H, hd), w[f"l{i}.q_norm"], eps)
+                k = plain.rms_norm((h @ w[f"l{i}.k"].T).reshape(T, Hkv, hd), w[f"l{i}.k_norm"], eps)
+                q, k = turn(turn(q, g[:, 0], 0), g[:, 1], 1), turn(turn(k, g[:, 0], 0), g[:, 1], 1)
+                v = (h @ w[f"l{i}.v"].T).reshape(T, Hkv, hd)
+                k, v = k.repeat_interleave(H // Hkv, 1), v.repeat_interleave(H // Hkv, 1)
+                s_ = torch.einsum("thd,shd->hts", q, k) / math.sqrt(hd)
+                s_ = s_.masked_fill(~torch.ones(T, T, dtype=torch.bool).tril(), float("-inf"))
+                x = x + torch.einsum("hts,shd->thd", torch.softmax(s_, -1), v).reshape(T, H * hd) @ w[f"l{i}.o"].T
+                x = x + plain.swiglu(plain.rms_norm(x, w[f"l{i}.n2"], eps), w[f"l{i}.g"], w[f"l{i}.u"], w[f"l{i}.d"])
+            return plain.rms_norm(x, w["fn"], eps) @ w["emb"].T
+
+        reqs = {f"r{i}": util.rand_tokens(n, V, 50 + i) for i, n in enumerate([60, 33, 47, 20])}
+        plan = util.plan_mixed(reqs, seed=5, decode_tail=10)
+        eng = Engine(model, {k: v.to(gpu) for k, v in weights.items()}, dtype=dtype, page_size=16,
+                     max_tokens=util.live_tokens_peak(plan))
+        runs = [util.run_plan(eng, p, grid_of) for p in (util.plan_whole(reqs), plan, util.plan_chunks(reqs))]
+        eng.manager.check()
+        for rid, toks in reqs.items():
+            want = logits_of(rid, toks)
+            for got in runs:
+                util.assert_close(dtype, got[rid], want, rid)
+        # the coordinates matter: the same tokens along one long row give other logits
+        flat = util.run_plan(eng, util.plan_whole({"r0": reqs["r0"]}),
+                             lambda rid, start, n: {"grid": [[0, c] for c in range(start, start + n)]})["r0"]
+        assert (flat.double() - logits_of("r0", reqs["r0"])).abs().max() > 1e-2
+        # a step that leaves them out is refused by name, and the engine goes on
+        eng.begin("x")
+        with pytest.raises(ValueError, match="reads the input 'grid'"):
+            eng.step([("x", [1, 2, 3], [2])])
+        eng.end("x")
+        if dtype == "float32":
+            # through the scheduler: prompts in portions of 16 beside decoding requests, the inputs as a function of the place
+            llm = LLM(engine=eng, max_num_seqs=3, max_batched_tokens=16, ctx_size=96)
+            prompts = {f"r{i}": util.rand_tokens(n, V, 70 + i) for i, n in enumerate([21, 9, 30])}
+            gens = llm.generate(list(prompts.values()), SamplingParams(temp=0.0, max_new_tokens=6),
+                                inputs=[lambda start, n, rid=rid: grid_of(rid, start, n) for rid in prompts])
+            for (rid, prompt), gen in zip(prompts.items(), gens):
+                ids = list(prompt)
+                for tok in gen.token_ids:
+                    row = logits_of(rid, ids)[-1]
+                    top = torch.topk(row, 2).values
+                    if float(top[0] - top[1]) > 1e-3:
+                        assert tok == int(row.argmax()), rid
+                    ids.append(tok)
+    finally:
+        registry.unregister_architecture("ToyGridForCausalLM")
+
+
 # --------------------------------------------------------------- a toy routed feed-forward
 def test_toy_feed_forward_with_routing_beside_the_frameworks_parts(gpu):
     """A feed-forward defined here: a float32 router picks one of three small SwiGLU experts per

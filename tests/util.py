@@ -247,9 +247,11 @@ def live_tokens_peak(plan) -> int:
 
 
 # ---------------------------------------------------------------------------- running
-def run_plan(engine, plan) -> dict:
+def run_plan(engine, plan, inputs_of=None) -> dict:
     """Runs a plan on an Engine in this process.  Returns {req id: float32 [n_tokens, vocab]}
-    with the logits of every wanted place (NaN rows where nothing was wanted)."""
+    with the logits of every wanted place (NaN rows where nothing was wanted).
+    inputs_of(req id, start, n): what comes with the request's tokens start .. start + n - 1 beside their
+    ids (StepEntry.inputs), for models whose parts read such."""
     from tuff_amd.engine.batch import StepEntry
     fed: dict = {}
     rows: dict = {}
@@ -260,7 +262,8 @@ def run_plan(engine, plan) -> dict:
                 engine.begin(e["id"])
                 fed[e["id"]] = 0
                 rows[e["id"]] = {}
-            entries.append(StepEntry(e["id"], e["tokens"], e["want"]))
+            more = inputs_of(e["id"], fed[e["id"]], len(e["tokens"])) if inputs_of is not None else None
+            entries.append(StepEntry(e["id"], e["tokens"], e["want"], more))
         logits = engine.step(entries)
         if logits is not None:
             logits = logits.float().cpu()

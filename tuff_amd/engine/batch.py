@@ -7,7 +7,7 @@ buffer alone was refreshed.
 from __future__ import annotations
 
 import dataclasses
-from typing import Hashable, Optional, Sequence
+from typing import Hashable, Mapping, Optional, Sequence
 
 import numpy as np
 import torch
@@ -19,6 +19,7 @@ class StepEntry:
     req_id: Hashable
     tokens: Sequence[int]
     want: Sequence[int] = ()
+    inputs: Optional[Mapping[str, Sequence]] = None    # name -> integers [n tokens] or [n tokens, cols], for what the model's parts declare (parts.base.TokenInput)
 
 
 @dataclasses.dataclass
@@ -47,6 +48,7 @@ class StepContext:
     max_ctx_len: int = 1           # an upper bound of every position + 1 of the step
     host: dict = dataclasses.field(default_factory=dict)     # 'q_len', 'ctx_len' (numpy) and what parts cache
     recorder: object = None        # set while a step is recorded in sections
+    inputs: dict = dataclasses.field(default_factory=dict)   # name -> int32 [T, cols]: what parts declared as TokenInput
 
     def run_eagerly(self, fn) -> None:
         """fn(ctx) now; where the step is being recorded in sections, fn is kept instead and runs at
@@ -72,15 +74,70 @@ class PackedStep:
     q_len: np.ndarray
     ctx_len: np.ndarray
     logit_rows_identity: bool = False     # logits are wanted of every token of the step, in order
+    token_inputs: tuple = ()              # the TokenInput declarations whose values lie behind the last piece, in this order
 
     def shape_key(self):
         return (self.T, self.R, self.n_logits, self.n_groups, self.max_blocks, self.logit_rows_identity)
 
 
+def merge_token_inputs(decls) -> tuple:
+    """The declarations of all parts of a model as one tuple, a name once; two parts that name the same input
+    must mean the same."""
+    out: dict = {}
+    for d in decls:
+        if d.name in out and out[d.name] != d:
+            raise ValueError(f"two parts declare the token input '{d.name}' differently: {out[d.name]} and {d}")
+        if d.cols < 1:
+            raise ValueError(f"token input '{d.name}': {d.cols} columns")
+        out[d.name] = d
+    return tuple(out.values())
+
+
+def check_token_inputs(entries, token_inputs) -> None:
+    """Raises ValueError, by request and name, where an entry's inputs are not what the model's parts declared:
+    one that is missing and has no default, a wrong shape or type, one that no part reads."""
+    if not token_inputs and not any(e.inputs for e in entries):
+        return
+    for e in entries:
+        n = len(e.tokens)
+        for d in token_inputs:
+            given = None if e.inputs is None else e.inputs.get(d.name)
+            if given is None:
+                if d.default is None:
+                    raise ValueError(f"request {e.req_id!r}: the model reads the input '{d.name}' of every token, and this "
+                                     f"entry brings none")
+                continue
+            a = np.asarray(given)
+            if a.dtype.kind not in "iu" or a.shape not in ((n, d.cols),) + (((n,),) if d.cols == 1 else ()):
+                raise ValueError(f"request {e.req_id!r}: input '{d.name}' must be integers of shape [{n}, {d.cols}], "
+                                 f"got {a.dtype} {list(a.shape)}")
+        for name in (e.inputs or ()):
+            if all(name != d.name for d in token_inputs):
+                raise ValueError(f"request {e.req_id!r}: no part of the model reads an input '{name}'")
+
+
+def _fill_token_inputs(buf, offs, first, token_inputs, entries, manager) -> None:
+    for i, d in enumerate(token_inputs):
+        dst = buf[offs[first + i]:offs[first + i + 1]].reshape(-1, d.cols)
+        t = 0
+        for e in entries:
+            n = len(e.tokens)
+            given = None if e.inputs is None else e.inputs.get(d.name)
+            if given is not None:
+                dst[t:t + n] = np.asarray(given).reshape(n, d.cols)
+            elif isinstance(d.default, str) and d.default == "position":
+                total = manager.length(e.req_id)
+                dst[t:t + n] = np.arange(total - n, total)[:, None]
+            else:
+                dst[t:t + n] = int(d.default)
+            t += n
+
+
 def pack_step(entries: Sequence[StepEntry], manager, vocab_size: int,
-              max_blocks: Optional[int] = None) -> PackedStep:
+              max_blocks: Optional[int] = None, token_inputs: tuple = ()) -> PackedStep:
     """`manager` has already been extended by every entry's tokens.  max_blocks: width of the
-    block tables (default: the longest table of the step)."""
+    block tables (default: the longest table of the step).  token_inputs: the model's TokenInput
+    declarations; their values go behind everything else, [T, cols] each."""
     R = len(entries)
     T = sum(len(e.tokens) for e in entries)
     n_groups = len(manager.groups)
@@ -94,7 +151,7 @@ def pack_step(entries: Sequence[StepEntry], manager, vocab_size: int,
     ps = manager.page_size
     # [tokens | positions | req_of_token | q_start | q_len | ctx_len | slot | logit_rows |
     #  per group: slot_mapping, block_table]
-    sizes = [T, T, T, R, R, R, R, n_logits] + [T, R * max_blocks] * n_groups + [4 * R]
+    sizes = [T, T, T, R, R, R, R, n_logits] + [T, R * max_blocks] * n_groups + [4 * R] + [T * d.cols for d in token_inputs]
     offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
     buf = np.zeros(int(offs[-1]), dtype=np.int32)
     tokens, positions, req_of = (buf[offs[i]:offs[i + 1]] for i in range(3))
@@ -146,8 +203,10 @@ def pack_step(entries: Sequence[StepEntry], manager, vocab_size: int,
         t += n
         max_q, max_ctx = max(max_q, n), max(max_ctx, total)
     identity = n_logits == T and bool((rows == np.arange(T)).all())
+    check_token_inputs(entries, token_inputs)
+    _fill_token_inputs(buf, offs, 9 + 2 * n_groups, token_inputs, entries, manager)
     return PackedStep(buf, offs, T, R, n_logits, n_groups, max_blocks, max_q, max_ctx, q_len.copy(), ctx_len.copy(),
-                      identity)
+                      identity, tuple(token_inputs))
 
 
 def context_on(dev: torch.Tensor, p: PackedStep, max_ctx_len: Optional[int] = None) -> StepContext:
@@ -162,11 +221,12 @@ def context_on(dev: torch.Tensor, p: PackedStep, max_ctx_len: Optional[int] = No
                        max_ctx_len=max_ctx_len if max_ctx_len is not None else p.max_ctx_len,
                        host={"q_len": p.q_len, "ctx_len": p.ctx_len, "logit_rows_identity": p.logit_rows_identity,
                              "packed": {name: p.buf[int(offs[i]):int(offs[i + 1])] for i, name in
-                                        ((0, "tokens"), (2, "req_of_token"), (3, "q_start"), (4, "q_len"), (6, "state_slot"))}})
+                                        ((0, "tokens"), (2, "req_of_token"), (3, "q_start"), (4, "q_len"), (6, "state_slot"))}},
+                       inputs={d.name: sl(9 + 2 * p.n_groups + i).view(p.T, d.cols) for i, d in enumerate(p.token_inputs)})
 
 
-def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int) -> StepContext:
-    p = pack_step(entries, manager, vocab_size)
+def build_context(entries: Sequence[StepEntry], manager, device, vocab_size: int, token_inputs: tuple = ()) -> StepContext:
+    p = pack_step(entries, manager, vocab_size, token_inputs=token_inputs)
     host = torch.from_numpy(p.buf)
     dev = host.pin_memory().to(device, non_blocking=True) if p.buf.size else host.to(device)
     return context_on(dev, p)

@@ -21,7 +21,7 @@ from ..models.registry import build_model, load_config
 from ..parts.base import Runtime
 from ..weights.loader import load_weights
 from ..weights.random_init import random_weights
-from .batch import StepContext, StepEntry, build_context, context_on, pack_step
+from .batch import StepContext, StepEntry, build_context, check_token_inputs, context_on, pack_step
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
            "fp32": torch.float32, "f32": torch.float32}
@@ -69,6 +69,8 @@ class Engine:
         for m in model.kernel_modules() + (["gemm_f32"] if self.dtype == torch.float32 else ["gemm_bf16"]):
             ops.load(m)                      # compile or load now, not in the middle of a step
         model.bind(weights, self.rt)
+        # what the parts read of a step's tokens beside ids and positions (StepEntry.inputs brings it)
+        self.token_inputs = tuple(model.token_inputs()) if hasattr(model, "token_inputs") else ()
         self.layout = CacheLayout.from_specs(model.cache_specs)
         self.page_size = int(page_size)
         if num_pages is None:
@@ -156,6 +158,7 @@ class Engine:
                 raise ValueError(f"request {e.req_id!r}: token id outside [0, {V})")
             if any((not 0 <= w < len(e.tokens)) for w in e.want):
                 raise ValueError(f"request {e.req_id!r}: a wanted place is outside its {len(e.tokens)} tokens")
+        check_token_inputs(entries, self.token_inputs)
         done = []
         try:
             for e in entries:
@@ -193,7 +196,7 @@ class Engine:
     def _run(self, entries, device_tokens):
         if self.use_graphs and all(len(e.tokens) == 1 for e in entries):
             return self._decode_step(entries, device_tokens)
-        ctx = build_context(entries, self.manager, self.device, self.model.vocab_size)
+        ctx = build_context(entries, self.manager, self.device, self.model.vocab_size, self.token_inputs)
         # Recorded in sections: steps with portions (a step of single tokens takes other kernels), keyed by
         # everything their launches depend on outside of the sections that run eagerly.
         if (self.record_portions and ctx.T >= self.SECTIONS_MIN_TOKENS and ctx.max_q_len > 1
@@ -298,7 +301,7 @@ class Engine:
         longest = max([len(self.manager.block_table(e.req_id, g)) for e in entries
                        for g in range(len(self.manager.groups))] + [1])
         width = -(-longest // self.GRAPH_TABLE_BUCKET) * self.GRAPH_TABLE_BUCKET
-        p = pack_step(entries, self.manager, self.model.vocab_size, max_blocks=width)
+        p = pack_step(entries, self.manager, self.model.vocab_size, max_blocks=width, token_inputs=self.token_inputs)
         key = p.shape_key()
         g = self._graphs.get(key)
         if g is None:

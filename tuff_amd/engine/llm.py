@@ -77,17 +77,23 @@ class LLM:
                 on_step(*done)
         self.last_stats = loop.stats()
 
-    def generate(self, prompts: Sequence[Sequence[int]], params=None) -> list[Generation]:
-        """prompts: token id lists.  params: one SamplingParams for all, or one per prompt."""
+    def generate(self, prompts: Sequence[Sequence[int]], params=None, inputs=None) -> list[Generation]:
+        """prompts: token id lists.  params: one SamplingParams for all, or one per prompt.  inputs: for a
+        model whose parts read more of a token than its id and position, one function a prompt (or None),
+        inputs[i](start, n) -> {name: integers [n] or [n, cols]} for the tokens at places start .. start + n - 1
+        of prompt i and what is generated after it (scheduler.Request.inputs)."""
         if params is None:
             params = SamplingParams()
         plist = [params] * len(prompts) if isinstance(params, SamplingParams) else list(params)
         if len(plist) != len(prompts):
             raise ValueError("one SamplingParams per prompt, or one for all")
+        ilist = [None] * len(prompts) if inputs is None else list(inputs)
+        if len(ilist) != len(prompts):
+            raise ValueError("one inputs function per prompt (or None)")
         sched = self.new_scheduler()
         reqs = []
-        for prompt, p in zip(prompts, plist):
-            r = Request(next(self._ids), [int(t) for t in prompt], dataclasses.replace(p))
+        for prompt, p, more in zip(prompts, plist, ilist):
+            r = Request(next(self._ids), [int(t) for t in prompt], dataclasses.replace(p), inputs=more)
             reqs.append(r)
             sched.add(r)
         self.run(sched)
@@ -121,7 +127,8 @@ class Loop:
                 places.append(at)
                 sources.append(row[id(s.request)])
                 toks = [0]
-            entries.append(StepEntry(s.request.id, toks, [len(toks) - 1] if s.samples else []))
+            more = s.request.inputs(s.start, len(toks)) if s.request.inputs is not None else None
+            entries.append(StepEntry(s.request.id, toks, [len(toks) - 1] if s.samples else [], more))
             at += len(toks)
         device_tokens = None
         if places:

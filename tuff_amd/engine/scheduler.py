@@ -27,7 +27,7 @@ from __future__ import annotations
 
 import collections
 import dataclasses
-from typing import Hashable, Optional
+from typing import Callable, Hashable, Optional
 
 from ..cache.manager import CacheManager
 from ..sampling.params import SamplerState, SamplingParams
@@ -47,6 +47,10 @@ class Request:
     finish_reason: Optional[str] = None
     preemptions: int = 0
     sampler: Optional[SamplerState] = None
+    # inputs(start, n) -> {name: integers [n] or [n, cols]} for the tokens at places start .. start + n - 1 of
+    # prompt + output, where the model's parts read more of a token than its id and position (StepEntry.inputs);
+    # a function of the place, so that it also answers for tokens that are not drawn yet and after a preemption
+    inputs: Optional[Callable] = None
 
     def tokens(self) -> list:
         return self.prompt + self.output

@@ -108,6 +108,11 @@ class DecoderModel:
         mods += self.final_norm.kernel_modules()
         return sorted(set(mods))
 
+    def token_inputs(self) -> tuple:
+        """What the parts read of a step's tokens beside ids and positions (parts.base.TokenInput), a name once."""
+        from ..engine.batch import merge_token_inputs
+        return merge_token_inputs([t for b in self.blocks for t in b.token_inputs()])
+
     def graph_safe(self) -> bool:
         return all(b.graph_safe for b in self.blocks) and self.final_norm.graph_safe
 

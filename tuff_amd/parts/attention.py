@@ -70,6 +70,9 @@ class AttentionMixer(Mixer):
             mods += self.position.kernel_modules()
         return mods
 
+    def token_inputs(self):
+        return self.position.token_inputs() if self.position is not None else []
+
     def cache_spec(self):
         return PagedKV(self.Hkv, self.hd, self.window)
 
@@ -124,7 +127,7 @@ class AttentionMixer(Mixer):
                              **norm, **rot, **wr)
             else:
                 ops.qkv_post(qkv, q, H=H, Hkv=Hkv, hd=hd, positions=ctx.positions, k_out=k, **norm)
-                self.position.apply(q, k, ctx.positions)
+                self.position.apply_step(q, k, ctx)
                 if write_cache:
                     v = qkv[:, (H + Hkv) * hd:].contiguous()
                     ops.kv_write(k, v, cache.k, cache.v, g.slot_mapping, Hkv=Hkv, hd=hd, page_size=cache.page_size)

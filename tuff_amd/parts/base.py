@@ -60,6 +60,18 @@ class FixedState:
         return n
 
 
+@dataclasses.dataclass(frozen=True)
+class TokenInput:
+    """Integers that come with every token of a step beside its id: `cols` of them a token (the row and the
+    column of an image patch, a segment number).  A part that reads them declares them (Part.token_inputs); the
+    caller brings them in StepEntry.inputs[name], and a step's context holds them as ctx.inputs[name], int32
+    [T, cols].  `default`: what a token gets whose entry brings none ("position": its position in the request,
+    in every column; an int: that value; None: the entry must bring them)."""
+    name: str
+    cols: int = 1
+    default: object = None
+
+
 def cache_specs_of(mixer) -> tuple:
     """A mixer's cache declarations as a tuple (empty: it keeps nothing), and whether forward()
     is handed a tuple of views (True) or one view / None (False)."""
@@ -93,6 +105,10 @@ class Part:
 
     def kernel_modules(self) -> list[str]:
         """Kernel libraries (names of tuff_amd.csrc.build.MODULES) this part launches."""
+        return []
+
+    def token_inputs(self) -> list:
+        """TokenInput declarations: what this part reads of a step's tokens beside ids and positions."""
         return []
 
     #: True if forward() only launches kernels on the current stream and reads nothing back to
@@ -131,7 +147,9 @@ class PositionEncoding(Part):
 
     Either `rotary_tables()` returns (inv_freq float32 [rotary_dim/2], rotary_dim, interleaved)
     and the mixer applies it inside its fused kernel, or it returns None and the mixer calls
-    `apply(q [T, H*hd], k [T, Hkv*hd], positions int32 [T])`, which rewrites both in place.
+    `apply_step(q [T, H*hd], k [T, Hkv*hd], ctx)`, which rewrites both in place; that is
+    `apply(q, k, ctx.positions)` unless the encoding reads more of the step than positions (what it
+    declares in token_inputs(), from ctx.inputs).
     """
 
     def rotary_tables(self):
@@ -139,6 +157,9 @@ class PositionEncoding(Part):
 
     def apply(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor) -> None:
         raise NotImplementedError
+
+    def apply_step(self, q: torch.Tensor, k: torch.Tensor, ctx) -> None:
+        self.apply(q, k, ctx.positions)
 
 
 class Mixer(Part):

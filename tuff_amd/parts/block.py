@@ -36,6 +36,9 @@ class PreNormBlock(Block):
     def kernel_modules(self):
         return [m for p in self._parts() for m in p.kernel_modules()]
 
+    def token_inputs(self):
+        return [t for p in self._parts() for t in p.token_inputs()]
+
     def bind(self, weights, rt: Runtime):
         self.rt = rt
         for p in self._parts():
