@@ -1255,6 +1255,13 @@ TiledPlan plan_tiled(int M, int N, int K) {
         if (ceil_div(wide, 256) * 192 < ceil_div(large, 256) * 256) t.shape = 4;
         return t;
     }
+    // A little more than one round of pairs of 128 x 128 blocks (512 of them side by side), where blocks of 256 x 256
+    // would be too few for the CUs: the blocks beyond the round run a second one almost alone.  Blocks of 256 x 192
+    // in one round instead (4608 columns and 2048 rows, K = 1536: 37.1 us instead of 43.8; 256 x 256: 45.7).
+    if (t.shape == 1 && small > 512 && K % TBK == 0) {
+        const long long wide = (long long)ceil_div(N, 192) * ceil_div(M, 256);
+        if (wide <= 256) { t.shape = 4; return t; }
+    }
     // few blocks and a short K: blocks of 64 x 64 give enough workgroups without slices of K, whose partial
     // tiles cost a second kernel and as much traffic as the product's own (K = 1536 .. 2048, 96 to 512
     // rows: 9 to 14 us instead of 11 to 19); beyond 48 steps the slices win
