@@ -611,3 +611,44 @@ def test_the_run_loop_ends_the_requests_of_a_step_that_failed_midway(fail_at_cal
             assert r.finish_reason == "length" and r.output == expected_output([i, i + 1, i + 2], 6)
     ex.manager.check()
     assert ex.manager.live() == [] and ex.manager.groups[0].pool.num_free == 64
+
+
+@pytest.mark.parametrize("run_ahead", [True, False])
+@pytest.mark.parametrize("num_pages", [64, 9])
+def test_the_run_loop_brings_what_comes_with_the_tokens_for_the_places_it_feeds(run_ahead, num_pages):
+    """Requests whose tokens come with more than their ids (Request.inputs, a function of the place): every entry
+    of every step holds the inputs of exactly the places it feeds, for prompt portions, for tokens that are not
+    drawn yet when the step is decided, and for the tokens fed again after a preemption (the small pool)."""
+    import types
+    from tuff_amd.engine.llm import Loop
+    ex = AheadExecutor(num_pages=num_pages, page_size=4)
+    seen = []
+
+    class Engine(_FakeEngine):
+        def step(self, entries, device_tokens=None):
+            for e in entries:
+                at = self.ex.manager.length(e.req_id)
+                assert e.inputs is not None and list(e.inputs["place"]) == [[at + i, 100 * int(e.req_id)] for i in range(len(e.tokens))]
+                seen.append((e.req_id, at, len(e.tokens)))
+            return super().step(entries, device_tokens)
+
+    sched = make(ex, max_batched_tokens=5, max_num_seqs=3)
+    reqs = [Request(k, list(range(10 * k, 10 * k + n)), SamplingParams(max_new_tokens=new),
+                    inputs=lambda start, n, k=k: {"place": [[start + i, 100 * k] for i in range(n)]})
+            for k, (n, new) in enumerate([(7, 9), (3, 12), (11, 4), (2, 8)])]
+    for r in reqs:
+        sched.add(r)
+    llm = types.SimpleNamespace(engine=Engine(ex, fail_at_call=-1), sampler=_FakeSampler(), run_ahead=run_ahead)
+    loop = Loop(llm, sched)
+    for _ in range(500):
+        if loop.step() is None:
+            break
+    assert not sched.has_unfinished()
+    for k, r in enumerate(reqs):
+        assert r.finish_reason == "length" and r.output == expected_output(r.prompt, r.params.max_new_tokens)
+    if num_pages == 9:
+        assert sum(r.preemptions for r in reqs) >= 1
+        assert any(at == 0 and rid == r.id for r in reqs if r.preemptions for rid, at, n in seen[1:])
+    assert any(n > 1 for _, _, n in seen) and any(n == 1 for _, _, n in seen)
+    ex.manager.check()
+    assert ex.manager.live() == []
